@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""LRQK decode benchmark on one MI355X.
+
+A "step" is one decode step of ONE layer: ring append, factor update, proxy-score scan over
+all cached tokens, top-k, hit/miss diff, miss fetch from the pinned host store, and exact
+attention over the k + lite active tokens.  Default workload: Llama-3-8B attention shape at a
+128K-token context (32 q / 8 kv heads, d 128, bf16, r 32, k 2048, lite 64, max_iter (2,2)).
+
+Prints ONE JSON line.  `value` is microseconds per layer-step with all inputs resident (the
+per-step q,k,v are pre-staged in HBM; the host store is pinned host memory by definition
+of the path).  `roofline` is the proxy-score kernel (the dominant HBM stream): algorithmic
+bytes Hq * m * r * elem per launch over its HIP-event duration.  `cpu_baseline` times the CPU
+oracle on a few steps continued from the same state.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=128)
+    p.add_argument("--warmup", type=int, default=16)
+    p.add_argument("--workload", default="llama8b_128k_bf16")
+    p.add_argument("--context", type=int, default=None, help="override the context length")
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--cpu-steps", type=int, default=3, help="oracle steps timed for cpu_baseline (0 = skip)")
+    p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
+    p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
+    p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
+    return p.parse_args()
+
+
+def oracle_from_engine(eng, w, threads):
+    """A CPU oracle layer continued from the engine's current state."""
+    from oracle import lrqk_oracle as orc
+    orc.set_threads(threads)
+    o = orc.OracleLayer(num_lite_tokens=w.lite_tokens, attn_topk=w.num_active_tokens, num_key_value_groups=w.groups,
+                        r=w.r, max_iter=w.max_iter, tol=w.tol, capacity=eng._A_K.capacity,
+                        compute_dtype=torch.float32, no_hit_miss=eng.no_hit_miss)
+    torch.cuda.synchronize()
+    o.B_Q, o.B_K = eng.B_Q.cpu(), eng.B_K.cpu()
+    o._A_K.data, o._A_K.capacity, o._A_K.current_len = eng._A_K.data.cpu(), eng._A_K.capacity, eng._A_K.current_len
+    o._A_K.dtype = eng._A_K.data.dtype
+    o.KVcpu.data, o.KVcpu.capacity, o.KVcpu.current_len = eng.KVcpu.data.clone(), eng.KVcpu.capacity, eng.KVcpu.current_len
+    o.KVcpu.dtype = eng.KVcpu.data.dtype
+    o.Kgpu, o.Vgpu = eng.Kgpu.cpu(), eng.Vgpu.cpu()
+    o.hit_indices = eng.hit_indices.cpu()
+    o.lite_indices, o.lite_len = list(eng.lite_indices), eng.lite_len
+    o.current_len, o.prefill_length = eng.current_len, eng.prefill_length
+    return o, orc
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: the LRQK cache path has no multi-GPU part (heads shard trivially); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from lrqk_amd import synth
+    import lrqk_amd
+    from lrqk_amd import _lib
+    _lib.load()  # fail loudly if the HIP library is missing
+
+    dev = torch.device("cuda:0")
+    w = synth.WORKLOADS[a.workload]
+    l = a.context or w.context
+    t_setup = time.perf_counter()
+    # synthetic prompt, drawn on the GPU (128K x 48 heads x 128 would take minutes on the host)
+    Q, K, V, bases, gen = synth.prompt_qkv(w, a.seed, l, device=dev)
+    A0 = synth.init_factors(w, l, a.seed + 1, device=dev)
+    cls = lrqk_amd.LightAttentionIndicesNoHitMiss if a.variant == "no_hit_miss" else lrqk_amd.LightAttentionIndicesFactory
+    eng = cls(num_lite_tokens=w.lite_tokens, attn_topk=w.num_active_tokens, num_key_value_groups=w.groups, r=w.r,
+              max_iter=w.max_iter, tol=w.tol, capacity=4096)
+    eng.init_factors = A0
+    eng.attn_in_step = not a.no_attn
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.prefill(Q, K, V)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    del A0
+    stream = synth.DecodeStream(w, Q[:, :, -1:], bases, gen)
+    total = a.warmup + a.steps
+    qs, ks, vs = [], [], []
+    for _ in range(total):
+        q, k, v = stream.next()
+        qs.append(q.contiguous()); ks.append(k.contiguous()); vs.append(v.contiguous())
+    del Q, K, V
+    torch.cuda.empty_cache()
+    # reserve so that no step of the timed region allocates or grows a buffer
+    eng.ws.reserve(w.batch * w.num_heads, l + total + 64, w.num_active_tokens,
+                   w.num_active_tokens + w.lite_tokens, w.r, w.head_dim)
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t_setup
+
+    miss = sel = 0
+    for i in range(a.warmup):
+        eng.decode(qs[i], ks[i], vs[i])
+    torch.cuda.synchronize()
+    cap_before = (eng._A_K.capacity, eng.KVcpu.capacity)
+    m_first = eng.lite_indices[eng.lite_len] - 1
+
+    eng.ws.timing_enable(a.steps)
+    counts = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.warmup, total):
+        eng.decode(qs[i], ks[i], vs[i])
+        counts.append(eng.last_miss_count)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kern_ms, launches = eng.ws.timing_read()
+    eng.ws.timing_enable(0)
+    grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
+    m_last = eng.lite_indices[eng.lite_len] - 1
+
+    n_miss = int(torch.stack(counts).sum())
+    n_sel = len(counts) * w.batch * w.num_heads * w.num_active_tokens
+    e = 2 if w.dtype == torch.bfloat16 else 4
+    row_bytes = 2 * w.head_dim * e
+    us_step = elapsed / a.steps * 1e6
+    m_avg = (m_first + m_last) / 2.0
+    scan_bytes = w.batch * w.num_heads * m_avg * w.r * e
+    kern_us = kern_ms * 1e3 / max(launches, 1)
+    achieved = scan_bytes / (kern_us * 1e-6) / 1e9 if launches else 0.0
+    n_act = w.num_active_tokens + w.lite_tokens
+    bh = w.batch * w.num_heads
+    step_bytes = (scan_bytes + (0 if a.no_attn else 2 * bh * n_act * w.head_dim * e) + bh * n_act * w.head_dim * e
+                  + bh * n_act * w.r * e + 4 * bh * w.r * w.head_dim * e + 3 * bh * w.num_active_tokens * 4
+                  + n_miss / a.steps * row_bytes)
+
+    cpu = None
+    if a.cpu_steps > 0:
+        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        o, orc = oracle_from_engine(eng, w, threads)
+        extra = [stream.next() for _ in range(a.cpu_steps + 1)]
+        extra = [(q.cpu(), k.cpu(), v.cpu()) for q, k, v in extra]
+        q, k, v = extra[0]
+        Ko, Vo = o.decode(q, k, v)          # untimed warm-up step
+        orc.attention(q, Ko, Vo, torch.float32)
+        t0 = time.perf_counter()
+        for q, k, v in extra[1:]:
+            Ko, Vo = o.decode(q, k, v)
+            if not a.no_attn:
+                orc.attention(q, Ko, Vo, torch.float32)
+        cpu_s = (time.perf_counter() - t0) / a.cpu_steps
+        cpu = {"value": round(cpu_s * 1e6, 1), "unit": "us/layer-step", "cores": threads, "kind": "port",
+               "sample": f"{a.cpu_steps} decode steps of the same workload continued from the GPU state "
+                         f"(fp32 torch-CPU factor update + C scan/sort/diff/gather per head on {threads} threads)"}
+
+    out = {
+        "metric": "lrqk_decode_us_per_layer_step", "value": round(us_step, 2), "unit": "us",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(us_step / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
+                   "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
+                   "variant": a.variant, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
+        "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
+        "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
+        "h2d_bytes_per_step": round(n_miss / a.steps * row_bytes),
+        "step_algorithmic_bytes": round(step_bytes),
+        "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "roofline": {"bound": "hbm", "kernel": "score_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
+        "cpu_baseline": cpu,
+        "prefill_s": round(prefill_s, 3), "setup_s": round(setup_s, 2), "buffers_grew_in_timed_region": grew,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,179 @@
+/*
+ * C ABI of liblrqk_hip.so: the gfx950 (MI355X) kernels of the LRQK per-layer decode /
+ * prefill path.  Plain pointers and sizes only; no torch types.  Every entry point
+ * returns 0 on success and a negative LRQK_E* code on an argument error (the text is
+ * available from lrqk_last_error()); nothing throws across the boundary.  All device
+ * work is enqueued on the caller's stream (a hipStream_t passed as void*; NULL is the
+ * default stream) and nothing synchronises unless the comment says so.
+ *
+ * Shapes: "bh" is batch * query-heads, flattened row-major (b, h).  Query head h reads
+ * KV head h / groups.  dtype is the STORAGE type of factors and K/V rows; arithmetic is
+ * fp32.  Token / slot indices on the device are int32.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree; "py" = lrqk_attention.py, "cpp" = cpp_kernel/take_along_dim_grouped.cpp).
+ */
+#ifndef LRQK_HIP_H
+#define LRQK_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LRQK_F32 0
+#define LRQK_BF16 1
+
+#define LRQK_OK 0
+#define LRQK_EINVAL (-1)   /* bad shape / size / dtype / null pointer */
+#define LRQK_EHIP (-2)     /* a HIP runtime call failed */
+#define LRQK_ELIMIT (-3)   /* size beyond what the kernels support */
+
+#define LRQK_MAX_R 64
+#define LRQK_MAX_TOPK 8192
+#define LRQK_MAX_DECODE_ITERS 16
+
+typedef struct lrqk_ctx lrqk_ctx;
+
+int lrqk_version(void);
+const char* lrqk_last_error(void);
+
+/* Workspace (radix keys, histograms, split partials), sized on demand; growing it
+ * synchronises the device once.  One ctx per engine; calls on one ctx must not overlap. */
+int lrqk_ctx_create(lrqk_ctx** out);
+int lrqk_ctx_destroy(lrqk_ctx* ctx);
+/* Optional: pre-size the workspace so that later calls never allocate. */
+int lrqk_ctx_reserve(lrqk_ctx* ctx, int bh, int64_t max_tokens, int topk, int n_active, int r, int d);
+
+/* py:1260-1263 -- proxy scores A_K[:m] . q_hat^T as fp32 [bh][m].
+ * a_k: [bh] heads of head_stride elements each, rows of r elements; q_hat: [bh][r].
+ * score = fmaf chain over j = 0..r-1 from +0; -0 becomes +0; round_bf16 != 0 rounds the
+ * fp32 sum to bfloat16 (nearest even), which is what a bf16 matmul returns. */
+int lrqk_proxy_scores(const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
+                      int dtype, int round_bf16, float* out_scores, void* stream);
+
+/* py:1235-1273 compute_hit_indices -- scores (as above, never materialised as floats)
+ * + per-head top-k under the order (score descending, token index ascending), returned
+ * ASCENDING by index in out_idx[bh][out_stride] (first min(k,m) entries).  m <= k yields
+ * arange(m).  Returns min(k,m) (>= 0) on success. */
+int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh,
+                      int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* out_idx,
+                      int64_t out_stride, void* stream);
+
+/* Same selection from caller-provided fp32 scores [bh][m] (test hook for tie cases). */
+int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int bh, int64_t m, int topk,
+                            int32_t* out_idx, int64_t out_stride, void* stream);
+
+/* py:1275-1315 only_indices_in_cpu -- hit/miss diff, in place.
+ * hit: [bh][hit_stride] current GPU-resident token ids (first k used), any order, unique.
+ * new_idx: [bh][new_stride] ascending, unique.  On return the j-th evicted slot (ascending
+ * slot) of each head holds the j-th smallest token of new \ hit; evict[bh][k] is 1 for
+ * replaced slots; miss_slots[bh][k] lists the replaced slots ascending and miss_count[bh]
+ * their number.  Any of evict / miss_slots / miss_count may be NULL only if all callers of
+ * the result do not need it (miss_slots and miss_count are required by lrqk_fetch_rows). */
+int lrqk_diff(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t hit_stride, int bh, int k,
+              uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, void* stream);
+
+/* py:1752, 1762-1773 (LightAttentionIndicesNoHitMiss) -- the ablation without hit/miss
+ * bookkeeping: hit <- new_idx, every slot marked evicted (all k rows are refetched). */
+int lrqk_replace_all(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t hit_stride, int bh, int k,
+                     uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, void* stream);
+
+/* py:101-117 + cpp:133-183 (d0_indices_select) + py:1603-1608 -- fetch the missed rows of
+ * the host [K|V] store straight into the active-set slots.
+ * kv_store: [b][hkv][cap][2*d] (K row then V row), pinned host memory (or device memory);
+ * k_act/v_act: [bh][n_slots][d].  For every head and every j < miss_count: slot =
+ * miss_slots[j], token = hit[slot]; K/V slot rows are overwritten with the store row of
+ * (b, h/groups, token).  The kernel reads the store through the GPU's host mapping. */
+int lrqk_fetch_rows(const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
+                    const int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
+                    const int32_t* miss_count, int b, int hq, int hkv, int d, int k, int dtype,
+                    void* stream);
+
+/* py:1339-1351 fetch_by_hit (same-device branch) -- k_act[bh][j][:] = src[b][h/groups][idx[bh][j]][:]
+ * for j < count, src: [b][hkv][src_len][d] on the device. */
+int lrqk_gather_rows(const void* src, int64_t src_len, const int32_t* idx, int64_t idx_stride, int count,
+                     void* dst, int n_slots, int b, int hq, int hkv, int d, int dtype, void* stream);
+
+/* py:1133-1135, 1185-1188 -- write the new token's k,v ([b][hkv][d]) into ring slot `slot`
+ * of every query head and record its token id in active_idx[bh][slot]. */
+int lrqk_append_token(const void* k_new, const void* v_new, void* k_act, void* v_act, int n_slots, int slot,
+                      int32_t* active_idx, int64_t idx_stride, int32_t token, int b, int hq, int hkv, int d,
+                      int dtype, void* stream);
+
+/* py:1192-1196 + 959-963 -- flush ring slots [slot0, slot0+count) of heads 0, g, 2g, ... to
+ * store rows [row0, row0+count) as [K|V]. */
+int lrqk_flush_ring(const void* k_act, const void* v_act, int n_slots, int slot0, int count, void* kv_store,
+                    int64_t cap, int64_t row0, int b, int hq, int hkv, int d, int dtype, void* stream);
+
+/* py:2326-2327 (flash_attn_with_kvcache, one query, scale 1/sqrt(d)) -- exact attention
+ * over the first n_valid slots.  q,out: [bh][d]; k_act,v_act: [bh][n_slots][d]. */
+int lrqk_attention(lrqk_ctx* ctx, const void* q, const void* k_act, const void* v_act, int n_slots,
+                   int n_valid, void* out, int bh, int d, int dtype, void* stream);
+
+/* py:803-839 cast_lrqk_decode -> py:529-628 _lrqk_decode_inv_w1 + py:651-665 -- the per-step
+ * factor update.  b_q,b_k: [bh][r][d] storage dtype, updated in place.  The active A_K rows
+ * are gathered from a_k (heads of head_stride elements) at active_idx[bh][0..n) (py:1156-1171);
+ * if active_idx is NULL rows 0..n-1 are used (the prefix branch, py:1526-1539).
+ * k_prev: [bh][kprev_slots][d] (first n rows used); q: [bh][d]; k_new: [b][hkv][d].
+ * Outputs q_hat,k_hat: [bh][r] storage dtype.  If append_row >= 0, k_hat is also written to
+ * row append_row of every head of a_k (py:1560 sync_cache).  The stopping test
+ * mean((k_hat - k_hat')^2) < tol is taken over all heads at once, on the device. */
+int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
+                    const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots, int n,
+                    const void* q, const void* k_new, int b, int hq, int hkv, int r, int d, int max_iter,
+                    float tol, void* q_hat, void* k_hat, int64_t append_row, int dtype, void* stream);
+
+/* py:772-800 cast_lrqk_prefill -> py:319-423 _lrqk_prefill_inv_w1 -- joint rank-r ALS fit.
+ * q: [b][hq][l][d], k: [b][hkv][l][d] storage dtype (query head h uses KV head h/groups);
+ * a_q,a_k: [bh][l][r] fp32 work buffers holding the initial factors on entry and the
+ * result on return; b_q,b_k out: [bh][r][d] fp32.  Synchronises the stream once per
+ * iteration to evaluate the stopping test on the host.  Returns the number of
+ * iterations run (>= 0). */
+int lrqk_als_prefill(lrqk_ctx* ctx, const void* q, const void* k, float* a_q, float* a_k, float* b_q,
+                     float* b_k, int b, int hq, int hkv, int64_t l, int r, int d, int max_iter, float tol,
+                     int dtype, void* stream);
+
+/* py:1506-1613 LightAttentionIndicesFactory.decode (main branch) + the attention call
+ * site py:2326 -- one decode step of one layer as one host call that only enqueues
+ * kernels.  State: b_q,b_k [bh][r][d]; a_k heads of head_stride elements (zero beyond the
+ * rows written so far); active_idx [bh][topk+lite] = resident token ids then ring token
+ * ids; k_act,v_act [bh][topk+lite][d]; kv_store [b][hkv][cap][2d].
+ * Order: ring append of (k_new, v_new) at slot topk+ring_slot as token id `token`; if
+ * flush_row0 >= 0 the whole ring is flushed to store rows flush_row0.. ; factor update
+ * (k_hat appended as A_K row `token`); selection over candidates 0..m-1; diff (or
+ * replace-all when no_hit_miss); miss fetch; if attn_out != NULL, attention of q over all
+ * topk+lite slots.  evict ([bh][topk]) and miss_count ([bh]) are optional outputs. */
+int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
+                     void* k_act, void* v_act, void* kv_store, int64_t cap, const void* q, const void* k_new,
+                     const void* v_new, int b, int hq, int hkv, int r, int d, int topk, int lite, int ring_slot,
+                     int32_t token, int64_t m, int64_t flush_row0, int max_iter, float tol, int round_scores,
+                     int no_hit_miss, void* q_hat, void* k_hat, void* attn_out, uint8_t* evict,
+                     int32_t* miss_count, int dtype, void* stream);
+
+/* py:2031-2105 (WrapForwardTimer, the reference's only timing facility, wall clock around
+ * forward) -- device-side timing of the dominant kernel instead: after
+ * lrqk_timing_enable(ctx, n) the next n proxy-score kernel launches of lrqk_score_select /
+ * lrqk_decode_step on this ctx are bracketed by HIP events on the launch stream;
+ * lrqk_timing_read waits for them, returns the summed kernel time and the launch count, and
+ * re-arms.  n = 0 switches timing off. */
+int lrqk_timing_enable(lrqk_ctx* ctx, int max_launches);
+int lrqk_timing_read(lrqk_ctx* ctx, double* total_ms, int* launches);
+
+/* Host-side row gathers with the reference's native signatures (the staged fetch path
+ * and API parity); multi-threaded memcpy.
+ * cpp:133-183 d0_indices_select: dst[i,:] = src[idx[i],:]. */
+int lrqk_d0_indices_select(void* dst, const void* src, const int64_t* idx, int64_t n, int64_t row_bytes,
+                           int64_t src_rows, int threads);
+/* cpp:13-124 take_along_dim_with_mask: src [b][hkv][seq][row], indices int64 / mask u8
+ * [b][hkv][groups][k]; dst gets the masked rows in row-major mask order.  Returns the row
+ * count (>= 0); dst may be NULL to only count. */
+int64_t lrqk_take_along_dim_with_mask(void* dst, const void* src, const int64_t* indices, const uint8_t* mask,
+                                      int64_t b, int64_t hkv, int64_t groups, int64_t k, int64_t seq,
+                                      int64_t row_bytes, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

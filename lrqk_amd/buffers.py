@@ -1,0 +1,187 @@
+"""Growable and pre-allocated token buffers (interface of lrqk_attention.py:844-1028).
+
+The layouts are part of the kernel contract: the rank-r key factors live on the GPU as
+``[b, Hq, capacity, r]`` and the full-precision store lives in pinned host memory as
+``[b, Hkv, capacity, 2*d]`` with the K row followed by the V row.  Buffers are
+zero-initialised up to their capacity: the decode step gathers the not-yet-written row of
+the newest token and relies on reading zeros there.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+
+class AutoIncreaseTensor:
+    """Buffer that grows by ``scaling_ratio`` along ``dim`` (lrqk_attention.py:844-957)."""
+
+    def __init__(self, capacity: int = 4096, dim: int = 0, scaling_ratio: float = 1.5,
+                 device: Optional[torch.device] = None, dtype: Optional[torch.dtype] = None,
+                 pin_memory: bool = False):
+        self.capacity = capacity
+        self.dim = dim
+        self.scaling_ratio = scaling_ratio
+        self.device = device
+        self.dtype = dtype
+        self.data: Optional[torch.Tensor] = None
+        self.current_len = 0
+        self.pin_memory = pin_memory
+
+    # -- allocation policy (first allocation :877-889, growth :892-920)
+    def _alloc(self, shape):
+        pin = bool(self.pin_memory) and torch.cuda.is_available()
+        return torch.zeros(shape, device=self.device, dtype=self.dtype, pin_memory=pin)
+
+    def _ensure(self, like_shape, length: int):
+        target = self.current_len + length
+        if self.data is None:
+            cap = max(self.capacity, int(length * self.scaling_ratio))
+            shape = list(like_shape)
+            shape[self.dim] = cap
+            self.data = self._alloc(shape)
+            self.capacity = cap
+        elif target >= self.capacity:
+            cap = self.capacity
+            while cap <= target:
+                cap = int(cap * self.scaling_ratio)
+            shape = list(self.data.shape)
+            shape[self.dim] = cap
+            grown = self._alloc(shape)
+            if self.pin_memory and torch.cuda.is_available():
+                # kernels may still be writing flushed rows into (or fetching rows from) the old
+                # pinned block; the host copy below and the release of the block must wait
+                torch.cuda.synchronize()
+            if self.current_len:
+                grown.narrow(self.dim, 0, self.current_len).copy_(self.data.narrow(self.dim, 0, self.current_len))
+            self.data = grown
+            self.capacity = cap
+
+    @torch.inference_mode()
+    def append(self, x: torch.Tensor):
+        if self.device is None:
+            self.device = x.device
+        if self.dtype is None:
+            self.dtype = x.dtype
+        length = x.size(self.dim)
+        self._ensure(x.shape, length)
+        self.data.narrow(self.dim, self.current_len, length).copy_(x)
+        self.current_len += length
+
+    @torch.inference_mode()
+    def extend(self, like_shape, length: int) -> int:
+        """Make room for ``length`` more entries exactly as ``append`` would, without writing
+        them (a kernel fills the rows).  Returns the index of the first new entry."""
+        self._ensure(like_shape, length)
+        first = self.current_len
+        self.current_len += length
+        return first
+
+    def has_data(self):
+        return self.data is not None
+
+    @property
+    def shape(self) -> torch.Size:
+        s = list(self.data.shape)
+        s[self.dim] = self.current_len
+        return torch.Size(s)
+
+    def tensor(self) -> torch.Tensor:
+        return self.data.narrow(self.dim, 0, self.current_len)
+
+    def __len__(self):
+        return self.current_len
+
+    def __getitem__(self, idx):
+        if self.data is None:
+            raise IndexError("Cache is empty")
+        return self.tensor()[idx]
+
+    def take_along_dim(self, indices: torch.Tensor, dim: int = None, out=None) -> torch.Tensor:
+        """Gather on the FULL-capacity buffer (lrqk_attention.py:952-956)."""
+        if self.data is None:
+            raise IndexError("Cache is empty")
+        return torch.take_along_dim(self.data, indices, self.dim if dim is None else dim, out=out)
+
+
+class AutoIncreaseTensorSharedKV(AutoIncreaseTensor):
+    """K and V rows side by side on the last dim (lrqk_attention.py:959-963)."""
+
+    @torch.inference_mode()
+    def append(self, k: torch.Tensor, v: torch.Tensor):
+        if self.dtype is None:
+            self.dtype = k.dtype
+        if self.device is None:
+            self.device = torch.device("cpu")
+        length = k.size(self.dim)
+        d = k.size(-1)
+        shape = list(k.shape)
+        shape[-1] = 2 * d
+        self._ensure(shape, length)
+        dst = self.data.narrow(self.dim, self.current_len, length)
+        dst.narrow(-1, 0, d).copy_(k)
+        dst.narrow(-1, d, d).copy_(v)
+        self.current_len += length
+
+
+class PreAllocatedTensor:
+    """Fixed-capacity buffer; overflow raises ValueError (lrqk_attention.py:966-1011)."""
+
+    def __init__(self, capacity: int, dim: int, dtype: torch.dtype = None, device: torch.device = None):
+        self.capacity = capacity
+        self.dim = dim
+        self.dtype = dtype
+        self.device = device
+        self.data = None
+        self.current_len = 0
+
+    @classmethod
+    def from_tensor(cls, capacity: int, dim: int, data: torch.Tensor):
+        out = cls(capacity, dim, data.dtype, data.device)
+        out.append(data)
+        return out
+
+    def append(self, x: torch.Tensor):
+        if self.dtype is None:
+            self.dtype = x.dtype
+        if self.device is None:
+            self.device = x.device
+        n = x.shape[self.dim]
+        if self.data is None:
+            shape = list(x.shape)
+            shape[self.dim] = self.capacity
+            self.data = torch.empty(shape, dtype=self.dtype, device=self.device)
+        if self.current_len + n > self.capacity:
+            raise ValueError("Not enough capacity to store the tensor")
+        self.data.narrow(self.dim, self.current_len, n).copy_(x)
+        self.current_len += n
+
+    def has_data(self):
+        return self.data is not None
+
+    def tensor(self) -> torch.Tensor:
+        return self.data.narrow(self.dim, 0, self.current_len)
+
+    def __len__(self):
+        return self.current_len
+
+    def __getitem__(self, idx):
+        return self.tensor()[idx]
+
+
+class _CacheQKV:
+    """Prompt pieces shorter than the active set wait here (lrqk_attention.py:1014-1028)."""
+
+    def __init__(self, capacity: int, dim: int, dtype: torch.dtype = None, device: torch.device = None):
+        self.Q = PreAllocatedTensor(capacity, dim, dtype, device)
+        self.K = PreAllocatedTensor(capacity, dim, dtype, device)
+        self.V = PreAllocatedTensor(capacity, dim, dtype, device)
+
+    def append(self, Q, K, V):
+        self.Q.append(Q)
+        self.K.append(K)
+        self.V.append(V)
+        return self.Q.tensor(), self.K.tensor(), self.V.tensor()
+
+    def __len__(self):
+        return self.Q.current_len

@@ -1,0 +1,51 @@
+// Library-owned device workspace.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+
+namespace lrqk {
+
+struct DevBuf {
+  void* p = nullptr;
+  size_t bytes = 0;
+  // Grows (never shrinks).  Growing frees the old block after a device sync, because
+  // kernels of an earlier call may still be reading it.
+  int ensure(size_t need) {
+    if (need <= bytes) return LRQK_OK;
+    size_t want = need + need / 4;
+    void* np = nullptr;
+    LRQK_HIP_CHECK(hipMalloc(&np, want));
+    if (p) {
+      LRQK_HIP_CHECK(hipDeviceSynchronize());
+      LRQK_HIP_CHECK(hipFree(p));
+    }
+    p = np;
+    bytes = want;
+    return LRQK_OK;
+  }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+};
+
+}  // namespace lrqk
+
+struct lrqk_ctx {
+  lrqk::DevBuf keys;        // u32 [bh][key_stride]   orderable score keys
+  lrqk::DevBuf hist;        // u32 [bh][4096]         first-level radix histogram
+  lrqk::DevBuf cand;        // candidate (key,idx) pairs for the fast select path
+  lrqk::DevBuf cand_cnt;    // per-chunk counts / thresholds
+  lrqk::DevBuf attn_part;   // f32 [bh][S][d+2]
+  lrqk::DevBuf als_part;    // f32 [bh][S][r*(r+1)]
+  lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
+  lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
+  lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
+  lrqk::DevBuf misc;        // evict mask, miss lists, counters of the fused step
+  // optional event timing of the proxy-score kernel (two events per launch)
+  hipEvent_t* tev = nullptr;
+  int tev_pairs = 0;   // capacity in pairs
+  int tev_used = 0;    // pairs recorded since the last read
+};

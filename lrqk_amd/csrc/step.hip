@@ -1,0 +1,55 @@
+// One decode step of one layer as a single host call: ring append (+ flush), factor
+// update, proxy-score scan + top-k, hit/miss diff, miss fetch and (optionally) the exact
+// attention over the active set.  Only launches; never synchronises.
+#include "common.hpp"
+#include "ctx.hpp"
+
+using namespace lrqk;
+
+extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
+                                int32_t* active_idx, void* k_act, void* v_act, void* kv_store, int64_t cap,
+                                const void* q, const void* k_new, const void* v_new, int b, int hq, int hkv, int r, int d,
+                                int topk, int lite, int ring_slot, int32_t token, int64_t m, int64_t flush_row0,
+                                int max_iter, float tol, int round_scores, int no_hit_miss, void* q_hat, void* k_hat,
+                                void* attn_out, uint8_t* evict, int32_t* miss_count, int dtype, void* stream) {
+  LRQK_REQUIRE(ctx != nullptr, LRQK_EINVAL, "ctx is null");
+  LRQK_REQUIRE(topk > 0 && lite > 0 && ring_slot >= 0 && ring_slot < lite, LRQK_EINVAL, "bad ring slot %d of %d", ring_slot,
+               lite);
+  LRQK_REQUIRE(m >= topk, LRQK_EINVAL, "m=%lld < topk=%d: the main decode branch needs at least topk candidates",
+               (long long)m, topk);
+  const int bh = b * hq;
+  const int n = topk + lite;
+  int rc;
+  if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
+  // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | evict u8 [bh][topk]
+  if ((rc = ctx->misc.ensure((size_t)bh * topk * 5 + (size_t)bh * 4 + 64))) return rc;
+  int32_t* new_idx = (int32_t*)ctx->new_idx.p;
+  int32_t* miss_slots = (int32_t*)ctx->misc.p;
+  int32_t* mcount = miss_count ? miss_count : miss_slots + (size_t)bh * topk;
+  uint8_t* ev = evict ? evict : (uint8_t*)(miss_slots + (size_t)bh * topk + bh);
+
+  if ((rc = lrqk_append_token(k_new, v_new, k_act, v_act, n, topk + ring_slot, active_idx, n, token, b, hq, hkv, d, dtype,
+                              stream)))
+    return rc;
+  if (flush_row0 >= 0) {
+    if ((rc = lrqk_flush_ring(k_act, v_act, n, topk, lite, kv_store, cap, flush_row0, b, hq, hkv, d, dtype, stream)))
+      return rc;
+  }
+  if ((rc = lrqk_als_decode(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, n, n, q, k_new, b, hq, hkv, r, d,
+                            max_iter, tol, q_hat, k_hat, token, dtype, stream)))
+    return rc;
+  rc = lrqk_score_select(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, topk, stream);
+  if (rc < 0) return rc;
+  if (no_hit_miss)
+    rc = lrqk_replace_all(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
+  else
+    rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
+  if (rc) return rc;
+  if ((rc = lrqk_fetch_rows(kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv, d, topk, dtype,
+                            stream)))
+    return rc;
+  if (attn_out) {
+    if ((rc = lrqk_attention(ctx, q, k_act, v_act, n, n, attn_out, bh, d, dtype, stream))) return rc;
+  }
+  return LRQK_OK;
+}

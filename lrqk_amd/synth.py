@@ -60,24 +60,26 @@ def low_rank_noise(gen: torch.Generator, b: int, h: int, l: int, d: int, rho: in
     """Returns (X [b,h,l,d] in ``dtype``, W [b,h,rho,d] fp32).  Pass ``W`` to draw more rows
     from the same subspace (new decode tokens)."""
     std = rho ** -0.25
+    dev = gen.device
     if W is None:
-        W = torch.randn((b, h, rho, d), generator=gen) * std
-    out = torch.empty((b, h, l, d), dtype=dtype)
+        W = torch.randn((b, h, rho, d), generator=gen, device=dev) * std
+    out = torch.empty((b, h, l, d), dtype=dtype, device=dev)
     step = 16384
     for s in range(0, l, step):
         e = min(l, s + step)
-        U = torch.randn((b, h, e - s, rho), generator=gen) * std
+        U = torch.randn((b, h, e - s, rho), generator=gen, device=dev) * std
         X = torch.matmul(U, W)
         if sigma:
-            X = X + sigma * torch.randn((b, h, e - s, d), generator=gen)
+            X = X + sigma * torch.randn((b, h, e - s, d), generator=gen, device=dev)
         out[:, :, s:e] = X.to(dtype)
     return out, W
 
 
-def prompt_qkv(w: Workload, seed: int = 0, context: int = None):
+def prompt_qkv(w: Workload, seed: int = 0, context: int = None, device="cpu"):
     """Q [b,Hq,l,d], K,V [b,Hkv,l,d] in the workload dtype, and the subspace bases so decode
-    tokens can follow the same statistics."""
-    gen = torch.Generator().manual_seed(seed)
+    tokens can follow the same statistics.  ``device`` selects where the numbers are drawn
+    (the CPU stream is the portable one; a GPU draw is only reproducible on that GPU type)."""
+    gen = torch.Generator(device=device).manual_seed(seed)
     l = context or w.context
     Q, WQ = low_rank_noise(gen, w.batch, w.num_heads, l, w.head_dim, w.rho, w.sigma, w.dtype)
     K, WK = low_rank_noise(gen, w.batch, w.num_kv_heads, l, w.head_dim, w.rho, w.sigma, w.dtype)
@@ -90,9 +92,10 @@ def rotate_query(gen: torch.Generator, q: torch.Tensor, angle_std: float = 0.05,
     pairs with angles ~ N(0, angle_std).  q fp32 [b,H,1,d]."""
     b, H, _, d = q.shape
     n_rot = n_rot or d // 2
-    perm = torch.randperm(d, generator=gen)
+    dev = gen.device
+    perm = torch.randperm(d, generator=gen, device=dev)
     i, j = perm[0:2 * n_rot:2], perm[1:2 * n_rot:2]
-    th = torch.randn((b, H, 1, n_rot), generator=gen) * angle_std
+    th = torch.randn((b, H, 1, n_rot), generator=gen, device=dev) * angle_std
     c, s = torch.cos(th), torch.sin(th)
     out = q.clone()
     qi, qj = q[..., i], q[..., j]
@@ -119,9 +122,9 @@ class DecodeStream:
         return self.q.to(w.dtype), k, v
 
 
-def init_factors(w: Workload, l: int, seed: int = 1):
-    """Injected A_Q0, A_K0 (the ``randn`` initialiser drawn on the CPU): fp32 [b,Hq,l,r]."""
-    gen = torch.Generator().manual_seed(seed)
-    A_Q0 = torch.randn((w.batch, w.num_heads, l, w.r), generator=gen)
-    A_K0 = torch.randn((w.batch, w.num_heads, l, w.r), generator=gen)
+def init_factors(w: Workload, l: int, seed: int = 1, device="cpu"):
+    """Injected A_Q0, A_K0 (the ``randn`` initialiser with a fixed seed): fp32 [b,Hq,l,r]."""
+    gen = torch.Generator(device=device).manual_seed(seed)
+    A_Q0 = torch.randn((w.batch, w.num_heads, l, w.r), generator=gen, device=device)
+    A_K0 = torch.randn((w.batch, w.num_heads, l, w.r), generator=gen, device=device)
     return A_Q0, A_K0

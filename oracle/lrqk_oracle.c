@@ -48,9 +48,11 @@ static inline float round_to_bf16(float f) {
   return f;
 }
 
-/* Monotone map float -> uint32 (larger float <=> larger key). */
+/* Monotone map float -> uint32 (larger float <=> larger key); -0 and +0 compare equal,
+ * as they do for torch.topk, so they share one key. */
 static inline uint32_t order_key(float f) {
   uint32_t u;
+  if (f == 0.0f) f = 0.0f;
   memcpy(&u, &f, 4);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }

@@ -246,6 +246,25 @@ def cast_lrqk_decode(B_Q, A_K, B_K, K__, q, k, max_iter=8, tol=1e-5, compute_dty
 
 # --------------------------------------------------------------------------- selection
 
+_THREADS = 1
+
+
+def set_threads(n: int):
+    """Heads are independent: run the per-head C calls on ``n`` threads (ctypes drops the GIL)."""
+    global _THREADS
+    _THREADS = max(1, int(n))
+
+
+def _per_head(fn, count):
+    if _THREADS == 1 or count == 1:
+        for i in range(count):
+            fn(i)
+        return
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(_THREADS, count)) as ex:
+        list(ex.map(fn, range(count)))
+
+
 def proxy_scores(A_K_m: torch.Tensor, q_hat: torch.Tensor, round_to_storage: bool = True) -> torch.Tensor:
     """:1260-1263.  A_K_m [b,H,m,r], q_hat [b,H,1,r] in the storage dtype -> fp32 [b,H,m].
     fp32 fmaf chain over j; with bf16 storage and round_to_storage the result is rounded to
@@ -253,16 +272,23 @@ def proxy_scores(A_K_m: torch.Tensor, q_hat: torch.Tensor, round_to_storage: boo
     lib = _load()
     b, H, m, r = A_K_m.shape
     code = _dtype_code(A_K_m.dtype)
-    A = A_K_m.contiguous()
+    A = A_K_m
+    if A.stride(3) != 1 or A.stride(2) != r:   # rows must be contiguous; heads may be strided views
+        A = A.contiguous()
     qh = q_hat.contiguous()
     out = torch.empty((b, H, m), dtype=torch.float32)
     esz = A.element_size()
     rb = 1 if (round_to_storage and code == 1) else 0
-    for i in range(b * H):
-        rc = lib.oracle_proxy_scores(A.data_ptr() + i * m * r * esz, qh.data_ptr() + i * r * esz,
+    sb, sh = A.stride(0), A.stride(1)
+
+    def one(i):
+        off = (i // H) * sb + (i % H) * sh
+        rc = lib.oracle_proxy_scores(A.data_ptr() + off * esz, qh.data_ptr() + i * r * esz,
                                      m, r, code, rb, out.data_ptr() + i * m * 4)
         if rc != 0:
             raise RuntimeError(f"oracle_proxy_scores failed: {rc}")
+
+    _per_head(one, b * H)
     return out
 
 
@@ -274,10 +300,12 @@ def topk_sorted(scores: torch.Tensor, k: int) -> torch.Tensor:
     kk = min(k, m)
     sc = scores.contiguous()
     out = torch.empty((b, H, kk), dtype=torch.int32)
-    for i in range(b * H):
+    def one(i):
         n = lib.oracle_topk_sorted(sc.data_ptr() + i * m * 4, m, k, out.data_ptr() + i * kk * 4)
         if n != kk:
             raise RuntimeError("oracle_topk_sorted failed")
+
+    _per_head(one, b * H)
     return out.to(torch.int64).unsqueeze(-1)
 
 
@@ -297,11 +325,13 @@ def only_indices_in_cpu(now: torch.Tensor, new: torch.Tensor) -> Tuple[torch.Ten
     c = new.reshape(b * H, k).to(torch.int32).contiguous()
     upd = torch.empty_like(a)
     ev = torch.empty((b * H, k), dtype=torch.uint8)
-    for i in range(b * H):
+    def one(i):
         n = lib.oracle_only_indices(a.data_ptr() + i * k * 4, c.data_ptr() + i * k * 4, k,
                                     upd.data_ptr() + i * k * 4, ev.data_ptr() + i * k)
         if n < 0:
             raise RuntimeError("shape mismatch: evicted and missing counts differ")
+
+    _per_head(one, b * H)
     return upd.to(torch.int64).reshape(b, H, k, 1), ev.bool().reshape(b, H, k)
 
 
@@ -486,8 +516,10 @@ class OracleLayer:
         idx = torch.cat([self.hit_indices, lite], dim=2)
         return torch.take_along_dim(self._A_K.data, idx, 2)
 
-    def prefill(self, q, k, v, A_Q0=None, A_K0=None, generator=None):
-        """:1385-1504"""
+    def prefill(self, q, k, v, A_Q0=None, A_K0=None, generator=None, als_result=None):
+        """:1385-1504.  ``als_result`` = (A_Q, B_Q, A_K, B_K) in the storage dtype replaces the
+        oracle's own factorisation (to continue from the factors of the implementation under
+        test once those were checked within tolerance)."""
         b, H, l, d = q.shape
         assert l >= self.k, "seq_len must be larger than attn_topk"
         repk = repeat_kv(k, self.g)
@@ -495,8 +527,11 @@ class OracleLayer:
         self.Vgpu = torch.zeros((b, H, self.n, d), dtype=q.dtype)
         self.prefill_length = l
         self.current_len = l
-        A_Q, B_Q, A_K, B_K = cast_lrqk_prefill(q, repk, self.r, self.max_iter[0], self.tol[0], self.init,
-                                               A_Q0, A_K0, generator, self.compute_dtype)
+        if als_result is not None:
+            A_Q, B_Q, A_K, B_K = als_result
+        else:
+            A_Q, B_Q, A_K, B_K = cast_lrqk_prefill(q, repk, self.r, self.max_iter[0], self.tol[0], self.init,
+                                                   A_Q0, A_K0, generator, self.compute_dtype)
         self.B_Q, self.B_K = B_Q, B_K
         self._A_K.append(A_K)
         self.last_A_Q = A_Q
@@ -525,30 +560,30 @@ class OracleLayer:
 
     def decode(self, q, k, v):
         """:1506-1613 (and :1688-1775 when no_hit_miss)"""
+        return self.finish_decode(*self.begin_decode(q, k, v))
+
+    def begin_decode(self, q, k, v):
+        """Ring append + the factor update (:1519-1559), returned but not yet applied."""
         self._append(k, v)
         repk = repeat_kv(k, self.g)
         if self.current_len <= self.n:
-            B_Q, B_K, hq, hk = cast_lrqk_decode(self.B_Q, self.A_K, self.B_K,
-                                                self.Kgpu.narrow(2, 0, self.current_len - 1), q, repk,
-                                                self.max_iter[1], self.tol[1], self.compute_dtype)
-            self.B_Q, self.B_K = B_Q, B_K
-            self._A_K.append(hk)
-            self.last_q_hat, self.last_k_hat = hq, hk
-            return self.Kgpu.narrow(2, 0, self.current_len), self.Vgpu.narrow(2, 0, self.current_len)
-        B_Q, B_K, hq, hk = cast_lrqk_decode(self.B_Q, self._A_K_hitted_with_lite(), self.B_K, self.Kgpu, q, repk,
-                                            self.max_iter[1], self.tol[1], self.compute_dtype)
-        return self.finish_decode(B_Q, B_K, hq, hk)
+            return cast_lrqk_decode(self.B_Q, self.A_K, self.B_K, self.Kgpu.narrow(2, 0, self.current_len - 1), q,
+                                    repk, self.max_iter[1], self.tol[1], self.compute_dtype)
+        return cast_lrqk_decode(self.B_Q, self._A_K_hitted_with_lite(), self.B_K, self.Kgpu, q, repk,
+                                self.max_iter[1], self.tol[1], self.compute_dtype)
 
     def finish_decode(self, B_Q, B_K, hq, hk):
-        """Steps 3b-6 of the decode (:1560-1613) from given ALS outputs; split out so a test can
-        inject the ALS result of the implementation under test and compare the integer
-        stages bit for bit."""
+        """The rest of the step (:1540-1545 / :1560-1613) from given ALS outputs; split out so a
+        test can inject the ALS result of the implementation under test (after checking it
+        within tolerance) and compare the integer stages bit for bit."""
         self.B_Q, self.B_K = B_Q, B_K
         self._A_K.append(hk)
         self.last_q_hat, self.last_k_hat = hq, hk
+        if self.current_len <= self.n:
+            return self.Kgpu.narrow(2, 0, self.current_len), self.Vgpu.narrow(2, 0, self.current_len)
         m = self.lite_indices[self.lite_len] - 1
         self.last_m = m
-        new = compute_hit_indices(hq, self.A_K.narrow(2, 0, m).contiguous(), self.k, self.round_scores)
+        new = compute_hit_indices(hq, self.A_K.narrow(2, 0, m), self.k, self.round_scores)
         self.last_new_indices = new
         b, H = new.shape[:2]
         d = self.Kgpu.shape[-1]

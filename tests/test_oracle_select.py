@@ -124,6 +124,10 @@ def test_negative_scores_order(oracle):
     assert oracle.topk_sorted(s, 2)[0, 0, :, 0].tolist() == [1, 3]
     s = torch.tensor([[[-3.0, 1.0, -2.0, 0.0, 4.0, -0.0]]])
     assert oracle.topk_sorted(s, 3)[0, 0, :, 0].tolist() == [1, 3, 4]
+    # -0 and +0 are one value (as for torch.topk): the tie goes to the lower index
+    s = torch.tensor([[[-0.0, 0.0, 0.0, -1.0]]])
+    assert oracle.topk_sorted(s, 2)[0, 0, :, 0].tolist() == [0, 1]
+    assert torch.topk(s[0, 0], 3).values.tolist() == [0.0, 0.0, 0.0]
 
 
 # ---------------------------------------------------------------- diff
