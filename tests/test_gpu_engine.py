@@ -32,7 +32,7 @@ def _rel(a, b):
 
 
 def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter, tol, rho, cls=None, capacity=64,
-              seed=0, fp_tol=None, no_hit_miss=False, sigma=0.01):
+              seed=0, fp_tol=None, no_hit_miss=False, sigma=0.01, compare_factors=True):
     from lrqk_amd import synth, ops
     g = hq // hkv
     gen = torch.Generator().manual_seed(seed)
@@ -61,9 +61,20 @@ def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter
     # elements agree exactly, a few differ by one unit in the last place
     gA_K, gB_K, gB_Q = eng.A_K.cpu(), eng.B_K.cpu(), eng.B_Q.cpu()
     gA_Qrow = eng.last_A_Q_row.cpu()
-    for name, got, exp in (("A_K", gA_K, ref[2]), ("B_K", gB_K, ref[3]), ("B_Q", gB_Q, ref[1]),
-                           ("A_Q[-1]", gA_Qrow, ref[0][:, :, -1:])):
-        assert _rel(got, exp) < lim, ("prefill", name, _rel(got, exp))
+    if compare_factors:
+        for name, got, exp in (("A_K", gA_K, ref[2]), ("B_K", gB_K, ref[3]), ("B_Q", gB_Q, ref[1]),
+                               ("A_Q[-1]", gA_Qrow, ref[0][:, :, -1:])):
+            assert _rel(got, exp) < lim, ("prefill", name, _rel(got, exp))
+    # what the factors are for: the fit K ~ A_K B_K and the last query row q ~ a_q B_Q.  These
+    # are well determined even where the individual factors are not (badly scaled r x r
+    # systems: fp32 LAPACK itself is several percent away from fp64 there)
+    K4 = oracle.repeat_kv(K, g).double()
+    fit_g = _rel(gA_K.double() @ gB_K.double(), K4)
+    fit_o = _rel(ref[2].double() @ ref[3].double(), K4)
+    assert abs(fit_g - fit_o) < 2e-3 + 0.05 * fit_o, ("prefill fit K", fit_g, fit_o)
+    qfit_g = _rel(gA_Qrow.double() @ gB_Q.double(), Q[:, :, -1:].double())
+    qfit_o = _rel(ref[0][:, :, -1:].double() @ ref[1].double(), Q[:, :, -1:].double())
+    assert abs(qfit_g - qfit_o) < 2e-2 + 0.1 * qfit_o, ("prefill fit q", qfit_g, qfit_o)
     # continue the oracle from the GPU's factors
     A_Q_full = torch.zeros((b, hq, l, r), dtype=dtype)
     A_Q_full[:, :, -1:] = gA_Qrow
@@ -198,7 +209,7 @@ def test_llama_shape_bf16_short(lrqk, oracle):
     8K context."""
     _say("llama shape trace")
     _lockstep(lrqk, oracle, b=1, hq=32, hkv=8, d=128, l=8192, r=32, k=2048, L=64, steps=6, dtype=torch.bfloat16,
-              max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096, fp_tol=3e-2)
+              max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096, fp_tol=3e-2, compare_factors=False)
 
 
 def test_cache_front_door(lrqk, oracle):
