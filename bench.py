@@ -117,6 +117,7 @@ def main():
     m_first = eng.lite_indices[eng.lite_len] - 1
 
     eng.ws.timing_enable(a.steps)
+    eng.ws.select_stats(reset=True)
     counts = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -127,6 +128,7 @@ def main():
     elapsed = time.perf_counter() - t0
     kern_ms, launches = eng.ws.timing_read()
     eng.ws.timing_enable(0)
+    sel_fast, sel_full = eng.ws.select_stats()
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
 
@@ -178,9 +180,10 @@ def main():
         "h2d_bytes_per_step": round(n_miss / a.steps * row_bytes),
         "step_algorithmic_bytes": round(step_bytes),
         "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": {"bound": "hbm", "kernel": "score_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "score_filter_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
+        "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full},
         "cpu_baseline": cpu,
         "prefill_s": round(prefill_s, 3), "setup_s": round(setup_s, 2), "buffers_grew_in_timed_region": grew,
     }

@@ -56,7 +56,9 @@ int lrqk_proxy_scores(const void* a_k, int64_t head_stride, const void* q_hat, i
 /* py:1235-1273 compute_hit_indices -- scores (as above, never materialised as floats)
  * + per-head top-k under the order (score descending, token index ascending), returned
  * ASCENDING by index in out_idx[bh][out_stride] (first min(k,m) entries).  m <= k yields
- * arange(m).  Returns min(k,m) (>= 0) on success. */
+ * arange(m).  Returns min(k,m) (>= 0) on success.  The ctx remembers, per head, a lower
+ * bound of the previous call's threshold to pre-filter the next scan; the result never
+ * depends on it. */
 int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh,
                       int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* out_idx,
                       int64_t out_stride, void* stream);
@@ -64,6 +66,12 @@ int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
 /* Same selection from caller-provided fp32 scores [bh][m] (test hook for tie cases). */
 int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int bh, int64_t m, int topk,
                             int32_t* out_idx, int64_t out_stride, void* stream);
+
+/* Which selector path the heads took since the last reset: `fast_heads` selected from the
+ * candidate list of the streaming filter, `full_heads` rescanned their whole head (first
+ * call, or the score distribution moved).  Copies two counters from the device
+ * (synchronises).  No counterpart in the reference. */
+int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads, int reset);
 
 /* py:1275-1315 only_indices_in_cpu -- hit/miss diff, in place.
  * hit: [bh][hit_stride] current GPU-resident token ids (first k used), any order, unique.

@@ -1,36 +1,69 @@
-// Per-step factor update (the decode half of the alternating least squares).
+// Per-step factor update (the decode half of the alternating least squares), r <= 32.
 //
-//   gram   : per head, split over the active rows: A^T [A | w] with w = K_prev q
-//            (A = gathered active A_K rows) -> partial sums
-//   solve  : per head: reduce partials, form the r x r Gram systems, run every
-//            alternating iteration and record each iterate + its squared change
-//   finish : per head: pick the iterate at which the batch-wide stopping test fired,
-//            take the exact line-search step on B_Q, B_K, round and store
+//   gram   : grid (S, heads).  Each wave streams its share of the active rows once: w = K_prev q
+//            on the vector ALUs and A^T A / A^T w on the matrix cores (fp32 MFMA 32x32x2; both
+//            operands of A^T A are the same registers), A = the gathered active A_K rows.
+//            Per-workgroup partial sums go to HBM.
+//   solve  : one workgroup per head: adds the S partials in a fixed order, forms
+//            G_K = B_K B_K^T and G_Q = B_Q B_Q^T + A^T A (MFMA again), inverts both once and runs
+//            every alternating iteration as a rank-one (Sherman-Morrison) update of them,
+//            recording each iterate and its squared change.
+//   finish : per head: pick the iterate at which the batch-wide stopping test fired, take the
+//            exact line-search step on B_Q, B_K, round and store.
+//
+// One CU retires 64 fp32 lane-operations per clock and a global load costs about a
+// microsecond, so the per-head kernels avoid integer division, keep every batch of loads
+// independent, and never walk a chain of dependent loads.  (A single launch in which the
+// last-arriving workgroup continues was measured slower: the device-scope fence it needs
+// costs ~15 us per workgroup because each XCD has its own L2.)
+#include <algorithm>
+
 #include "common.hpp"
 #include "ctx.hpp"
 
 namespace lrqk {
 
-constexpr int kAlsThreads = 256;
-constexpr int kTileRows = 32;
+typedef float v16f __attribute__((ext_vector_type(16)));
 
+constexpr int kAlsMaxR = 32;  // one 32x32 MFMA tile
+constexpr int kGramThreads = 256;
+constexpr int kGramWaves = kGramThreads / kWave;
+constexpr int kGramChunk = 32;  // tokens per wave per chunk = 16 MFMA steps
+constexpr int kGramNe = 32 * 32 + 32;
+constexpr int kSolveThreads = 256;
+constexpr int kSolveWaves = kSolveThreads / kWave;
+constexpr int kFinThreads = 256;
+
+// C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
+__device__ __forceinline__ int mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
+
+// Partial layout per (head, split): 32*32 floats of A^T A (row stride 32) then 32 floats of
+// A^T w.  Rows/columns >= r are zero.
 template <typename T>
-__global__ __launch_bounds__(kAlsThreads) void als_gram_kernel(const T* __restrict__ a_k, int64_t head_stride,
-                                                               int64_t a_rows, const int32_t* __restrict__ active_idx,
-                                                               int64_t idx_stride, const T* __restrict__ k_prev,
-                                                               int kprev_slots, int n, const T* __restrict__ q, int r,
-                                                               int d, int lpr_log2, float* __restrict__ part, int S) {
+__global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restrict__ a_k, int64_t head_stride,
+                                                                int64_t a_rows, const int32_t* __restrict__ active_idx,
+                                                                int64_t idx_stride, const T* __restrict__ k_prev,
+                                                                int kprev_slots, int n, const T* __restrict__ q, int r,
+                                                                int d, int lpr_log2, float* __restrict__ part, int S) {
   constexpr int VEC = Vec16<T>::N;
-  __shared__ float a_s[kTileRows][LRQK_MAX_R + 2];  // [row][0..r) = A row, [r] = w
-  const int h = blockIdx.y, s = blockIdx.x;
+  __shared__ float w_all[kGramWaves][kGramChunk];
+  __shared__ float red[kGramWaves][kGramNe];
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int h = blockIdx.y, s = blockIdx.x;
+  float* w_s = w_all[wave];
+
   const int lpr = 1 << lpr_log2;
   const int sub = lane & (lpr - 1), grp = lane >> lpr_log2, gpw = kWave >> lpr_log2;
   const int rows_per_split = (n + S - 1) / S;
-  const int r0 = s * rows_per_split;
-  const int r1 = min(n, r0 + rows_per_split);
+  const int s0 = s * rows_per_split;
+  const int s1 = min(n, s0 + rows_per_split);
+  const int rows_per_wave = (rows_per_split + kGramWaves - 1) / kGramWaves;
+  const int w0 = s0 + wave * rows_per_wave;
+  const int w1 = min(s1, w0 + rows_per_wave);
+  const int n_chunks = (rows_per_wave + kGramChunk - 1) / kGramChunk;  // uniform over waves
   const T* A = a_k + (int64_t)h * head_stride;
   const T* Kp = k_prev + (int64_t)h * kprev_slots * d;
+  const int col = lane & 31, khalf = lane >> 5;
 
   float qf[VEC];
   {
@@ -38,210 +71,377 @@ __global__ __launch_bounds__(kAlsThreads) void als_gram_kernel(const T* __restri
     qv.load(q + (int64_t)h * d + sub * VEC);
     qv.unpack(qf);
   }
-  const int ne = r * (r + 1);
-  constexpr int kMaxPer = (LRQK_MAX_R * (LRQK_MAX_R + 1) + kAlsThreads - 1) / kAlsThreads;
-  float acc[kMaxPer];
+  v16f acc;
 #pragma unroll
-  for (int i = 0; i < kMaxPer; ++i) acc[i] = 0.0f;
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  float racc = 0.0f;
 
-  for (int t0 = r0; t0 < r1; t0 += kTileRows) {
-    const int rows = min(kTileRows, r1 - t0);
-    // A rows (gathered) -> LDS
-    for (int e = tid; e < rows * r; e += kAlsThreads) {
-      const int row = e / r, j = e % r;
-      const int64_t src = active_idx ? (int64_t)active_idx[(int64_t)h * idx_stride + t0 + row] : (int64_t)(t0 + row);
-      a_s[row][j] = (src >= 0 && src < a_rows) ? ld_f32<T>(A, src * r + j) : 0.0f;
-    }
-    // w = K_prev[row] . q
-    for (int base = 0; base < rows; base += gpw * (kAlsThreads / kWave)) {
-      const int row = base + wave * gpw + grp;
-      const bool valid = row < rows;
-      const int rr = valid ? row : rows - 1;
-      Vec16<T> kv;
-      kv.load(Kp + (int64_t)(t0 + rr) * d + sub * VEC);
-      float kf[VEC];
-      kv.unpack(kf);
-      float w = 0.0f;
+  for (int ch = 0; ch < n_chunks; ++ch) {
+    const int c0 = w0 + ch * kGramChunk;
+    // token ids this lane needs: tokens c0 + 2g + khalf, g = 0..15
+    int src[kGramChunk / 2];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) w = fmaf(kf[e], qf[e], w);
-      for (int off = 1; off < lpr; off <<= 1) w += __shfl_xor(w, off, kWave);
-      if (valid && sub == 0) a_s[row][r] = w;
+    for (int g = 0; g < kGramChunk / 2; ++g) {
+      const int t = c0 + 2 * g + khalf;
+      src[g] = -1;
+      if (t < w1) src[g] = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
     }
-    __syncthreads();
+    // K rows of the chunk -> w
+    for (int base0 = 0; base0 < kGramChunk; base0 += 8 * gpw) {
+      Vec16<T> kv[8];
 #pragma unroll
-    for (int i = 0; i < kMaxPer; ++i) {
-      const int e = tid + i * kAlsThreads;
-      if (e < ne) {
-        const int j = e / (r + 1), j2 = e % (r + 1);
-        float v = acc[i];
-        for (int row = 0; row < rows; ++row) v = fmaf(a_s[row][j], a_s[row][j2], v);
-        acc[i] = v;
+      for (int u = 0; u < 8; ++u) {
+        const int row = base0 + u * gpw + grp;
+        if (row < kGramChunk && c0 + row < w1) kv[u].load(Kp + (int64_t)(c0 + row) * d + sub * VEC);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int row = base0 + u * gpw + grp;
+        float wv = 0.0f;
+        if (row < kGramChunk && c0 + row < w1) {
+          float kf[VEC];
+          kv[u].unpack(kf);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) wv = fmaf(kf[e], qf[e], wv);
+        }
+        for (int off = 1; off < lpr; off <<= 1) wv += __shfl_xor(wv, off, kWave);
+        if (sub == 0 && row < kGramChunk) w_s[row] = wv;
       }
     }
-    __syncthreads();
-  }
-  float* out = part + ((int64_t)h * S + s) * ne;
+    // A elements of the chunk: lane (col, khalf) holds A[token 2g + khalf][col]
+    float a0[kGramChunk / 2];
 #pragma unroll
-  for (int i = 0; i < kMaxPer; ++i) {
-    const int e = tid + i * kAlsThreads;
-    if (e < ne) out[e] = acc[i];
+    for (int g = 0; g < kGramChunk / 2; ++g) {
+      const int64_t sr = src[g];
+      a0[g] = (sr >= 0 && sr < a_rows && col < r) ? ld_f32<T>(A, sr * r + col) : 0.0f;
+    }
+    __syncthreads();  // w_s of this chunk is complete (every wave runs the same number of chunks)
+#pragma unroll
+    for (int g = 0; g < kGramChunk / 2; ++g) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[g], a0[g], acc, 0, 0, 0);
+      racc = fmaf(w_s[2 * g + khalf], a0[g], racc);
+    }
+    __syncthreads();  // before the next chunk overwrites w_s
+  }
+  racc += __shfl_xor(racc, 32, kWave);
+  // ---- cross-wave reduction through LDS
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[wave][mfma_row(lane, v) * 32 + col] = acc[v];
+  if (lane < 32) red[wave][32 * 32 + col] = racc;
+  __syncthreads();
+  float* pout = part + ((int64_t)h * S + s) * kGramNe;
+  for (int e = tid; e < kGramNe; e += kGramThreads) {
+    float v = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kGramWaves; ++wv) v += red[wv][e];
+    pout[e] = v;
   }
 }
 
-// Gauss-Jordan elimination without pivoting on the augmented r x (r+1) system in LDS
-// (the systems here are Gram matrices plus positive semidefinite terms).  Row stride ldm.
-// On return x[i] = Mx[i][r] / Mx[i][i].  One barrier per eliminated column.
-__device__ __forceinline__ void solve_lds(float* Mx, int ldm, int r, float* x) {
+// Everything in the solve kernel works on 32 x 32 tiles padded with an identity block (rows
+// and columns >= r), so every loop has a compile-time trip count and its LDS reads pipeline.
+constexpr int kLdm = 65;  // row stride of an augmented [G | I] matrix (64 columns)
+constexpr int kLdi = 33;  // row stride of an inverse
+
+// Gauss-Jordan inversion of two SPD 32 x 32 matrices side by side in LDS, no pivoting, 256
+// threads.  Mx: two augmented matrices [G | I] (row stride kLdm), the second at 32*kLdm.  In
+// step p only columns p+1 .. p+32 of a row change (the identity half is lower triangular so
+// far), so a thread owns one column offset and 8 rows.  On return
+// inv{0,1}[i][c] = Mx[i][32+c] / Mx[i][i].
+__device__ __forceinline__ void invert_pair_lds(float* Mx, float* inv0, float* inv1) {
   const int tid = threadIdx.x;
-  for (int p = 0; p < r; ++p) {
-    const float inv = 1.0f / Mx[p * ldm + p];
-    const int w = r - p;  // columns p+1 .. r
-    for (int e = tid; e < r * w; e += kAlsThreads) {
-      const int i = e / w, j = p + 1 + e % w;
-      if (i != p) Mx[i * ldm + j] = fmaf(-(Mx[i * ldm + p] * inv), Mx[p * ldm + j], Mx[i * ldm + j]);
+  const int cw = tid & 31;
+  const int mat = (tid >> 5) & 1;
+  const int rc = tid >> 6;  // row class 0..3: rows rc + 4u
+  float* M = Mx + mat * 32 * kLdm;
+  for (int p = 0; p < 32; ++p) {
+    const float invp = 1.0f / M[p * kLdm + p];
+    const int c = p + 1 + cw;
+    const float mpc = M[p * kLdm + c];
+    float mip[8], mic[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      mip[u] = M[(rc + 4 * u) * kLdm + p];
+      mic[u] = M[(rc + 4 * u) * kLdm + c];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (rc + 4 * u != p) M[(rc + 4 * u) * kLdm + c] = fmaf(-(mip[u] * invp), mpc, mic[u]);
     }
     __syncthreads();
   }
-  for (int i = tid; i < r; i += kAlsThreads) x[i] = Mx[i * ldm + r] / Mx[i * ldm + i];
+  float* inv = mat ? inv1 : inv0;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int i = rc + 4 * u;
+    inv[i * kLdi + cw] = M[i * kLdm + 32 + cw] / M[i * kLdm + i];
+  }
   __syncthreads();
 }
 
-// iter_out layout per head: [max_iter][2r] (q_hat then k_hat of each iteration),
+// out[j] = sum_i v[i] * Minv[i][j], 32 terms
+__device__ __forceinline__ float row_times32(const float* v, const float* Minv, int j) {
+  float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 32; i += 2) {
+    s0 = fmaf(v[i], Minv[i * kLdi + j], s0);
+    s1 = fmaf(v[i + 1], Minv[(i + 1) * kLdi + j], s1);
+  }
+  return s0 + s1;
+}
+
+// x = b (G + v^T v)^-1 from G^-1 (Sherman-Morrison): x = y - (y.v / (1 + z.v)) z with
+// y = b G^-1, z = v G^-1.  Executed by the first wave; b, v, x are LDS vectors of 32.
+__device__ __forceinline__ void rank1_solve_wave(const float* b, const float* v, const float* Ginv, float* x) {
+  const int j = threadIdx.x & 31;  // caller guarantees threadIdx.x < 64; both halves compute the same
+  const float y = row_times32(b, Ginv, j);
+  const float z = row_times32(v, Ginv, j);
+  float yv = (threadIdx.x < 32) ? y * v[j] : 0.0f;
+  float zv = (threadIdx.x < 32) ? z * v[j] : 0.0f;
+  yv = wave_sum(yv);
+  zv = wave_sum(zv);
+  const float alpha = yv / (1.0f + zv);
+  if (threadIdx.x < 32) x[j] = fmaf(-alpha, z, y);
+}
+
+// iter_out per head: [max_iter][2r] (q_hat then k_hat of each iteration);
 // deltas: [bh][max_iter] sum over r of (k_hat - k_hat')^2.
 template <typename T>
-__global__ __launch_bounds__(kAlsThreads) void als_solve_kernel(const T* __restrict__ b_q, const T* __restrict__ b_k,
-                                                                const float* __restrict__ part, int S,
-                                                                const T* __restrict__ q, const T* __restrict__ k_new,
-                                                                int hq, int hkv, int r, int d, int max_iter,
-                                                                float* __restrict__ iter_out,
-                                                                float* __restrict__ deltas) {
+__global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __restrict__ b_q, const T* __restrict__ b_k,
+                                                                  const float* __restrict__ part, int S,
+                                                                  const T* __restrict__ q, const T* __restrict__ k_new,
+                                                                  int hq, int hkv, int r, int d, int vshift,
+                                                                  int max_iter, float* __restrict__ iter_out,
+                                                                  float* __restrict__ deltas) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int kMaxVec = 8;    // 16-byte vectors per thread per matrix: r * d / VEC <= 2048
+  constexpr int kMaxSplit = 32;
   extern __shared__ __align__(16) float sm[];
-  float* BQ = sm;                    // [r][d+1]
-  float* BK = BQ + r * (d + 1);      // [r][d+1]
-  float* qv = BK + r * (d + 1);      // [d]
-  float* kv = qv + d;                // [d]
-  float* GQ = kv + d;                // [r][r+1]
-  float* GK = GQ + r * (r + 1);      // [r][r+1]
-  float* Mx = GK + r * (r + 1);      // [r][r+2]
-  float* rhs_q = Mx + r * (r + 2);   // 5 vectors of r
-  float* kB = rhs_q + r;
-  float* hat_k = kB + r;
-  float* hat_q = hat_k + r;
-  float* new_k = hat_q + r;
   __shared__ float s_qk;
-  const int lg = r + 1, lm = r + 2;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.x;
   const int b = h / hq, head = h % hq;
   const int kvh = head / (hq / hkv);
   const int ld = d + 1;
-  const int ne = r * (r + 1);
+  float* BQ = sm;                   // [32][d+1]  (rows >= r are zero)
+  float* BK = BQ + 32 * ld;         // [32][d+1]
+  float* qv = BK + 32 * ld;         // [d]
+  float* kv = qv + d;               // [d]
+  float* G = kv + d;                // [kGramNe] summed A^T [A | w]
+  float* Mx = G + kGramNe;          // 2 x [32][kLdm]: [G_K | I] then [G_Q | I]
+  float* GKi = Mx + 2 * 32 * kLdm;  // [32][kLdi]
+  float* GQi = GKi + 32 * kLdi;     // [32][kLdi]
+  float* rhs_q = GQi + 32 * kLdi;   // 6 vectors of 32
+  float* kB = rhs_q + 32;
+  float* hat_k = kB + 32;
+  float* hat_q = hat_k + 32;
+  float* new_k = hat_q + 32;
+  float* tmp = new_k + 32;
+  float* cred = tmp + 32;           // [2 matrices][2 halves of d][32*32] MFMA tiles
 
-  for (int e = tid; e < r * d; e += kAlsThreads) {
-    BQ[(e / d) * ld + e % d] = ld_f32<T>(b_q, (int64_t)h * r * d + e);
-    BK[(e / d) * ld + e % d] = ld_f32<T>(b_k, (int64_t)h * r * d + e);
-  }
-  for (int c = tid; c < d; c += kAlsThreads) {
-    qv[c] = ld_f32<T>(q, (int64_t)h * d + c);
-    kv[c] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
-  }
-  __syncthreads();
-  // G_Q = B_Q B_Q^T + A^T A ; G_K = B_K B_K^T ; rhs_q = q B_Q^T + (q K^T) A ; kB = k B_K^T ; s = q.k
-  for (int e = tid; e < r * r; e += kAlsThreads) {
-    const int i = e / r, j = e % r;
-    float gq = 0.0f, gk = 0.0f;
-    for (int c = 0; c < d; ++c) {
-      gq = fmaf(BQ[i * ld + c], BQ[j * ld + c], gq);
-      gk = fmaf(BK[i * ld + c], BK[j * ld + c], gk);
+  // ---- every global load of the kernel is issued here, back to back
+  const float* pin = part + (int64_t)h * S * kGramNe;
+  constexpr int kPer = (kGramNe + kSolveThreads - 1) / kSolveThreads;  // 5 entries per thread
+  float gsum[kPer];
+  {
+    float x[kPer][kMaxSplit];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      const int e = tid + u * kSolveThreads;
+#pragma unroll
+      for (int t = 0; t < kMaxSplit; ++t) x[u][t] = (t < S && e < kGramNe) ? pin[(int64_t)t * kGramNe + e] : 0.0f;
     }
-    float ata = 0.0f;
-    for (int s = 0; s < S; ++s) ata += part[((int64_t)h * S + s) * ne + i * (r + 1) + j];
-    GQ[i * lg + j] = gq + ata;
-    GK[i * lg + j] = gk;
-  }
-  for (int i = tid; i < r; i += kAlsThreads) {
-    float a = 0.0f, c2 = 0.0f;
-    for (int c = 0; c < d; ++c) {
-      a = fmaf(qv[c], BQ[i * ld + c], a);
-      c2 = fmaf(kv[c], BK[i * ld + c], c2);
+    const int vpr = 1 << vshift;
+    const int nvec = r << vshift;
+    Vec16<T> vq[kMaxVec], vk[kMaxVec];
+#pragma unroll
+    for (int u = 0; u < kMaxVec; ++u) {
+      const int vi = tid + u * kSolveThreads;
+      if (vi < nvec) {
+        vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
+        vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
+      }
     }
-    float wa = 0.0f;
-    for (int s = 0; s < S; ++s) wa += part[((int64_t)h * S + s) * ne + i * (r + 1) + r];
-    rhs_q[i] = a + wa;
-    kB[i] = c2;
-  }
-  if (tid == 0) {
-    float s = 0.0f;
-    for (int c = 0; c < d; ++c) s = fmaf(qv[c], kv[c], s);
-    s_qk = s;
+    if (tid < d) {
+      qv[tid] = ld_f32<T>(q, (int64_t)h * d + tid);
+      kv[tid] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + tid);
+    }
+    // zero the padded rows of BQ/BK, then scatter the vectors
+    for (int e = tid; e < (32 - r) * ld; e += kSolveThreads) {
+      BQ[r * ld + e] = 0.0f;
+      BK[r * ld + e] = 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < kMaxVec; ++u) {
+      const int vi = tid + u * kSolveThreads;
+      if (vi < nvec) {
+        const int row = vi >> vshift, c0 = (vi & (vpr - 1)) * VEC;
+        float fq[VEC], fk[VEC];
+        vq[u].unpack(fq);
+        vk[u].unpack(fk);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          BQ[row * ld + c0 + e] = fq[e];
+          BK[row * ld + c0 + e] = fk[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      float v = 0.0f;
+#pragma unroll
+      for (int t = 0; t < kMaxSplit; ++t) v += x[u][t];  // fixed order 0..S-1 (zeros beyond)
+      gsum[u] = v;
+      const int e = tid + u * kSolveThreads;
+      if (e < kGramNe) G[e] = v;
+    }
   }
   __syncthreads();
-  // k_hat_0 = kB G_K^{-1}
-  for (int e = tid; e < r * (r + 1); e += kAlsThreads) {
-    const int i = e / (r + 1), j = e % (r + 1);
-    Mx[i * lm + j] = j < r ? GK[i * lg + j] : kB[i];
+  // ---- B_Q B_Q^T and B_K B_K^T on the matrix cores: wave -> (matrix, half of the d axis)
+  {
+    const int col = lane & 31, khalf = lane >> 5;
+    const int which = wave & 1, half = wave >> 1;
+    const float* B = (which ? BK : BQ) + col * ld + khalf;
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    const int k1 = (half + 1) * (d / 2);
+#pragma unroll 8
+    for (int kk = half * (d / 2); kk < k1; kk += 2)  // d >= 8 is a power of two
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(B[kk], B[kk], acc, 0, 0, 0);
+    float* mine = cred + (which * 2 + half) * 1024;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mine[mfma_row(lane, v) * 32 + col] = acc[v];
+  }
+  // rhs_q = q B_Q^T + (q K^T) A ; kB = k B_K^T : thread -> (output i = tid >> 2, quarter of d)
+  {
+    const int i = tid >> 2, qtr = tid & 3;
+    const int which = i >> 5, row = i & 31;
+    const float* B = (which ? BK : BQ) + row * ld;
+    const float* vec = which ? kv : qv;
+    float v = 0.0f;
+#pragma unroll 8
+    for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], B[c], v);
+    v += __shfl_xor(v, 1, kWave);
+    v += __shfl_xor(v, 2, kWave);
+    if (qtr == 0) {
+      if (which == 0) rhs_q[row] = v + G[32 * 32 + row];
+      else kB[row] = v;
+    }
+  }
+  if (wave == 0) {
+    float v = 0.0f;
+    for (int c = lane; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
+    v = wave_sum(v);
+    if (lane == 0) s_qk = v;
   }
   __syncthreads();
-  solve_lds(Mx, lm, r, hat_k);
+  // [G_K | I], [G_Q | I], identity-padded beyond r
+  {
+    float* MK = Mx;
+    float* MQ = Mx + 32 * kLdm;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + u * kSolveThreads;
+      const int i = e >> 5, j = e & 31;
+      const bool in = i < r && j < r;
+      const float eye = (i == j) ? 1.0f : 0.0f;
+      MQ[i * kLdm + j] = in ? (cred[e] + cred[1024 + e]) + G[e] : eye;
+      MK[i * kLdm + j] = in ? cred[2048 + e] + cred[3072 + e] : eye;
+      MQ[i * kLdm + 32 + j] = eye;
+      MK[i * kLdm + 32 + j] = eye;
+    }
+  }
+  (void)gsum;
+  __syncthreads();
+  invert_pair_lds(Mx, GKi, GQi);
+  // k_hat_0 = kB G_K^-1
+  if (tid < 32) hat_k[tid] = row_times32(kB, GKi, tid);
+  __syncthreads();
   for (int it = 0; it < max_iter; ++it) {
-    // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat      (all matrices symmetric)
-    for (int e = tid; e < r * (r + 1); e += kAlsThreads) {
-      const int i = e / (r + 1), j = e % (r + 1);
-      Mx[i * lm + j] = j < r ? fmaf(hat_k[i], hat_k[j], GQ[i * lg + j]) : fmaf(s_qk, hat_k[i], rhs_q[i]);
-    }
+    // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
+    if (tid < 32) tmp[tid] = fmaf(s_qk, hat_k[tid], rhs_q[tid]);
     __syncthreads();
-    solve_lds(Mx, lm, r, hat_q);
+    if (tid < kWave) rank1_solve_wave(tmp, hat_k, GQi, hat_q);
+    __syncthreads();
     // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat
-    for (int e = tid; e < r * (r + 1); e += kAlsThreads) {
-      const int i = e / (r + 1), j = e % (r + 1);
-      Mx[i * lm + j] = j < r ? fmaf(hat_q[i], hat_q[j], GK[i * lg + j]) : fmaf(s_qk, hat_q[i], kB[i]);
-    }
+    if (tid < 32) tmp[tid] = fmaf(s_qk, hat_q[tid], kB[tid]);
     __syncthreads();
-    solve_lds(Mx, lm, r, new_k);
     if (tid < kWave) {
+      rank1_solve_wave(tmp, hat_q, GKi, new_k);
       float dsq = 0.0f;
-      for (int i = tid; i < r; i += kWave) {
-        const float df = hat_k[i] - new_k[i];
-        dsq = fmaf(df, df, dsq);
+      if (tid < r) {
+        const float df = hat_k[tid] - new_k[tid];  // each lane reads back only what it wrote
+        dsq = df * df;
       }
       dsq = wave_sum(dsq);
       if (tid == 0) deltas[(int64_t)h * max_iter + it] = dsq;
     }
-    float* o = iter_out + ((int64_t)h * max_iter + it) * 2 * r;
-    for (int i = tid; i < r; i += kAlsThreads) {
-      o[i] = hat_q[i];
-      o[r + i] = new_k[i];
-    }
     __syncthreads();
-    for (int i = tid; i < r; i += kAlsThreads) hat_k[i] = new_k[i];
+    float* o = iter_out + ((int64_t)h * max_iter + it) * 2 * r;
+    if (tid < 32) {
+      if (tid < r) {
+        o[tid] = hat_q[tid];
+        o[r + tid] = new_k[tid];
+      }
+      hat_k[tid] = new_k[tid];
+    }
     __syncthreads();
   }
 }
 
+// One workgroup per head.  B_Q and B_K of the head are held in registers as 16-byte vectors
+// (vector vi = tid + 256 u covers row vi >> vshift, columns (vi & (vpr-1)) * VEC ..).
 template <typename T>
-__global__ __launch_bounds__(kAlsThreads) void als_finish_kernel(T* __restrict__ b_q, T* __restrict__ b_k,
+__global__ __launch_bounds__(kFinThreads) void als_finish_kernel(T* __restrict__ b_q, T* __restrict__ b_k,
                                                                  const T* __restrict__ q, const T* __restrict__ k_new,
                                                                  const float* __restrict__ iter_out,
                                                                  const float* __restrict__ deltas, int bh, int hq,
-                                                                 int hkv, int r, int d, int max_iter, float tol,
-                                                                 T* __restrict__ q_hat_out, T* __restrict__ k_hat_out,
-                                                                 T* __restrict__ a_k, int64_t head_stride,
-                                                                 int64_t append_row) {
-  __shared__ float hat[2][LRQK_MAX_R];
+                                                                 int hkv, int r, int d, int vshift, int max_iter,
+                                                                 float tol, T* __restrict__ q_hat_out,
+                                                                 T* __restrict__ k_hat_out, T* __restrict__ a_k,
+                                                                 int64_t head_stride, int64_t append_row) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int kMaxVec = 8;  // vectors per thread per matrix: r * d / VEC <= 2048
+  __shared__ float hat[2][kAlsMaxR];
   __shared__ float err[2][256];
-  __shared__ float red[2][kAlsThreads / kWave];
+  __shared__ float red[kFinThreads / kWave][2][256];
+  __shared__ float dsum[LRQK_MAX_DECODE_ITERS];
   __shared__ int s_it;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.x;
   const int b = h / hq, head = h % hq;
   const int kvh = head / (hq / hkv);
-  // batch-wide stopping test, summed in a fixed order
+  const int vpr = 1 << vshift;  // vectors per row, a power of two <= 64
+  const int nvec = r << vshift;
+  // B tiles -> registers (independent loads, issued first)
+  Vec16<T> vq[kMaxVec], vk[kMaxVec];
+#pragma unroll
+  for (int u = 0; u < kMaxVec; ++u) {
+    const int vi = tid + u * kFinThreads;
+    if (vi < nvec) {
+      vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
+      vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
+    }
+  }
+  float qreg = 0.0f, kreg = 0.0f;
+  if (tid < d) {
+    qreg = ld_f32<T>(q, (int64_t)h * d + tid);
+    kreg = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + tid);
+  }
+  // batch-wide stopping test: wave `it` adds the heads' terms of iteration `it` in a fixed
+  // lane-strided order (the loads of one wave are in flight together)
+  for (int it = wave; it < max_iter; it += kFinThreads / kWave) {
+    float sacc = 0.0f;
+    for (int hh = lane; hh < bh; hh += kWave) sacc += deltas[(int64_t)hh * max_iter + it];
+    sacc = wave_sum(sacc);
+    if (lane == 0) dsum[it] = sacc;
+  }
+  __syncthreads();
   if (tid == 0) {
     int chosen = max_iter - 1;
     for (int it = 0; it < max_iter; ++it) {
-      float s = 0.0f;
-      for (int hh = 0; hh < bh; ++hh) s += deltas[(int64_t)hh * max_iter + it];
-      if (s / (float)((int64_t)bh * r) < tol) {
+      if (dsum[it] / (float)((int64_t)bh * r) < tol) {
         chosen = it;
         break;
       }
@@ -250,55 +450,99 @@ __global__ __launch_bounds__(kAlsThreads) void als_finish_kernel(T* __restrict__
   }
   __syncthreads();
   const float* o = iter_out + ((int64_t)h * max_iter + s_it) * 2 * r;
-  for (int i = tid; i < 2 * r; i += kAlsThreads) hat[i / r][i % r] = o[i];
+  if (tid < 2 * r) hat[tid >= r ? 1 : 0][tid >= r ? tid - r : tid] = o[tid];
   __syncthreads();
-  // e_q = q_hat B_Q - q ; e_k = k_hat B_K - k
-  float hn[2] = {0.0f, 0.0f};
-  for (int i = 0; i < r; ++i) {
-    hn[0] = fmaf(hat[0][i], hat[0][i], hn[0]);
-    hn[1] = fmaf(hat[1][i], hat[1][i], hn[1]);
-  }
-  float en[2] = {0.0f, 0.0f};
-  for (int c = tid; c < d; c += kAlsThreads) {
-    float eq = 0.0f, ek = 0.0f;
-    for (int i = 0; i < r; ++i) {
-      eq = fmaf(hat[0][i], ld_f32<T>(b_q, ((int64_t)h * r + i) * d + c), eq);
-      ek = fmaf(hat[1][i], ld_f32<T>(b_k, ((int64_t)h * r + i) * d + c), ek);
+  // column sums  sum_i hat[i] B[i][c]  for this thread's column group, both matrices
+  const int cg = tid & (vpr - 1);  // vpr divides 256, so the column group is fixed per thread
+  float pq[VEC], pk[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) pq[e] = pk[e] = 0.0f;
+#pragma unroll
+  for (int u = 0; u < kMaxVec; ++u) {
+    const int vi = tid + u * kFinThreads;
+    if (vi < nvec) {
+      const int row = vi >> vshift;
+      float fq[VEC], fk[VEC];
+      vq[u].unpack(fq);
+      vk[u].unpack(fk);
+      const float hq_ = hat[0][row], hk_ = hat[1][row];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        pq[e] = fmaf(hq_, fq[e], pq[e]);
+        pk[e] = fmaf(hk_, fk[e], pk[e]);
+      }
     }
-    eq -= ld_f32<T>(q, (int64_t)h * d + c);
-    ek -= ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
-    err[0][c] = eq;
-    err[1][c] = ek;
-    en[0] = fmaf(eq, eq, en[0]);
-    en[1] = fmaf(ek, ek, en[1]);
   }
-  en[0] = wave_sum(en[0]);
-  en[1] = wave_sum(en[1]);
-  if (lane_id() == 0) {
-    red[0][wave_id()] = en[0];
-    red[1][wave_id()] = en[1];
+  // lanes of a wave that share a column group differ in the lane-id bits >= vshift
+  for (int off = vpr; off < kWave; off <<= 1) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      pq[e] += __shfl_xor(pq[e], off, kWave);
+      pk[e] += __shfl_xor(pk[e], off, kWave);
+    }
+  }
+  if (lane < vpr) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      red[wave][0][cg * VEC + e] = pq[e];
+      red[wave][1][cg * VEC + e] = pk[e];
+    }
   }
   __syncthreads();
-  float e2[2] = {0.0f, 0.0f};
-  for (int w = 0; w < kAlsThreads / kWave; ++w) {
-    e2[0] += red[0][w];
-    e2[1] += red[1][w];
+  float en0 = 0.0f, en1 = 0.0f;
+  if (tid < d) {
+    float eq = -qreg, ek = -kreg;
+#pragma unroll
+    for (int w = 0; w < kFinThreads / kWave; ++w) {
+      eq += red[w][0][tid];
+      ek += red[w][1][tid];
+    }
+    err[0][tid] = eq;
+    err[1][tid] = ek;
+    en0 = eq * eq;
+    en1 = ek * ek;
+  }
+  en0 = wave_sum(en0);
+  en1 = wave_sum(en1);
+  __syncthreads();  // everyone is done reading red
+  if (lane == 0) {
+    red[wave][0][0] = en0;
+    red[wave][1][0] = en1;
+  }
+  __syncthreads();
+  float e2q = 0.0f, e2k = 0.0f, hnq = 0.0f, hnk = 0.0f;
+  for (int w = 0; w < kFinThreads / kWave; ++w) {
+    e2q += red[w][0][0];
+    e2k += red[w][1][0];
+  }
+  for (int i = 0; i < r; ++i) {
+    hnq = fmaf(hat[0][i], hat[0][i], hnq);
+    hnk = fmaf(hat[1][i], hat[1][i], hnk);
   }
   // dB = hat^T e : |dB|^2 = |hat|^2 |e|^2 ; hat dB = |hat|^2 e : |hat dB|^2 = |hat|^4 |e|^2
-  float lr[2];
-  for (int s = 0; s < 2; ++s) lr[s] = (hn[s] * e2[s]) / (hn[s] * hn[s] * e2[s] + 1e-6f);
-  for (int e = tid; e < r * d; e += kAlsThreads) {
-    const int i = e / d, c = e % d;
-    const int64_t off = (int64_t)h * r * d + e;
-    const float nq = ld_f32<T>(b_q, off) - lr[0] * (hat[0][i] * err[0][c]);
-    const float nk = ld_f32<T>(b_k, off) - lr[1] * (hat[1][i] * err[1][c]);
-    st_f32<T>(b_q, off, nq);
-    st_f32<T>(b_k, off, nk);
+  const float lrq = (hnq * e2q) / (hnq * hnq * e2q + 1e-6f);
+  const float lrk = (hnk * e2k) / (hnk * hnk * e2k + 1e-6f);
+#pragma unroll
+  for (int u = 0; u < kMaxVec; ++u) {
+    const int vi = tid + u * kFinThreads;
+    if (vi < nvec) {
+      const int row = vi >> vshift;
+      float fq[VEC], fk[VEC];
+      vq[u].unpack(fq);
+      vk[u].unpack(fk);
+      const float sq = lrq * hat[0][row], sk = lrk * hat[1][row];
+      const int64_t off = (int64_t)h * r * d + (int64_t)vi * VEC;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        st_f32<T>(b_q, off + e, fq[e] - sq * err[0][cg * VEC + e]);
+        st_f32<T>(b_k, off + e, fk[e] - sk * err[1][cg * VEC + e]);
+      }
+    }
   }
-  for (int i = tid; i < r; i += kAlsThreads) {
-    st_f32<T>(q_hat_out, (int64_t)h * r + i, hat[0][i]);
-    st_f32<T>(k_hat_out, (int64_t)h * r + i, hat[1][i]);
-    if (append_row >= 0) st_f32<T>(a_k, (int64_t)h * head_stride + append_row * r + i, hat[1][i]);
+  if (tid < r) {
+    st_f32<T>(q_hat_out, (int64_t)h * r + tid, hat[0][tid]);
+    st_f32<T>(k_hat_out, (int64_t)h * r + tid, hat[1][tid]);
+    if (append_row >= 0) st_f32<T>(a_k, (int64_t)h * head_stride + append_row * r + tid, hat[1][tid]);
   }
 }
 
@@ -312,35 +556,41 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   const int lpr = d / VEC;
   int lpr_log2 = 0;
   while ((1 << lpr_log2) < lpr) ++lpr_log2;
-  LRQK_REQUIRE(d % VEC == 0 && (1 << lpr_log2) == lpr && lpr <= kWave && d <= 256, LRQK_ELIMIT,
-               "head_dim %d unsupported (need a power-of-two number of 16-byte chunks, <= 256 elements)", d);
-  int S = (n + 63) / 64;
+  LRQK_REQUIRE(d % VEC == 0 && (1 << lpr_log2) == lpr && lpr <= kWave && d <= 256 && d >= 8, LRQK_ELIMIT,
+               "head_dim %d unsupported (need a power of two in 8..256 with at least one 16-byte chunk)", d);
+  LRQK_REQUIRE(((uintptr_t)b_q % 16 == 0) && ((uintptr_t)b_k % 16 == 0) && ((int64_t)r * d * sizeof(T)) % 16 == 0,
+               LRQK_EINVAL, "b_q/b_k must be 16-byte aligned");
+  // one 32-token chunk per wave where possible: a workgroup then pays two memory latencies
+  int S = (n + kGramWaves * kGramChunk - 1) / (kGramWaves * kGramChunk);
   if (S < 1) S = 1;
-  if (S > 64) S = 64;
-  const int ne = r * (r + 1);
-  int rc = ctx->als_part.ensure((size_t)bh * S * ne * sizeof(float));
+  if (S > 32) S = 32;
+  int rc = ctx->als_part.ensure((size_t)bh * S * kGramNe * sizeof(float));
   if (rc) return rc;
-  rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float));
-  if (rc) return rc;
+  if ((rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float)))) return rc;
   float* part = (float*)ctx->als_part.p;
   float* iter_out = (float*)ctx->als_iter.p;
   float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
   const int64_t a_rows = head_stride / r;
-  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kAlsThreads), 0, st, (const T*)a_k,
+
+  const size_t smem_solve = ((size_t)2 * 32 * (d + 1) + 2 * d + kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 +
+                             4 * 1024) * sizeof(float);
+  static size_t solve_allowed = 48 * 1024;
+  if (smem_solve > solve_allowed) {
+    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_solve_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem_solve));
+    solve_allowed = smem_solve;
+  }
+  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kGramThreads), 0, st, (const T*)a_k,
                      head_stride, a_rows, active_idx, idx_stride, (const T*)k_prev, kprev_slots, n, (const T*)q, r, d,
                      lpr_log2, part, S);
   LRQK_HIP_CHECK(hipGetLastError());
-  const size_t smem = ((size_t)2 * r * (d + 1) + 2 * d + 2 * r * (r + 1) + r * (r + 2) + 5 * r) * sizeof(float);
-  if (smem > 48 * 1024) {
-    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_solve_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem));
-  }
-  hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kAlsThreads), smem, st, (const T*)b_q,
-                     (const T*)b_k, part, S, (const T*)q, (const T*)k_new, hq, hkv, r, d, max_iter, iter_out, deltas);
+  hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const T*)b_q,
+                     (const T*)b_k, part, S, (const T*)q, (const T*)k_new, hq, hkv, r, d, lpr_log2, max_iter, iter_out,
+                     deltas);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((als_finish_kernel<T>), dim3((unsigned)bh), dim3(kAlsThreads), 0, st, (T*)b_q, (T*)b_k,
-                     (const T*)q, (const T*)k_new, iter_out, deltas, bh, hq, hkv, r, d, max_iter, tol, (T*)q_hat,
-                     (T*)k_hat, (T*)a_k, head_stride, append_row);
+  hipLaunchKernelGGL((als_finish_kernel<T>), dim3((unsigned)bh), dim3(kFinThreads), 0, st, (T*)b_q, (T*)b_k,
+                     (const T*)q, (const T*)k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol,
+                     (T*)q_hat, (T*)k_hat, (T*)a_k, head_stride, append_row);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -358,7 +608,8 @@ extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, i
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(b > 0 && hq > 0 && hkv > 0 && hq % hkv == 0 && (int64_t)b * hq <= 65535, LRQK_EINVAL,
                "bad heads b=%d hq=%d hkv=%d", b, hq, hkv);
-  LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_ELIMIT, "r=%d not in 1..%d", r, LRQK_MAX_R);
+  LRQK_REQUIRE(r > 0 && r <= kAlsMaxR, LRQK_ELIMIT, "r=%d not in 1..%d (the factor update supports rank <= %d)", r,
+               kAlsMaxR, kAlsMaxR);
   LRQK_REQUIRE(n > 0 && n <= kprev_slots, LRQK_EINVAL, "n=%d outside 1..%d", n, kprev_slots);
   LRQK_REQUIRE(!active_idx || idx_stride >= n, LRQK_EINVAL, "idx_stride < n");
   LRQK_REQUIRE(head_stride >= r && head_stride % r == 0, LRQK_EINVAL, "head_stride must be a multiple of r");

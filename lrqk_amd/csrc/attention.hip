@@ -1,5 +1,8 @@
 // Exact single-query attention over the active set: softmax(q K^T / sqrt(d)) V, split
-// along the slot axis so that one head fills many CUs, then a per-head combine.
+// along the slot axis so that one head fills many CUs, then a per-head combine of the
+// partial (max, sum, accumulator) triples.  (A device-scope fence per workgroup, which a
+// single-launch "last arrival combines" scheme needs, costs more than the second launch:
+// the L2 is per XCD.)
 #include <math.h>
 
 #include "common.hpp"
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
     for (int e = 0; e < VEC; ++e) red[wave][2 + sub * VEC + e] = acc[e];
   }
   __syncthreads();
-  float* out = part + ((int64_t)h * S + s) * (d + 2);
+  float* pout = part + ((int64_t)h * S + s) * (d + 2);
   float M = -INFINITY;
 #pragma unroll
   for (int w = 0; w < kAttnWaves; ++w) M = fmaxf(M, red[w][0]);
@@ -110,29 +113,54 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
         v += red[w][c] * f;
       }
     }
-    out[c] = v;
+    pout[c] = v;
   }
 }
 
+// One workgroup per head merges the S partial triples.  d is a power of two <= 256: thread ->
+// (column c, split group tg); every batch of loads is independent, so it costs one latency.
 template <typename T>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part, int S, int d,
-                                                           T* __restrict__ out) {
+__global__ __launch_bounds__(kAttnThreads) void attn_combine_kernel(const float* __restrict__ part, int S, int d,
+                                                                    T* __restrict__ out) {
+  __shared__ float red[kAttnThreads];
   const int h = blockIdx.x;
   const float* p = part + (int64_t)h * S * (d + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < S; ++s) M = fmaxf(M, p[(int64_t)s * (d + 2)]);
-  float L = 0.0f;
-  for (int s = 0; s < S; ++s) {
-    const float ms = p[(int64_t)s * (d + 2)];
-    L += (ms == -INFINITY) ? 0.0f : p[(int64_t)s * (d + 2) + 1] * exp2f(ms - M);
+  __shared__ float ms_s[64], ls_s[64];  // S <= 64
+  if (threadIdx.x < S) {
+    ms_s[threadIdx.x] = p[(int64_t)threadIdx.x * (d + 2)];
+    ls_s[threadIdx.x] = p[(int64_t)threadIdx.x * (d + 2) + 1];
   }
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float v = 0.0f;
-    for (int s = 0; s < S; ++s) {
-      const float ms = p[(int64_t)s * (d + 2)];
-      if (ms != -INFINITY) v += p[(int64_t)s * (d + 2) + 2 + c] * exp2f(ms - M);
+  __syncthreads();
+  float Mh = -INFINITY;
+  for (int t = 0; t < S; ++t) Mh = fmaxf(Mh, ms_s[t]);
+  float L = 0.0f;
+  for (int t = 0; t < S; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
+  // d is a power of two <= 256: thread -> (column c, split group tg)
+  const int c = threadIdx.x & (d - 1);
+  const int ntg = kAttnThreads / d;
+  const int tg = threadIdx.x / d;
+  float v = 0.0f;
+  for (int t0 = tg; t0 < S; t0 += 8 * ntg) {
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = t0 + u * ntg;
+      x[u] = 0.0f;
+      if (t < S) x[u] = p[(int64_t)t * (d + 2) + 2 + c];
     }
-    st_f32<T>(out, (int64_t)h * d + c, L > 0.0f ? v / L : 0.0f);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = t0 + u * ntg;
+      if (t < S && ms_s[t] != -INFINITY) v = fmaf(x[u], exp2f(ms_s[t] - Mh), v);
+    }
+  }
+  float* comb = red;
+  comb[threadIdx.x] = v;
+  __syncthreads();
+  if (tg == 0) {
+    float tot = 0.0f;
+    for (int g = 0; g < ntg; ++g) tot += comb[g * d + c];
+    st_f32<T>(out, (int64_t)h * d + c, L > 0.0f ? tot / L : 0.0f);
   }
 }
 
@@ -155,7 +183,7 @@ static int attention_impl(lrqk_ctx* ctx, const void* q, const void* k_act, const
                      (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, n_valid, d, lpr_log2, scale_log2e,
                      (float*)ctx->attn_part.p, S);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(d < 64 ? 64 : d), 0, st,
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kAttnThreads), 0, st,
                      (const float*)ctx->attn_part.p, S, d, (T*)out);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;

@@ -24,6 +24,14 @@ struct DevBuf {
     bytes = want;
     return LRQK_OK;
   }
+  // Same, and the block is zero-filled whenever it is (re)allocated.
+  int ensure_zeroed(size_t need) {
+    if (need <= bytes) return LRQK_OK;
+    int rc = ensure(need);
+    if (rc) return rc;
+    LRQK_HIP_CHECK(hipMemset(p, 0, bytes));
+    return LRQK_OK;
+  }
   void release() {
     if (p) (void)hipFree(p);
     p = nullptr;
@@ -39,7 +47,7 @@ struct lrqk_ctx {
   lrqk::DevBuf cand;        // candidate (key,idx) pairs for the fast select path
   lrqk::DevBuf cand_cnt;    // per-chunk counts / thresholds
   lrqk::DevBuf attn_part;   // f32 [bh][S][d+2]
-  lrqk::DevBuf als_part;    // f32 [bh][S][r*(r+1)]
+  lrqk::DevBuf als_part;    // f32 [bh][S][32*32 + 32]
   lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
@@ -48,4 +56,5 @@ struct lrqk_ctx {
   hipEvent_t* tev = nullptr;
   int tev_pairs = 0;   // capacity in pairs
   int tev_used = 0;    // pairs recorded since the last read
+  int sel_bh = 0;      // head count the selector state (t_low, counters) was initialised for
 };

@@ -56,6 +56,12 @@ class Workspace:
         check(_lib.load().lrqk_timing_read(self._h, ctypes.byref(ms), ctypes.byref(n)))
         return ms.value, n.value
 
+    def select_stats(self, reset: bool = True):
+        """(heads served from the candidate list, heads that rescanned) since the last reset."""
+        a, b = ctypes.c_int(), ctypes.c_int()
+        check(_lib.load().lrqk_select_stats(self._h, ctypes.byref(a), ctypes.byref(b), 1 if reset else 0))
+        return a.value, b.value
+
     def close(self):
         if self._h:
             _lib.load().lrqk_ctx_destroy(self._h)

@@ -104,6 +104,58 @@ def test_score_select_full_size(ops, ws, oracle, dtype, r):
         assert torch.all(got[..., 1:] > got[..., :-1]) and int(got.max()) < m
 
 
+def test_score_select_filtered_path(ops, oracle):
+    """Repeated calls on one workspace with a slowly drifting query: after the first call the
+    heads are served from the candidate list of the streaming filter; every result must
+    still equal the oracle's full sort, bit for bit."""
+    _say("score_select filtered path")
+    from lrqk_amd import synth
+    ws = ops.Workspace()
+    g = torch.Generator().manual_seed(11)
+    b, H, m, cap, r, k = 1, 6, 30000, 30016, 32, 2048
+    A = (torch.randn((b, H, cap, r), generator=g) * 0.5).bfloat16()
+    q = torch.randn((b, H, 1, r), generator=g)
+    Ad = A.to(DEV)
+    ws.select_stats()
+    for step in range(6):
+        qb = q.bfloat16()
+        exp = oracle.compute_hit_indices(qb, A[:, :, :m + step].contiguous(), k, True)[..., 0].to(torch.int32)
+        got = ops.score_select(ws, Ad, qb.to(DEV), m + step, k, True).cpu()
+        assert torch.equal(got, exp), step
+        q = synth.rotate_query(g, q, 0.05)
+    fast, full = ws.select_stats()
+    assert full >= H and fast >= 4 * H, (fast, full)       # first call rescans, later calls do not
+    # a jump of the score distribution must fall back, not fail: scale the query by 100 and by 0.01
+    for scale in (100.0, 0.01, -1.0):
+        qb = (q * scale).bfloat16()
+        exp = oracle.compute_hit_indices(qb, A[:, :, :m].contiguous(), k, True)[..., 0].to(torch.int32)
+        got = ops.score_select(ws, Ad, qb.to(DEV), m, k, True).cpu()
+        assert torch.equal(got, exp), scale
+
+
+def test_score_select_filtered_path_ties(ops, oracle):
+    """Scores crafted through a one-hot query: heavy ties at the threshold on the filtered path."""
+    _say("score_select filtered ties")
+    ws = ops.Workspace()
+    g = torch.Generator().manual_seed(12)
+    b, H, m, r, k = 1, 3, 20000, 8, 512
+    A = torch.zeros((b, H, m, r))
+    A[..., 0] = (torch.randn((b, H, m), generator=g) * 2).round() / 2    # about 20 distinct score values
+    A[..., 1:] = torch.randn((b, H, m, r - 1), generator=g)              # ignored by the query
+    q = torch.zeros((b, H, 1, r))
+    q[..., 0] = 1.0
+    exp = oracle.compute_hit_indices(q, A, k, False)[..., 0].to(torch.int32)
+    for _ in range(3):
+        got = ops.score_select(ws, A.to(DEV), q.to(DEV), m, k, False).cpu()
+        assert torch.equal(got, exp)
+    fast, full = ws.select_stats()
+    assert fast >= H, (fast, full)
+    # all scores equal: the candidate list overflows every time and the rescan path answers
+    A[..., 0] = 1.0
+    got = ops.score_select(ws, A.to(DEV), q.to(DEV), m, k, False).cpu()
+    assert torch.equal(got, torch.arange(k, dtype=torch.int32).expand(b, H, k))
+
+
 # ---------------------------------------------------------------- diff
 
 def _check_diff(ops, oracle, now, new):
