@@ -129,6 +129,7 @@ def main():
     kern_ms, launches = eng.ws.timing_read()
     eng.ws.timing_enable(0)
     sel_fast, sel_full = eng.ws.select_stats()
+    sel_short, sel_over = eng.ws.select_stats_detail()
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
 
@@ -183,7 +184,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "score_filter_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
-        "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full},
+        "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full, "list_short": sel_short,
+                           "list_overflow": sel_over},
         "cpu_baseline": cpu,
         "prefill_s": round(prefill_s, 3), "setup_s": round(setup_s, 2), "buffers_grew_in_timed_region": grew,
     }

@@ -72,6 +72,9 @@ int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int bh, int64_t 
  * call, or the score distribution moved).  Copies two counters from the device
  * (synchronises).  No counterpart in the reference. */
 int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads, int reset);
+/* Split of the full_heads reported by the last lrqk_select_stats call: lists that held fewer
+ * than k candidates, lists that overflowed. */
+int lrqk_select_stats_detail(lrqk_ctx* ctx, int* list_short, int* list_overflow);
 
 /* py:1275-1315 only_indices_in_cpu -- hit/miss diff, in place.
  * hit: [bh][hit_stride] current GPU-resident token ids (first k used), any order, unique.

@@ -78,42 +78,47 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
 
   for (int ch = 0; ch < n_chunks; ++ch) {
     const int c0 = w0 + ch * kGramChunk;
+    // Loads are unconditional (indices clamped into range, results masked afterwards): a
+    // conditional load compiles to a branch with a full wait, which would serialise them.
     // token ids this lane needs: tokens c0 + 2g + khalf, g = 0..15
     int src[kGramChunk / 2];
 #pragma unroll
     for (int g = 0; g < kGramChunk / 2; ++g) {
-      const int t = c0 + 2 * g + khalf;
-      src[g] = -1;
-      if (t < w1) src[g] = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      const int t = min(c0 + 2 * g + khalf, n - 1);
+      src[g] = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
     }
     // K rows of the chunk -> w
     for (int base0 = 0; base0 < kGramChunk; base0 += 8 * gpw) {
       Vec16<T> kv[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int row = base0 + u * gpw + grp;
-        if (row < kGramChunk && c0 + row < w1) kv[u].load(Kp + (int64_t)(c0 + row) * d + sub * VEC);
+        const int row = min(c0 + base0 + u * gpw + grp, n - 1);
+        kv[u].load(Kp + (int64_t)row * d + sub * VEC);
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int row = base0 + u * gpw + grp;
+        float kf[VEC];
+        kv[u].unpack(kf);
         float wv = 0.0f;
-        if (row < kGramChunk && c0 + row < w1) {
-          float kf[VEC];
-          kv[u].unpack(kf);
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) wv = fmaf(kf[e], qf[e], wv);
-        }
+        for (int e = 0; e < VEC; ++e) wv = fmaf(kf[e], qf[e], wv);
         for (int off = 1; off < lpr; off <<= 1) wv += __shfl_xor(wv, off, kWave);
-        if (sub == 0 && row < kGramChunk) w_s[row] = wv;
+        if (sub == 0 && row < kGramChunk) w_s[row] = (c0 + row < w1) ? wv : 0.0f;
       }
     }
     // A elements of the chunk: lane (col, khalf) holds A[token 2g + khalf][col]
     float a0[kGramChunk / 2];
+    const int colc = min(col, r - 1);
 #pragma unroll
     for (int g = 0; g < kGramChunk / 2; ++g) {
-      const int64_t sr = src[g];
-      a0[g] = (sr >= 0 && sr < a_rows && col < r) ? ld_f32<T>(A, sr * r + col) : 0.0f;
+      const int64_t sr = min(max((int64_t)src[g], (int64_t)0), a_rows - 1);
+      a0[g] = ld_f32<T>(A, sr * r + colc);
+    }
+#pragma unroll
+    for (int g = 0; g < kGramChunk / 2; ++g) {
+      const bool ok = (c0 + 2 * g + khalf < w1) && src[g] >= 0 && (int64_t)src[g] < a_rows && col < r;
+      a0[g] = ok ? a0[g] : 0.0f;
     }
     __syncthreads();  // w_s of this chunk is complete (every wave runs the same number of chunks)
 #pragma unroll
@@ -249,22 +254,25 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
     for (int u = 0; u < kPer; ++u) {
       const int e = tid + u * kSolveThreads;
 #pragma unroll
-      for (int t = 0; t < kMaxSplit; ++t) x[u][t] = (t < S && e < kGramNe) ? pin[(int64_t)t * kGramNe + e] : 0.0f;
+      for (int t = 0; t < kMaxSplit; ++t) x[u][t] = pin[(int64_t)min(t, S - 1) * kGramNe + min(e, kGramNe - 1)];
     }
     const int vpr = 1 << vshift;
     const int nvec = r << vshift;
     Vec16<T> vq[kMaxVec], vk[kMaxVec];
 #pragma unroll
     for (int u = 0; u < kMaxVec; ++u) {
-      const int vi = tid + u * kSolveThreads;
-      if (vi < nvec) {
-        vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
-        vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
-      }
+      const int vi = min(tid + u * kSolveThreads, nvec - 1);
+      vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
+      vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
     }
-    if (tid < d) {
-      qv[tid] = ld_f32<T>(q, (int64_t)h * d + tid);
-      kv[tid] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + tid);
+    {
+      const int c = min(tid, d - 1);
+      const float qx = ld_f32<T>(q, (int64_t)h * d + c);
+      const float kx = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
+      if (tid < d) {
+        qv[tid] = qx;
+        kv[tid] = kx;
+      }
     }
     // zero the padded rows of BQ/BK, then scatter the vectors
     for (int e = tid; e < (32 - r) * ld; e += kSolveThreads) {
@@ -290,7 +298,7 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
     for (int u = 0; u < kPer; ++u) {
       float v = 0.0f;
 #pragma unroll
-      for (int t = 0; t < kMaxSplit; ++t) v += x[u][t];  // fixed order 0..S-1 (zeros beyond)
+      for (int t = 0; t < kMaxSplit; ++t) v += (t < S) ? x[u][t] : 0.0f;  // fixed order 0..S-1
       gsum[u] = v;
       const int e = tid + u * kSolveThreads;
       if (e < kGramNe) G[e] = v;
@@ -418,17 +426,12 @@ __global__ __launch_bounds__(kFinThreads) void als_finish_kernel(T* __restrict__
   Vec16<T> vq[kMaxVec], vk[kMaxVec];
 #pragma unroll
   for (int u = 0; u < kMaxVec; ++u) {
-    const int vi = tid + u * kFinThreads;
-    if (vi < nvec) {
-      vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
-      vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
-    }
+    const int vi = min(tid + u * kFinThreads, nvec - 1);
+    vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
+    vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
   }
-  float qreg = 0.0f, kreg = 0.0f;
-  if (tid < d) {
-    qreg = ld_f32<T>(q, (int64_t)h * d + tid);
-    kreg = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + tid);
-  }
+  const float qreg = ld_f32<T>(q, (int64_t)h * d + min(tid, d - 1));
+  const float kreg = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + min(tid, d - 1));
   // batch-wide stopping test: wave `it` adds the heads' terms of iteration `it` in a fixed
   // lane-strided order (the loads of one wave are in flight together)
   for (int it = wave; it < max_iter; it += kFinThreads / kWave) {

@@ -50,29 +50,35 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
 #pragma unroll
   for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
 
-  for (int base = r0; base < r1; base += rows_per_iter) {
-    const int row = base + wave * gpw + grp;
-    const bool valid = row < r1;
-    const int rr = valid ? row : r1 - 1;
-    Vec16<T> kv, vv;
-    kv.load(Kh + (int64_t)rr * d + sub * VEC);
-    vv.load(Vh + (int64_t)rr * d + sub * VEC);
-    float kf[VEC], vf[VEC];
-    kv.unpack(kf);
-    vv.unpack(vf);
-    float sc = 0.0f;
+  // four row groups per pass: their K and V loads are issued together (one memory latency)
+  for (int base = r0; base < r1; base += 4 * rows_per_iter) {
+    Vec16<T> kv[4], vv[4];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) sc = fmaf(kf[e], qf[e], sc);
-    for (int off = 1; off < lpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);
-    if (!valid) sc = -INFINITY;
-    const float m_new = fmaxf(m_run, sc);
-    // exp2 of (-inf) - (-inf) must not produce NaN: while nothing valid was seen keep zeros
-    const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(m_run - m_new);
-    const float p = (m_new == -INFINITY) ? 0.0f : exp2f(sc - m_new);
-    l_run = l_run * alpha + p;
+    for (int u = 0; u < 4; ++u) {
+      const int rr = min(base + u * rows_per_iter + wave * gpw + grp, r1 - 1);
+      kv[u].load(Kh + (int64_t)rr * d + sub * VEC);
+      vv[u].load(Vh + (int64_t)rr * d + sub * VEC);
+    }
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = acc[e] * alpha + p * vf[e];
-    m_run = m_new;
+    for (int u = 0; u < 4; ++u) {
+      const bool valid = base + u * rows_per_iter + wave * gpw + grp < r1;
+      float kf[VEC], vf[VEC];
+      kv[u].unpack(kf);
+      vv[u].unpack(vf);
+      float sc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sc = fmaf(kf[e], qf[e], sc);
+      for (int off = 1; off < lpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);
+      if (!valid) sc = -INFINITY;
+      const float m_new = fmaxf(m_run, sc);
+      // exp2 of (-inf) - (-inf) must not produce NaN: while nothing valid was seen keep zeros
+      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(m_run - m_new);
+      const float p = (m_new == -INFINITY) ? 0.0f : exp2f(sc - m_new);
+      l_run = l_run * alpha + p;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = acc[e] * alpha + p * vf[e];
+      m_run = m_new;
+    }
   }
   // merge the row groups of this wave
   for (int off = lpr; off < kWave; off <<= 1) {
@@ -126,9 +132,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_combine_kernel(const float*
   const int h = blockIdx.x;
   const float* p = part + (int64_t)h * S * (d + 2);
   __shared__ float ms_s[64], ls_s[64];  // S <= 64
-  if (threadIdx.x < S) {
-    ms_s[threadIdx.x] = p[(int64_t)threadIdx.x * (d + 2)];
-    ls_s[threadIdx.x] = p[(int64_t)threadIdx.x * (d + 2) + 1];
+  if (threadIdx.x < 64) {
+    const int t = min((int)threadIdx.x, S - 1);
+    const float mv = p[(int64_t)t * (d + 2)], lv = p[(int64_t)t * (d + 2) + 1];
+    ms_s[threadIdx.x] = mv;
+    ls_s[threadIdx.x] = lv;
   }
   __syncthreads();
   float Mh = -INFINITY;
@@ -145,8 +153,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_combine_kernel(const float*
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int t = t0 + u * ntg;
-      x[u] = 0.0f;
-      if (t < S) x[u] = p[(int64_t)t * (d + 2) + 2 + c];
+      x[u] = p[(int64_t)min(t, S - 1) * (d + 2) + 2 + c];  // unconditional (clamped), masked below
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {

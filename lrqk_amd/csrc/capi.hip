@@ -90,6 +90,13 @@ extern "C" int lrqk_ctx_reserve(lrqk_ctx* ctx, int bh, int64_t max_tokens, int t
   return LRQK_OK;
 }
 
+extern "C" int lrqk_select_stats_detail(lrqk_ctx* ctx, int* list_short, int* list_overflow) {
+  LRQK_REQUIRE(ctx && list_short && list_overflow, LRQK_EINVAL, "null pointer");
+  *list_short = ctx->last_short;
+  *list_overflow = ctx->last_overflow;
+  return LRQK_OK;
+}
+
 extern "C" int lrqk_timing_enable(lrqk_ctx* ctx, int max_launches) {
   LRQK_REQUIRE(ctx != nullptr && max_launches >= 0 && max_launches <= (1 << 20), LRQK_EINVAL, "bad arguments");
   if (ctx->tev) {

@@ -57,4 +57,13 @@ struct lrqk_ctx {
   int tev_pairs = 0;   // capacity in pairs
   int tev_used = 0;    // pairs recorded since the last read
   int sel_bh = 0;      // head count the selector state (t_low, counters) was initialised for
+  int last_short = 0, last_overflow = 0;  // split of the rescans seen by the last lrqk_select_stats
 };
+
+namespace lrqk {
+// Proxy-score scan + top-k with the hit/miss diff fused into the select kernel when the
+// sizes allow.  Returns 1 if the diff ran, 0 if the caller still has to, negative on error.
+int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
+                      int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
+                      uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st);
+}  // namespace lrqk

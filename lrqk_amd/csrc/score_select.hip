@@ -1,4 +1,5 @@
-// Proxy-score scan q_hat . A_K^T and the per-head top-k selector.
+// Proxy-score scan q_hat . A_K^T, the per-head top-k selector, and (fused behind it) the
+// hit/miss diff against the resident set.
 //
 // Score contract: fp32 fmaf chain over j = 0..r-1 starting at +0, optional rounding to
 // bf16, -0 -> +0.  Selection order: (score descending, token index ascending); the
@@ -11,10 +12,14 @@
 //                  appended to a small per-head list.
 //   select       : one workgroup per head.  If the list holds at least k (and not too many)
 //                  candidates it provably contains the exact top-k including every tie at
-//                  the threshold, and the exact radix select runs on the list alone.
-//                  Otherwise (first call, distribution shift) the workgroup recomputes the
-//                  head's scores itself and selects over all of them.  Either way it leaves
-//                  the next t_low.  Results never depend on t_low, only speed does.
+//                  the threshold, and the exact radix select runs on the list alone, held
+//                  in registers.  Otherwise (first call, distribution shift) the workgroup
+//                  recomputes the head's scores itself and selects over all of them.  Either
+//                  way it leaves the next t_low.  Results never depend on t_low, only speed.
+//                  The radix digits are taken from (key - lowest key) shifted so that the
+//                  occupied range fills the 4096 bins: one or two passes instead of three.
+//                  The selected ids are emitted in order through two bitmaps (key > T,
+//                  key == T) and, when asked, diffed in place against the resident set.
 #include "common.hpp"
 #include "ctx.hpp"
 
@@ -36,6 +41,19 @@ struct RowScorer {
 #pragma unroll
       for (int j = 0; j < R; ++j) qf[j] = ld_f32<T>(q_head, j);
     }
+  }
+  __device__ __forceinline__ float q_norm() const {
+    float s = 0.0f;
+    if (R > 0) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) s = __builtin_fmaf(qf[j], qf[j], s);
+    } else {
+      for (int j = 0; j < r; ++j) {
+        const float x = ld_f32<T>(qh, j);
+        s = __builtin_fmaf(x, x, s);
+      }
+    }
+    return sqrtf(s);
   }
   __device__ __forceinline__ float score(const T* A, int64_t i) const {
     float acc = 0.0f;
@@ -94,13 +112,36 @@ __global__ __launch_bounds__(256) void arange_kernel(int32_t* out, int64_t out_s
     out[(int64_t)h * out_stride + i] = i;
 }
 
-__global__ void init_select_state_kernel(uint32_t* t_low, int* cand_count, int* stats, int bh) {
+// Per-head selector state: t_low (key that had rank ~2k at the previous call), q_norm (|q_hat|
+// of that call), t_used / q_cur (bound and norm the filter of the current call used).
+struct SelState {
+  uint32_t* t_low;
+  float* q_norm;
+  uint32_t* t_used;
+  float* q_cur;
+  int* cand_count;
+  int* stats;
+};
+
+__global__ void init_select_state_kernel(SelState st, int bh) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < bh) {
-    t_low[i] = 0xffffffffu;
-    cand_count[i] = 0;
+    st.t_low[i] = 0xffffffffu;
+    st.q_norm[i] = 0.0f;
+    st.t_used[i] = 0xffffffffu;
+    st.q_cur[i] = 0.0f;
+    st.cand_count[i] = 0;
   }
-  if (i < 2) stats[i] = 0;
+  if (i < 3) st.stats[i] = 0;
+}
+
+// The proxy scores scale with |q_hat|, so the bound carried over from the previous call is
+// rescaled by the ratio of the norms (positive bounds only) and relaxed by 2 %.
+__device__ __forceinline__ uint32_t rescaled_bound(uint32_t t_low, float q_norm_prev, float q_norm_now) {
+  if (t_low == 0xffffffffu || !(q_norm_prev > 0.0f) || !(q_norm_now > 0.0f)) return t_low;
+  const float s = key_score(t_low);
+  if (!(s > 0.0f)) return t_low;
+  return score_key(s * (q_norm_now / q_norm_prev) * 0.98f);
 }
 
 // --------------------------------------------------------------------------- score + filter
@@ -111,39 +152,58 @@ constexpr int kFiltRows = kFiltThreads * kFiltRPT;
 template <typename T, int R>
 __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __restrict__ a_k, int64_t head_stride,
                                                                     const T* __restrict__ q_hat, int64_t m, int r,
-                                                                    int round_bf16, const uint32_t* __restrict__ t_low,
-                                                                    uint2* __restrict__ cand, int cand_cap,
-                                                                    int* __restrict__ cand_count) {
+                                                                    int round_bf16, SelState st,
+                                                                    uint2* __restrict__ cand, int cand_cap) {
   __shared__ uint2 lc[kFiltRows];
   __shared__ int l_count, g_base;
   const int h = blockIdx.y;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = lane_id();
   const T* A = a_k + (int64_t)h * head_stride;
   RowScorer<T, R> rs;
-  rs.init(q_hat + (int64_t)h * r, r, round_bf16);
-  const uint32_t tl = t_low[h];
   if (tid == 0) l_count = 0;
   __syncthreads();
+  rs.init(q_hat + (int64_t)h * r, r, round_bf16);
+  const uint32_t t_prev = st.t_low[h];
+  const float qn_prev = st.q_norm[h];
   const int64_t base = (int64_t)blockIdx.x * kFiltRows;
-#pragma unroll 4
+  // pure streaming part: 8 rows per thread, loads unconditional (clamped), hits kept as a mask;
+  // the bound is derived after the row loads were issued so that its own loads overlap them
+  uint32_t keys[kFiltRPT];
+#pragma unroll
   for (int it = 0; it < kFiltRPT; ++it) {
     const int64_t i = base + it * kFiltThreads + tid;
-    const bool valid = i < m;
-    const uint32_t key = valid ? score_key(rs.score(A, i)) : 0u;
-    const bool pred = valid && key >= tl;
-    int tot;
-    const int rank = wave_rank(pred, tot);
+    keys[it] = score_key(rs.score(A, min(i, m - 1)));
+  }
+  const float qn = rs.q_norm();
+  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn);
+  if (tid == 0 && blockIdx.x == 0) {
+    st.t_used[h] = tl;
+    st.q_cur[h] = qn;
+  }
+  uint32_t mask = 0;
+#pragma unroll
+  for (int it = 0; it < kFiltRPT; ++it) {
+    const int64_t i = base + it * kFiltThreads + tid;
+    if (i < m && keys[it] >= tl) mask |= 1u << it;
+  }
+  // one LDS allocation per wave for all of its hits
+  const int cnt = __popc(mask);
+  const int incl = wave_inclusive_sum(cnt);
+  const int wtot = __shfl(incl, kWave - 1, kWave);
+  if (wtot) {
     int wbase = 0;
-    if (tot) {
-      if (lane_id() == 0) wbase = atomicAdd(&l_count, tot);
-      wbase = __shfl(wbase, 0, kWave);
-      if (pred) lc[wbase + rank] = make_uint2(key, (uint32_t)i);
+    if (lane == kWave - 1) wbase = atomicAdd(&l_count, wtot);
+    wbase = __shfl(wbase, kWave - 1, kWave);
+    int pos = wbase + incl - cnt;
+#pragma unroll
+    for (int it = 0; it < kFiltRPT; ++it) {
+      if ((mask >> it) & 1u) lc[pos++] = make_uint2(keys[it], (uint32_t)(base + it * kFiltThreads + tid));
     }
   }
   __syncthreads();
   const int n = l_count;
   if (n == 0) return;
-  if (tid == 0) g_base = atomicAdd(&cand_count[h], n);
+  if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n);
   __syncthreads();
   const int gb = g_base;
   for (int j = tid; j < n; j += kFiltThreads) {
@@ -152,81 +212,124 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
   }
 }
 
-// --------------------------------------------------------------------------- select
+// --------------------------------------------------------------------------- select (+ diff)
 constexpr int kSelThreads = 1024;
+constexpr int kSelWaves = kSelThreads / kWave;
 constexpr int kChunkBits = 262144;            // token ids covered by one bitmap pass
 constexpr int kChunkWords = kChunkBits / 32;  // 8192 words = 32 KB per bitmap
+constexpr int kBins = 4096;
+constexpr int kFusedDiffMaxK = 4096;          // LDS budget of the in-kernel diff
 
-__device__ __forceinline__ int block_inclusive_sum_1024(int v, int* scratch, int& total) {
-  int inc = wave_inclusive_sum(v);
-  if (lane_id() == kWave - 1) scratch[wave_id()] = inc;
-  __syncthreads();
-  int base = 0, tot = 0;
-  const int nw = blockDim.x >> 6;
-  for (int w = 0; w < nw; ++w) {
-    int c = scratch[w];
-    if (w < wave_id()) base += c;
-    tot += c;
+// Inclusive block scan of two counters at once.  scratch: 2 * kSelWaves ints.  Two barriers.
+__device__ __forceinline__ void block_inclusive_sum2(int& a, int& b, int* scratch, int& tot_a, int& tot_b) {
+  int ia = a, ib = b;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int ta = __shfl_up(ia, off, kWave), tb = __shfl_up(ib, off, kWave);
+    if (lane_id() >= off) {
+      ia += ta;
+      ib += tb;
+    }
+  }
+  if (lane_id() == kWave - 1) {
+    scratch[wave_id()] = ia;
+    scratch[kSelWaves + wave_id()] = ib;
   }
   __syncthreads();
-  total = tot;
-  return base + inc;
+  int base_a = 0, base_b = 0, ta = 0, tb = 0;
+#pragma unroll
+  for (int w = 0; w < kSelWaves; ++w) {
+    const int ca = scratch[w], cb = scratch[kSelWaves + w];
+    if (w < wave_id()) {
+      base_a += ca;
+      base_b += cb;
+    }
+    ta += ca;
+    tb += cb;
+  }
+  __syncthreads();
+  a = base_a + ia;
+  b = base_b + ib;
+  tot_a = ta;
+  tot_b = tb;
 }
 
-// Digit of the `need`-th largest element from a histogram of nb bins (nb = 4096 or 1024):
-// the largest digit D with count(digit > D) < need <= count(digit >= D).  Every thread
-// gets (D, need - count(digit > D)).  s_pair: 2 shared ints.
-__device__ __forceinline__ int find_digit(const uint32_t* hist, int nb, int need, int* scratch, int* s_pair,
-                                          int& need_out) {
+// From two histograms of kBins bins (4 bins per thread): the digit of the need_a-th largest
+// element of hist_a and of the need_b-th largest of hist_b, with the ranks inside those
+// digits.  s_res: 4 shared ints.  Three barriers.
+__device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32_t* hist_b, int need_a, int need_b,
+                                            int* scratch, int* s_res, int& dig_a, int& rem_a, int& dig_b, int& rem_b) {
   const int tid = threadIdx.x;
-  const int per = nb / kSelThreads;  // 4 or 1
-  int local = 0;
-  for (int b = 0; b < per; ++b) local += (int)hist[tid * per + b];
-  if (tid == 0) {
-    s_pair[0] = 0;
-    s_pair[1] = need;
+  int ca[4], cb[4], la = 0, lb = 0;
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    ca[x] = (int)hist_a[tid * 4 + x];
+    cb[x] = (int)hist_b[tid * 4 + x];
+    la += ca[x];
+    lb += cb[x];
   }
-  int total;
-  const int incl = block_inclusive_sum_1024(local, scratch, total);  // barriers order the init above
-  const int above = total - incl;
-  if (above < need && need <= above + local) {
-    int c = above;
-    for (int b = per - 1; b >= 0; --b) {
-      const int cnt = (int)hist[tid * per + b];
-      if (c + cnt >= need) {
-        s_pair[0] = tid * per + b;
-        s_pair[1] = need - c;
-        break;
+  int ia = la, ib = lb, ta, tb;
+  block_inclusive_sum2(ia, ib, scratch, ta, tb);
+  const int above_a = ta - ia, above_b = tb - ib;  // elements in bins above this thread's bins
+  if (above_a < need_a && need_a <= above_a + la) {
+    int c = above_a;
+#pragma unroll
+    for (int x = 3; x >= 0; --x) {
+      if (c < need_a && c + ca[x] >= need_a) {
+        s_res[0] = tid * 4 + x;
+        s_res[1] = need_a - c;
       }
-      c += cnt;
+      c += ca[x];
+    }
+  }
+  if (above_b < need_b && need_b <= above_b + lb) {
+    int c = above_b;
+#pragma unroll
+    for (int x = 3; x >= 0; --x) {
+      if (c < need_b && c + cb[x] >= need_b) {
+        s_res[2] = tid * 4 + x;
+        s_res[3] = need_b - c;
+      }
+      c += cb[x];
     }
   }
   __syncthreads();
-  const int d = s_pair[0];
-  need_out = s_pair[1];
-  __syncthreads();
-  return d;
+  dig_a = s_res[0];
+  rem_a = s_res[1];
+  dig_b = s_res[2];
+  rem_b = s_res[3];
 }
 
+struct DiffArgs {
+  int32_t* hit;        // [bh][hit_stride] resident token ids, nullptr = no diff
+  int64_t hit_stride;
+  uint8_t* evict;      // [bh][k] or nullptr
+  int32_t* miss_slots; // [bh][k] or nullptr
+  int32_t* miss_count; // [bh] or nullptr
+  int replace_all;     // ablation: hit <- new, everything refetched
+};
+
 // mode: 0 = use the candidate list if valid, else compute the head's keys from A_K;
-//       1 = keys[] already holds the head's keys (test hook / caller-provided scores).
+//       1 = keys[] already holds the head's keys (caller-provided scores).
+// Dynamic LDS: gt | eq bitmaps (2 * kChunkWords words), then, with a diff, 10*k bytes.
 template <typename T, int R>
 __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uint2* __restrict__ cand_all, int cand_cap,
-                                                             int* __restrict__ cand_count, uint32_t* __restrict__ t_low,
-                                                             uint32_t* __restrict__ keys_all, int64_t key_stride,
+                                                             SelState st, uint32_t* __restrict__ keys_all,
+                                                             int64_t key_stride,
                                                              const T* __restrict__ a_k, int64_t head_stride,
                                                              const T* __restrict__ q_hat, int64_t m, int r, int round_bf16,
                                                              int k, int32_t* __restrict__ out_all, int64_t out_stride,
-                                                             int* __restrict__ stats) {
-  extern __shared__ __align__(16) uint32_t bitmaps[];  // gt[kChunkWords] | eq[kChunkWords]
-  __shared__ uint32_t hist[4096];
-  __shared__ uint32_t hist_b[1024];
-  __shared__ int scratch[kSelThreads / kWave + 1];
-  __shared__ int s_pair[2];
+                                                             DiffArgs df) {
+  extern __shared__ __align__(16) uint32_t dyn[];
+  __shared__ uint32_t hist[kBins];
+  __shared__ uint32_t hist_b[kBins];
+  __shared__ int scratch[2 * kSelWaves];
+  __shared__ uint32_t wred[2 * kSelWaves];
+  __shared__ int s_res[4];
   __shared__ int s_n;
-  uint32_t* gt = bitmaps;
-  uint32_t* eq = bitmaps + kChunkWords;
-  const int tid = threadIdx.x;
+  uint32_t* gt = dyn;
+  uint32_t* eq = dyn + kChunkWords;
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.x;
   uint32_t* keys = keys_all + (int64_t)h * key_stride;
   const uint2* cand = cand_all + (int64_t)h * cand_cap;
@@ -234,16 +337,18 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
 
   bool fast = false;
   int64_t N = m;
+  uint32_t lo = 0;
   if (mode == 0) {
     if (tid == 0) {
-      s_n = cand_count[h];
-      cand_count[h] = 0;  // re-arm for the next call
+      s_n = st.cand_count[h];
+      st.cand_count[h] = 0;  // re-arm for the next call
     }
     __syncthreads();
     const int n = s_n;
     fast = n >= k && n <= cand_cap;
     if (fast) {
       N = n;
+      lo = st.t_used[h];  // every candidate key is >= the bound the filter used
     } else {
       const T* A = a_k + (int64_t)h * head_stride;
       RowScorer<T, R> rs;
@@ -252,7 +357,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       __threadfence_block();
       __syncthreads();
     }
-    if (tid == 0) atomicAdd(&stats[fast ? 0 : 1], 1);
+    if (tid == 0) atomicAdd(&st.stats[fast ? 0 : (n < k ? 1 : 2)], 1);
   }
   // The candidate list is read once into registers (one batch of independent loads); the
   // rescan path walks the key array in batches of 8 independent loads per thread.
@@ -263,7 +368,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
 #pragma unroll
     for (int u = 0; u < kRegCand; ++u) {
       const int64_t j = tid + (int64_t)u * kSelThreads;
-      creg[u] = j < N ? cand[j] : make_uint2(0u, 0u);
+      creg[u] = cand[min(j, N - 1)];  // unconditional (clamped); entries with j >= N are never used
     }
   }
   auto for_each = [&](auto&& f) {
@@ -282,10 +387,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       for (int64_t j0 = tid; j0 < N; j0 += (int64_t)8 * kSelThreads) {
         uint32_t kk[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int64_t j = j0 + (int64_t)u * kSelThreads;
-          kk[u] = j < N ? keys[j] : 0u;
-        }
+        for (int u = 0; u < 8; ++u) kk[u] = keys[min(j0 + (int64_t)u * kSelThreads, N - 1)];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int64_t j = j0 + (int64_t)u * kSelThreads;
@@ -295,45 +397,107 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
   };
 
-  const int k2 = (int)min((int64_t)2 * k, N);  // rank that defines the next t_low
-  // ---- pass 1: top 12 bits, shared by both ranks
-  for (int i = tid; i < 4096; i += kSelThreads) hist[i] = 0;
-  __syncthreads();
-  for_each([&](uint32_t key, int64_t) { atomicAdd(&hist[key >> 20], 1u); });
-  __syncthreads();
-  int need1, needE;
-  const uint32_t D1 = (uint32_t)find_digit(hist, 4096, k, scratch, s_pair, need1);
-  const uint32_t E1 = (uint32_t)find_digit(hist, 4096, k2, scratch, s_pair, needE);
-  // ---- pass 2: next 10 bits under each prefix
-  for (int i = tid; i < 1024; i += kSelThreads) {
+  // ---- range of the keys: lowest key (known for candidates), highest key, and the common
+  // trailing zero bits of (key - lo) (bf16-rounded scores leave 16 of them)
+  uint32_t vmin = 0xffffffffu, vmax = 0u, vor = 0u;
+  for_each([&](uint32_t key, int64_t) {
+    vmin = min(vmin, key);
+    vmax = max(vmax, key);
+  });
+  if (!fast) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) vmin = min(vmin, (uint32_t)__shfl_xor((int)vmin, off, kWave));
+    if (lane == 0) wred[wave] = vmin;
+    __syncthreads();
+    vmin = 0xffffffffu;
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) vmin = min(vmin, wred[w]);
+    lo = vmin;
+    __syncthreads();
+  }
+  for_each([&](uint32_t key, int64_t) { vor |= key - lo; });
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    vmax = max(vmax, (uint32_t)__shfl_xor((int)vmax, off, kWave));
+    vor |= (uint32_t)__shfl_xor((int)vor, off, kWave);
+  }
+  if (lane == 0) {
+    wred[wave] = vmax;
+    wred[kSelWaves + wave] = vor;
+  }
+  for (int i = tid; i < kBins; i += kSelThreads) {  // first-pass histograms, zeroed under the same barrier
     hist[i] = 0;
     hist_b[i] = 0;
   }
+  if (tid == 0) s_res[0] = s_res[1] = s_res[2] = s_res[3] = 0;
   __syncthreads();
-  for_each([&](uint32_t key, int64_t) {
-    const uint32_t top = key >> 20;
-    if (top == D1) atomicAdd(&hist[(key >> 10) & 1023u], 1u);
-    if (top == E1) atomicAdd(&hist_b[(key >> 10) & 1023u], 1u);
-  });
+  vmax = 0u;
+  vor = 0u;
+#pragma unroll
+  for (int w = 0; w < kSelWaves; ++w) {
+    vmax = max(vmax, wred[w]);
+    vor |= wred[kSelWaves + w];
+  }
+  const uint32_t range = vmax - lo;
+  const int tz = vor ? (__ffs((int)vor) - 1) : 0;              // bits that are zero in every offset
+  const int nbits = range ? (32 - __clz((int)(range >> tz))) : 0;  // significant bits of (key - lo) >> tz
+  const int s1 = max(nbits - 12, 0), s2 = max(s1 - 12, 0);
+
+  const int k2 = (int)min((int64_t)2 * k, N);  // rank that defines the next t_low
+  // ---- pass 1 (both ranks share it)
+  for_each([&](uint32_t key, int64_t) { atomicAdd(&hist[((key - lo) >> tz) >> s1], 1u); });
   __syncthreads();
-  int need2, needE2;
-  const uint32_t D2 = (uint32_t)find_digit(hist, 1024, need1, scratch, s_pair, need2);
-  const uint32_t E2 = (uint32_t)find_digit(hist_b, 1024, needE, scratch, s_pair, needE2);
-  if (tid == 0) t_low[h] = (E1 << 20) | (E2 << 10);
-  // ---- pass 3: last 10 bits
-  const uint32_t pre22 = (D1 << 10) | D2;
-  for (int i = tid; i < 1024; i += kSelThreads) hist[i] = 0;
-  __syncthreads();
-  for_each([&](uint32_t key, int64_t) {
-    if ((key >> 10) == pre22) atomicAdd(&hist[key & 1023u], 1u);
-  });
-  __syncthreads();
-  int need_eq;
-  const uint32_t D3 = (uint32_t)find_digit(hist, 1024, need2, scratch, s_pair, need_eq);
-  const uint32_t Tk = (pre22 << 10) | D3;
+  int D1, need1, E1, needE;
+  find_digits(hist, hist, k, k2, scratch, s_res, D1, need1, E1, needE);
+  uint32_t offT = (uint32_t)D1 << s1, offE = (uint32_t)E1 << s1;
+  int need_eq = need1;
+  if (s1 > 0) {
+    // ---- pass 2: next (up to) 12 bits under each prefix
+    for (int i = tid; i < kBins; i += kSelThreads) {
+      hist[i] = 0;
+      hist_b[i] = 0;
+    }
+    __syncthreads();
+    const uint32_t m2 = (1u << (s1 - s2)) - 1u;
+    for_each([&](uint32_t key, int64_t) {
+      const uint32_t o = (key - lo) >> tz;
+      const uint32_t top = o >> s1;
+      if (top == (uint32_t)D1) atomicAdd(&hist[(o >> s2) & m2], 1u);
+      if (top == (uint32_t)E1) atomicAdd(&hist_b[(o >> s2) & m2], 1u);
+    });
+    __syncthreads();
+    int D2, need2, E2, needE2;
+    find_digits(hist, hist_b, need1, needE, scratch, s_res, D2, need2, E2, needE2);
+    offT |= (uint32_t)D2 << s2;
+    offE |= (uint32_t)E2 << s2;
+    need_eq = need2;
+    if (s2 > 0) {
+      // ---- pass 3: the last s2 <= 8 bits
+      for (int i = tid; i < kBins; i += kSelThreads) hist[i] = 0;
+      __syncthreads();
+      const uint32_t m3 = (1u << s2) - 1u;
+      const uint32_t pre = offT >> s2;
+      for_each([&](uint32_t key, int64_t) {
+        const uint32_t o = (key - lo) >> tz;
+        if ((o >> s2) == pre) atomicAdd(&hist[o & m3], 1u);
+      });
+      __syncthreads();
+      int D3, need3, dummy_d, dummy_r;
+      find_digits(hist, hist, need2, need2, scratch, s_res, D3, need3, dummy_d, dummy_r);
+      offT |= (uint32_t)D3;
+      need_eq = need3;
+    }
+  }
+  const uint32_t Tk = lo + (offT << tz);
+  if (tid == 0) {
+    st.t_low[h] = lo + (offE << tz);  // rank >= 2k (rounded down to the resolved bits)
+    st.q_norm[h] = mode == 0 ? st.q_cur[h] : 0.0f;
+  }
 
   // ---- ordered output through two bitmaps over the token ids: gt (key > T), eq (key == T).
   // Every index with key > T is emitted, plus the first need_eq indices with key == T.
+  const bool do_diff = df.hit != nullptr;
+  int32_t* new_s = reinterpret_cast<int32_t*>(dyn + 2 * kChunkWords);  // [k] when do_diff
   int out_pos = 0, eq_seen = 0;
   for (int64_t c0 = 0; c0 < m; c0 += kChunkBits) {
     const int span = (int)min((int64_t)kChunkBits, m - c0);
@@ -355,23 +519,26 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       cg += __popc(gt[w]);
       ce += __popc(eq[w]);
     }
-    int g_tot, e_tot;
-    const int g_incl = block_inclusive_sum_1024(cg, scratch, g_tot);
-    const int e_incl = block_inclusive_sum_1024(ce, scratch, e_tot);
+    int g_incl = cg, e_incl = ce, g_tot, e_tot;
+    block_inclusive_sum2(g_incl, e_incl, scratch, g_tot, e_tot);
     int e_run = eq_seen + e_incl - ce;  // equal keys before this thread's words (all chunks)
     int pos = out_pos + (g_incl - cg) + (min(e_run, need_eq) - min(eq_seen, need_eq));
     for (int w = w0; w < min(words, w0 + W); ++w) {
       const uint32_t gw = gt[w], ew = eq[w];
       uint32_t both = gw | ew;
       while (both) {
-        const int bit = __ffs(both) - 1;
+        const int bit = __ffs((int)both) - 1;
         both &= both - 1;
         const int32_t idx = (int32_t)(c0 + (int64_t)w * 32 + bit);
-        if ((gw >> bit) & 1u) {
-          out[pos++] = idx;
-        } else {
-          if (e_run < need_eq) out[pos++] = idx;
+        bool take = true;
+        if (!((gw >> bit) & 1u)) {
+          take = e_run < need_eq;
           ++e_run;
+        }
+        if (take) {
+          out[pos] = idx;
+          if (do_diff) new_s[pos] = idx;
+          ++pos;
         }
       }
     }
@@ -379,6 +546,63 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     eq_seen += e_tot;
     __syncthreads();
   }
+  if (!do_diff) return;
+
+  // ---- hit/miss diff of this head (the selection is still in LDS).  new_s is ascending, so
+  // membership of a resident token is a binary search; a resident token that is found marks
+  // its position as matched, which yields the missing tokens without sorting the resident set.
+  int32_t* hit = df.hit + (int64_t)h * df.hit_stride;
+  if (df.replace_all) {
+    for (int s = tid; s < k; s += kSelThreads) {
+      hit[s] = new_s[s];
+      if (df.evict) df.evict[(int64_t)h * k + s] = 1;
+      if (df.miss_slots) df.miss_slots[(int64_t)h * k + s] = s;
+    }
+    if (tid == 0 && df.miss_count) df.miss_count[h] = k;
+    return;
+  }
+  int32_t* miss_s = new_s + k;                                   // [k] missing tokens, ascending
+  uint8_t* matched = reinterpret_cast<uint8_t*>(miss_s + k);     // [k]
+  uint8_t* evict_s = matched + k;                                // [k]
+  for (int i = tid; i < k; i += kSelThreads) matched[i] = 0;
+  __syncthreads();
+  for (int s = tid; s < k; s += kSelThreads) {
+    const int32_t v = hit[s];
+    int lo_i = 0, hi_i = k;
+    while (lo_i < hi_i) {
+      const int mid = (lo_i + hi_i) >> 1;
+      if (new_s[mid] < v) lo_i = mid + 1; else hi_i = mid;
+    }
+    const bool found = lo_i < k && new_s[lo_i] == v;
+    if (found) matched[lo_i] = 1;
+    evict_s[s] = found ? 0 : 1;
+  }
+  __syncthreads();
+  // both ordered compactions in one sweep: rank of missing tokens and of evicted slots
+  int n_missing = 0, n_evict = 0;
+  for (int base = 0; base < k; base += kSelThreads) {
+    const int i = base + tid;
+    const bool miss = i < k && matched[i] == 0;
+    const bool ev = i < k && evict_s[i] != 0;
+    int a = miss ? 1 : 0, b2 = ev ? 1 : 0, ta, tb;
+    block_inclusive_sum2(a, b2, scratch, ta, tb);
+    if (miss) miss_s[n_missing + a - 1] = new_s[i];
+    if (ev) reinterpret_cast<int32_t*>(gt)[n_evict + b2 - 1] = i;  // evicted slots, ascending (bitmaps are free now)
+    n_missing += ta;
+    n_evict += tb;
+  }
+  __syncthreads();
+  const int n_pair = min(n_missing, n_evict);
+  const int32_t* ev_list = reinterpret_cast<const int32_t*>(gt);
+  for (int j = tid; j < n_pair; j += kSelThreads) {
+    const int s = ev_list[j];
+    hit[s] = miss_s[j];
+    if (df.miss_slots) df.miss_slots[(int64_t)h * k + j] = s;
+  }
+  if (df.evict) {
+    for (int s = tid; s < k; s += kSelThreads) df.evict[(int64_t)h * k + s] = evict_s[s];
+  }
+  if (tid == 0 && df.miss_count) df.miss_count[h] = n_pair;
 }
 
 // --------------------------------------------------------------------------- host side
@@ -405,14 +629,14 @@ static int launch_scores(const void* a_k, int64_t head_stride, const void* q_hat
   return LRQK_OK;
 }
 
-constexpr size_t kSelSmem = (size_t)2 * kChunkWords * sizeof(uint32_t);
+static size_t select_smem(int k, bool with_diff) {
+  return (size_t)2 * kChunkWords * sizeof(uint32_t) + (with_diff ? (size_t)k * 10 : 0);
+}
 
 struct SelectBufs {
   uint2* cand;
   int cand_cap;
-  int* cand_count;
-  uint32_t* t_low;
-  int* stats;
+  SelState st;
   uint32_t* keys;
   int64_t key_stride;
 };
@@ -427,15 +651,19 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
   sb->cand_cap = 4 * topk < 4096 ? 4096 : 4 * topk;
   if ((rc = ctx->cand.ensure((size_t)bh * sb->cand_cap * sizeof(uint2)))) return rc;
   sb->cand = (uint2*)ctx->cand.p;
-  // layout: t_low u32 [bh] | cand_count i32 [bh] | stats i32 [2]
+  // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | cand_count i32 [bh] |
+  // stats i32 [3]: served from the list, rescans because the list was too short, because it overflowed
   void* before = ctx->cand_cnt.p;
-  if ((rc = ctx->cand_cnt.ensure((size_t)(2 * bh + 2) * 4))) return rc;
-  sb->t_low = (uint32_t*)ctx->cand_cnt.p;
-  sb->cand_count = (int*)(sb->t_low + bh);
-  sb->stats = sb->cand_count + bh;
+  if ((rc = ctx->cand_cnt.ensure((size_t)(5 * bh + 3) * 4))) return rc;
+  uint32_t* base = (uint32_t*)ctx->cand_cnt.p;
+  sb->st.t_low = base;
+  sb->st.q_norm = (float*)(base + bh);
+  sb->st.t_used = base + 2 * bh;
+  sb->st.q_cur = (float*)(base + 3 * bh);
+  sb->st.cand_count = (int*)(base + 4 * bh);
+  sb->st.stats = (int*)(base + 5 * bh);
   if (before != ctx->cand_cnt.p || ctx->sel_bh != bh) {
-    hipLaunchKernelGGL(init_select_state_kernel, dim3((unsigned)((bh + 255) / 256)), dim3(256), 0, st, sb->t_low,
-                       sb->cand_count, sb->stats, bh);
+    hipLaunchKernelGGL(init_select_state_kernel, dim3((unsigned)((bh + 255) / 256)), dim3(256), 0, st, sb->st, bh);
     LRQK_HIP_CHECK(hipGetLastError());
     ctx->sel_bh = bh;
   }
@@ -445,26 +673,27 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
 template <typename T, int R>
 static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void* a_k, int64_t head_stride,
                                 const void* q_hat, int bh, int64_t m, int r, int round_bf16, int topk, int32_t* out_idx,
-                                int64_t out_stride, hipStream_t st) {
-  static bool attr_done = false;
-  if (!attr_done) {
+                                int64_t out_stride, const DiffArgs& df, hipStream_t st) {
+  const size_t smem = select_smem(topk, df.hit != nullptr);
+  static size_t smem_allowed = 0;
+  if (smem > smem_allowed) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_kernel<T, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kSelSmem));
-    attr_done = true;
+                                       (int)smem));
+    smem_allowed = smem;
   }
   const bool timed = ctx->tev && ctx->tev_used < ctx->tev_pairs;
   if (timed) LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used], st));
   dim3 grid((unsigned)((m + kFiltRows - 1) / kFiltRows), (unsigned)bh);
   hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), 0, st, (const T*)a_k, head_stride,
-                     (const T*)q_hat, m, r, round_bf16, sb.t_low, sb.cand, sb.cand_cap, sb.cand_count);
+                     (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap);
   LRQK_HIP_CHECK(hipGetLastError());
   if (timed) {
     LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used + 1], st));
     ++ctx->tev_used;
   }
-  hipLaunchKernelGGL((select_kernel<T, R>), dim3((unsigned)bh), dim3(kSelThreads), kSelSmem, st, 0, sb.cand, sb.cand_cap,
-                     sb.cand_count, sb.t_low, sb.keys, sb.key_stride, (const T*)a_k, head_stride, (const T*)q_hat, m, r,
-                     round_bf16, topk, out_idx, out_stride, sb.stats);
+  hipLaunchKernelGGL((select_kernel<T, R>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, 0, sb.cand, sb.cand_cap,
+                     sb.st, sb.keys, sb.key_stride, (const T*)a_k, head_stride, (const T*)q_hat, m, r, round_bf16, topk,
+                     out_idx, out_stride, df);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -472,10 +701,11 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
 template <typename T>
 static int dispatch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void* a_k, int64_t head_stride,
                                   const void* q_hat, int bh, int64_t m, int r, int round_bf16, int topk,
-                                  int32_t* out_idx, int64_t out_stride, hipStream_t st) {
+                                  int32_t* out_idx, int64_t out_stride, const DiffArgs& df, hipStream_t st) {
   const bool vec_ok = ((uintptr_t)a_k % 16 == 0) && ((head_stride * sizeof(T)) % 16 == 0);
-#define LRQK_FS_CASE(RR) \
-  return launch_filter_select<T, RR>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, out_idx, out_stride, st)
+#define LRQK_FS_CASE(RR)                                                                                            \
+  return launch_filter_select<T, RR>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, out_idx, out_stride, \
+                                     df, st)
   if (vec_ok && r == 64) LRQK_FS_CASE(64);
   if (vec_ok && r == 32) LRQK_FS_CASE(32);
   if (vec_ok && r == 16) LRQK_FS_CASE(16);
@@ -501,6 +731,29 @@ static int arange_result(int bh, int64_t m, int32_t* out_idx, int64_t out_stride
     LRQK_HIP_CHECK(hipGetLastError());
   }
   return (int)m;
+}
+
+// Scan + select with the hit/miss diff fused into the select kernel (k <= kFusedDiffMaxK and
+// m > k); used by the fused decode step.  Returns 1 if the diff was fused, 0 if the caller
+// still has to run it, negative on error.
+int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
+                      int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
+                      uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st) {
+  int rc = check_select_args(ctx, bh, m, topk, new_idx, topk);
+  if (rc) return rc;
+  if (m <= topk || topk > kFusedDiffMaxK) {
+    rc = lrqk_score_select(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_bf16, new_idx, topk, st);
+    return rc < 0 ? rc : 0;
+  }
+  SelectBufs sb;
+  if ((rc = prepare_select(ctx, bh, m, topk, st, &sb))) return rc;
+  DiffArgs df{hit, hit_stride, evict, miss_slots, miss_count, replace_all};
+  if (dtype == LRQK_F32)
+    rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, new_idx, topk, df, st);
+  else
+    rc = dispatch_filter_select<bf16_t>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, new_idx, topk, df,
+                                        st);
+  return rc ? rc : 1;
 }
 
 }  // namespace lrqk
@@ -534,11 +787,12 @@ extern "C" int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_st
   if (m <= topk) return arange_result(bh, m, out_idx, out_stride, st);
   SelectBufs sb;
   if ((rc = prepare_select(ctx, bh, m, topk, st, &sb))) return rc;
+  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0};
   if (dtype == LRQK_F32)
-    rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, out_idx, out_stride, st);
+    rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, out_idx, out_stride, df, st);
   else
     rc = dispatch_filter_select<bf16_t>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, out_idx,
-                                        out_stride, st);
+                                        out_stride, df, st);
   return rc ? rc : topk;
 }
 
@@ -556,15 +810,17 @@ extern "C" int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int b
   hipLaunchKernelGGL(keys_from_scores_kernel, dim3((unsigned)blocks, (unsigned)bh), dim3(256), 0, st, scores, m, sb.keys,
                      sb.key_stride);
   LRQK_HIP_CHECK(hipGetLastError());
+  const size_t smem = select_smem(topk, false);
   static bool attr_done = false;
   if (!attr_done) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_kernel<float, 0>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kSelSmem));
+                                       (int)smem));
     attr_done = true;
   }
-  hipLaunchKernelGGL((select_kernel<float, 0>), dim3((unsigned)bh), dim3(kSelThreads), kSelSmem, st, 1, sb.cand,
-                     sb.cand_cap, sb.cand_count, sb.t_low, sb.keys, sb.key_stride, (const float*)nullptr, (int64_t)0,
-                     (const float*)nullptr, m, 1, 0, topk, out_idx, out_stride, sb.stats);
+  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0};
+  hipLaunchKernelGGL((select_kernel<float, 0>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, 1, sb.cand, sb.cand_cap,
+                     sb.st, sb.keys, sb.key_stride, (const float*)nullptr, (int64_t)0, (const float*)nullptr, m, 1, 0,
+                     topk, out_idx, out_stride, df);
   LRQK_HIP_CHECK(hipGetLastError());
   return topk;
 }
@@ -573,11 +829,13 @@ extern "C" int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads
   LRQK_REQUIRE(ctx && fast_heads && full_heads, LRQK_EINVAL, "null pointer");
   *fast_heads = *full_heads = 0;
   if (!ctx->cand_cnt.p || ctx->sel_bh <= 0) return LRQK_OK;
-  int* stats = (int*)ctx->cand_cnt.p + 2 * ctx->sel_bh;
-  int v[2];
+  int* stats = (int*)ctx->cand_cnt.p + 5 * ctx->sel_bh;
+  int v[3];
   LRQK_HIP_CHECK(hipMemcpy(v, stats, sizeof(v), hipMemcpyDeviceToHost));
   *fast_heads = v[0];
-  *full_heads = v[1];
+  *full_heads = v[1] + v[2];
+  ctx->last_short = v[1];
+  ctx->last_overflow = v[2];
   if (reset) LRQK_HIP_CHECK(hipMemset(stats, 0, sizeof(v)));
   return LRQK_OK;
 }

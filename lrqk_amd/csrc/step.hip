@@ -38,13 +38,16 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   if ((rc = lrqk_als_decode(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, n, n, q, k_new, b, hq, hkv, r, d,
                             max_iter, tol, q_hat, k_hat, token, dtype, stream)))
     return rc;
-  rc = lrqk_score_select(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, topk, stream);
+  rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, active_idx, n, ev,
+                         miss_slots, mcount, no_hit_miss, (hipStream_t)stream);
   if (rc < 0) return rc;
-  if (no_hit_miss)
-    rc = lrqk_replace_all(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
-  else
-    rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
-  if (rc) return rc;
+  if (rc == 0) {  // sizes outside the fused kernel's LDS budget: separate diff launch
+    if (no_hit_miss)
+      rc = lrqk_replace_all(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
+    else
+      rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
+    if (rc) return rc;
+  }
   if ((rc = lrqk_fetch_rows(kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv, d, topk, dtype,
                             stream)))
     return rc;

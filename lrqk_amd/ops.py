@@ -62,6 +62,12 @@ class Workspace:
         check(_lib.load().lrqk_select_stats(self._h, ctypes.byref(a), ctypes.byref(b), 1 if reset else 0))
         return a.value, b.value
 
+    def select_stats_detail(self):
+        """(lists too short, lists overflowed) among the rescans of the last select_stats()."""
+        a, b = ctypes.c_int(), ctypes.c_int()
+        check(_lib.load().lrqk_select_stats_detail(self._h, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
     def close(self):
         if self._h:
             _lib.load().lrqk_ctx_destroy(self._h)
