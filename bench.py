@@ -27,6 +27,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch of the proxy-score kernel read from hardware counters (rocprofv3 --pmc FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB device copy: x2.000 and x1.000), per
+# workload at its default context.  The summary of those runs is kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {"llama8b_128k_bf16": (131206.3 * 2.000 + 1106.6 * 1.000) * 1024}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -40,6 +45,9 @@ def parse():
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
+    p.add_argument("--calib-copy-mb", type=int, default=0,
+                   help="after the timed region, run one plain device copy of this many MiB (a known-size "
+                        "kernel to scale hardware counters by)")
     return p.parse_args()
 
 
@@ -148,6 +156,14 @@ def main():
                   + bh * n_act * w.r * e + 4 * bh * w.r * w.head_dim * e + 3 * bh * w.num_active_tokens * 4
                   + n_miss / a.steps * row_bytes)
 
+    if a.calib_copy_mb > 0:
+        src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     cpu = None
     if a.cpu_steps > 0:
         threads = a.cpu_threads or min(16, os.cpu_count() or 1)
@@ -182,7 +198,9 @@ def main():
         "step_algorithmic_bytes": round(step_bytes),
         "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": "score_filter_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": (round(MEASURED_TRAFFIC_BYTES[w.name]) if w.name in MEASURED_TRAFFIC_BYTES
+                                 and a.context is None and a.variant == "default" else None),
                      "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
         "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full, "list_short": sel_short,
                            "list_overflow": sel_over},
