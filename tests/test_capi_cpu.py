@@ -91,3 +91,14 @@ def test_take_along_dim_with_mask_rejects_like_the_reference():
         ops.take_along_dim_with_mask(src.transpose(2, 3), ind, mask)
     with pytest.raises(ValueError):
         ops.take_along_dim_with_mask(src, ind + 4, mask)                                    # out of range
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path is measured on one GPU: any other count exits non-zero with a message."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert p.returncode != 0
+    assert "one GPU" in p.stderr
