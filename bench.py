@@ -45,6 +45,9 @@ def parse():
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
+    p.add_argument("--mode", default="decode", choices=["decode", "prefill_als"],
+                   help="prefill_als: time the prefill factorisation alone (workload llama8b_32k_prefill_als unless "
+                        "--workload is given); a step is one whole factorisation")
     p.add_argument("--calib-copy-mb", type=int, default=0,
                    help="after the timed region, run one plain device copy of this many MiB (a known-size "
                         "kernel to scale hardware counters by)")
@@ -71,6 +74,64 @@ def oracle_from_engine(eng, w, threads):
     return o, orc
 
 
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak, published
+
+
+def prefill_als(a):
+    """Times lrqk_als_prefill on synthetic low-rank + noise Q, K and reports fit residuals."""
+    from lrqk_amd import synth, ops
+    dev = torch.device("cuda:0")
+    w = synth.WORKLOADS[a.workload if a.workload != "llama8b_128k_bf16" else "llama8b_32k_prefill_als"]
+    l = a.context or w.context
+    Q, K, V, bases, gen = synth.prompt_qkv(w, a.seed, l, device=dev)
+    del V
+    A0 = synth.init_factors(w, l, a.seed + 1, device=dev)
+    ws = ops.Workspace()
+    iters, tol = w.max_iter[0], w.tol[0]
+    steps, warm = min(a.steps, 8), min(a.warmup, 2)
+    res = None
+    times = []
+    for i in range(warm + steps):
+        aq, ak = A0[0].clone(), A0[1].clone()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        res = ops.als_prefill(ws, Q, K, aq, ak, iters, tol)
+        torch.cuda.synchronize()
+        if i >= warm:
+            times.append(time.perf_counter() - t0)
+    ms = sum(times) / len(times) * 1e3
+    AQ, BQ, AK, BK = res
+    g = w.num_heads // w.num_kv_heads
+    # residuals head by head (the fp32 copy of all heads at once would double the footprint)
+    num_k = den_k = num_q = den_q = 0.0
+    for h in range(w.num_heads):
+        Kh = K[:, h // g].float()
+        Qh = Q[:, h].float()
+        num_k += float((Kh - AK[:, h] @ BK[:, h]).pow(2).sum()); den_k += float(Kh.pow(2).sum())
+        num_q += float((Qh - AQ[:, h] @ BQ[:, h]).pow(2).sum()); den_q += float(Qh.pow(2).sum())
+    bh = w.batch * w.num_heads
+    r, d = w.r, w.head_dim
+    # one pass = apply (2 l d r) + Grams (2 l r (r + d)); 2 initial Gram passes + 2 passes per iteration
+    flops = bh * (2 * 2.0 * l * r * (r + d) + iters * 2 * (2.0 * l * d * r + 2.0 * l * r * (r + d)))
+    e = 2 if w.dtype == torch.bfloat16 else 4
+    # HBM bytes: every pass reads X once; apply passes read and write A (fp32), Gram passes read A
+    bytes_ = bh * ((2 + 2 * iters) * l * d * e + 2 * l * r * 4 + iters * 2 * 2 * l * r * 4)
+    tf = flops / (ms * 1e-3) / 1e12
+    out = {"metric": "lrqk_prefill_als_ms", "value": round(ms, 3), "unit": "ms", "n_gpus": 1, "steps": steps,
+           "warmup": warm, "ms_per_step": round(ms, 3), "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": d, "r": r,
+                      "max_iter": iters, "tol": tol, "input_dtype": "bf16" if e == 2 else "f32"},
+           "rel_residual_K": round((num_k / den_k) ** 0.5, 6), "rel_residual_Q": round((num_q / den_q) ** 0.5, 6),
+           "roofline": {"bound": "mfma", "kernel": "pf_pass_mfma_kernel", "achieved": round(tf, 2),
+                        "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
+                        "traffic": None, "flops_per_call": round(flops),
+                        "hbm_bytes_per_call": round(bytes_),
+                        "hbm_frac": round(bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+           "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -84,6 +145,8 @@ def main():
     import lrqk_amd
     from lrqk_amd import _lib
     _lib.load()  # fail loudly if the HIP library is missing
+    if a.mode == "prefill_als":
+        return prefill_als(a)
 
     dev = torch.device("cuda:0")
     w = synth.WORKLOADS[a.workload]

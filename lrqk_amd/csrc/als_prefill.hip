@@ -8,6 +8,10 @@
 // The stopping test (a batch-wide mean squared change) is evaluated on the device; once
 // it fires the remaining launches of the loop return immediately, so the host never
 // waits inside the loop.
+//
+// Two implementations of each kernel: fp32 MFMA (32x32x2) tiles for r <= 32 and head
+// dimensions that are a multiple of the 16-byte vector, and a generic VALU version for
+// every other shape.  Both write the same partial-sum layout.
 #include <algorithm>
 
 #include "common.hpp"
@@ -41,7 +45,7 @@ __device__ __forceinline__ void accumulate_gram(const float* a_s, int lda, const
 
 // X: [b][xh][l][d] storage dtype; head h of the factors reads X head (h % hq) / (hq / xh).
 template <typename T>
-__global__ __launch_bounds__(kPfThreads) void pf_pass_kernel(const T* __restrict__ X, int xh, int hq, int64_t l, int r,
+__global__ __launch_bounds__(kPfThreads) void pf_pass_generic_kernel(const T* __restrict__ X, int xh, int hq, int64_t l, int r,
                                                              int d, const float* __restrict__ Mt, float* __restrict__ A,
                                                              float* __restrict__ part, float* __restrict__ delta_part,
                                                              const int* __restrict__ done_flag, int S) {
@@ -138,7 +142,7 @@ __device__ __forceinline__ void reduce_part(const float* part, int S, int ne, fl
 // stage 0: (stopping test) B_Q, B_K from the current Grams, then Mt for the A_Q update
 // stage 1: Mt for the A_K update from the new A_Q Grams
 // stage 2: final B_Q, B_K
-__global__ __launch_bounds__(kPfThreads) void pf_small_kernel(int stage, int it, const float* __restrict__ partQ,
+__global__ __launch_bounds__(kPfThreads) void pf_small_generic_kernel(int stage, int it, const float* __restrict__ partQ,
                                                               const float* __restrict__ partK, int S, int bh, int r,
                                                               int d, int64_t l, float tol,
                                                               const float* __restrict__ delta_all, int* __restrict__ flags,
@@ -249,14 +253,483 @@ __global__ __launch_bounds__(kPfThreads) void pf_small_kernel(int stage, int it,
   }
 }
 
+
+// ============================================================================ MFMA path
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kPfSmallThreads = 320;  // one thread per column of [32 x 32 | 32 x d], d <= 288
+
+// C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
+__device__ __forceinline__ int pf_mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
+
+// One wave owns 32 rows of X at a time (staged as fp32 in its private LDS tile, row stride
+// 32*NB+4, zero beyond d and beyond the last row).
+//   apply:  C[32 x 32] = X[32 x d] Mt^T          (A operand from LDS, B operand = Mt)
+//   gram:   G_AA += C^T C, G_AX += C^T X          (the C registers are the A operand as they are:
+//           element v of lane l is row pf_mfma_row(l, v), and a sum over rows may visit them in any order)
+// The k index of the apply and the column index of G_AX are permuted so that every lane reads
+// consecutive floats of its LDS row with 16-byte loads: MFMA step kk multiplies columns kk and
+// kk + 16*NB; tile nb of G_AX holds the columns n*NB + nb.
+// NB = number of 32-column blocks of X.  NW waves per workgroup; the tiles are wave-private, so
+// the waves only meet at the start and in the final reduction and otherwise drift apart (one
+// wave's staging overlaps another's MFMAs on the same SIMD).  MT_LDS: Mt is kept in LDS (shared
+// by the waves) instead of registers, which leaves room for two waves per SIMD.
+
+// orders this wave's LDS writes before its later LDS reads (the tile is exchanged between lanes)
+__device__ __forceinline__ void pf_wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T, int NB, int NW, bool MT_LDS>
+__global__ __launch_bounds__(NW * kWave) void pf_pass_mfma_kernel(const T* __restrict__ X, int xh, int hq, int64_t l,
+                                                                  int r, int d, const float* __restrict__ Mt,
+                                                                  float* __restrict__ A, float* __restrict__ part,
+                                                                  float* __restrict__ delta_part,
+                                                                  const int* __restrict__ done_flag, int S) {
+  if (done_flag && *done_flag) return;
+  constexpr int LDX = 32 * NB + 4;
+  constexpr int KH = 16 * NB;
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int NL = 32 * 32 * NB / (kWave * VEC);
+  constexpr int NT = NW * kWave;
+  extern __shared__ __align__(16) float sm[];
+  __shared__ float red[NW];
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int col = lane & 31, half = lane >> 5;
+  float* x_s = sm + wave * 32 * LDX;
+  float* mt_s = sm + NW * 32 * LDX;  // [32][LDX], MT_LDS only
+  const int h = blockIdx.y, s = blockIdx.x;
+  const int b = h / hq, head = h % hq;
+  const int64_t xhead = (int64_t)b * xh + head / (hq / xh);
+  const T* Xh = X + xhead * l * d;
+  float* Ah = A + (int64_t)h * l * r;
+  const bool apply = Mt != nullptr;
+  const bool full_rows = d == 32 * NB;  // row / column of a flat element index by shifts
+
+  float mt[MT_LDS ? 1 : KH];
+  if (apply) {
+    const float* Mh = Mt + (int64_t)h * r * d;
+    if constexpr (MT_LDS) {
+      for (int e = tid; e < 32 * 32 * NB; e += NT) {
+        const int n = e / (32 * NB), k = e % (32 * NB);
+        const float v = Mh[min(n, r - 1) * d + min(k, d - 1)];
+        mt_s[n * LDX + k] = (n < r && k < d) ? v : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < KH; ++kk) {
+        const int k = kk + half * KH;
+        const float v = Mh[min(col, r - 1) * d + min(k, d - 1)];
+        mt[kk] = (col < r && k < d) ? v : 0.0f;
+      }
+    }
+  }
+  for (int e = lane; e < 32 * LDX; e += kWave) x_s[e] = 0.0f;
+
+  const int64_t rows_per_split = (((l + S - 1) / S) + 31) / 32 * 32;
+  const int64_t r0 = (int64_t)s * rows_per_split;
+  const int64_t r1 = min(l, r0 + rows_per_split);
+
+  floatx16 gAA;
+  floatx16 gAX[NB];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) gAA[v] = 0.0f;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) gAX[nb][v] = 0.0f;
+  float dsum = 0.0f;
+
+  Vec16<T> pre[NL];
+  auto issue = [&](int64_t t0) {
+    const int nvalid = t0 < r1 ? (int)min((int64_t)32, r1 - t0) * d : 0;
+    const int64_t base = (t0 < r1 ? t0 : r0) * d;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int e = (i * kWave + lane) * VEC;
+      pre[i].load(Xh + base + (e < nvalid ? e : 0));
+    }
+  };
+  if (r0 + (int64_t)wave * 32 < r1) issue(r0 + (int64_t)wave * 32);
+  __syncthreads();  // Mt staged, tiles cleared
+
+  for (int64_t t0 = r0 + (int64_t)wave * 32; t0 < r1; t0 += 32 * NW) {
+    const int rows = (int)min((int64_t)32, r1 - t0);
+    // stage this wave's rows
+    {
+      const int nvalid = rows * d;
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int e = (i * kWave + lane) * VEC;
+        if (e < 32 * d) {
+          float f[VEC];
+          pre[i].unpack(f);
+          const int row = full_rows ? e / (32 * NB) : e / d;
+          const int c0 = full_rows ? e % (32 * NB) : e - row * d;
+          const bool ok = e < nvalid;
+#pragma unroll
+          for (int u = 0; u < VEC; u += 4)
+            *reinterpret_cast<float4*>(&x_s[row * LDX + c0 + u]) =
+                make_float4(ok ? f[u] : 0.0f, ok ? f[u + 1] : 0.0f, ok ? f[u + 2] : 0.0f, ok ? f[u + 3] : 0.0f);
+        }
+      }
+    }
+    pf_wave_sync();
+    if (t0 + 32 * NW < r1) issue(t0 + 32 * NW);
+
+    floatx16 c;
+    float old[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      // unconditional (clamped) load, masked below
+      const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
+      old[v] = Ah[rr * r + min(col, r - 1)];
+    }
+    if (apply) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) c[v] = 0.0f;
+      // operands of group g4 + 1 are fetched from LDS while the MFMAs of group g4 run
+      auto lds4 = [&](const float* base, int g4) {
+        return *reinterpret_cast<const float4*>(&base[col * LDX + half * KH + 4 * g4]);
+      };
+      float4 xa = lds4(x_s, 0);
+      float4 mb;
+      if constexpr (MT_LDS) mb = lds4(mt_s, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, MT_LDS ? 2 : 1, 0);  // the first reads have their own slot
+#pragma unroll
+      for (int g4 = 0; g4 < KH / 4; ++g4) {
+        float4 xn = xa, mn = mb;
+        if (g4 + 1 < KH / 4) {
+          xn = lds4(x_s, g4 + 1);
+          if constexpr (MT_LDS) mn = lds4(mt_s, g4 + 1);
+        }
+        if constexpr (!MT_LDS)
+          mb = make_float4(mt[(4 * g4) % (MT_LDS ? 1 : KH)], mt[(4 * g4 + 1) % (MT_LDS ? 1 : KH)],
+                           mt[(4 * g4 + 2) % (MT_LDS ? 1 : KH)], mt[(4 * g4 + 3) % (MT_LDS ? 1 : KH)]);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, mb.x, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, mb.y, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, mb.z, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, mb.w, c, 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, MT_LDS ? 2 : 1, 0);  // DS reads of the next group
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);               // then this group's MFMAs
+        xa = xn;
+        if constexpr (MT_LDS) mb = mn;
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = pf_mfma_row(lane, v);
+        if (row < rows && col < r) {
+          const float df = old[v] - c[v];
+          dsum = fmaf(df, df, dsum);
+          Ah[(t0 + row) * r + col] = c[v];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) c[v] = (pf_mfma_row(lane, v) < rows && col < r) ? old[v] : 0.0f;
+    }
+    auto ldsb = [&](int v, float (&xb)[NB]) {
+      const int row = pf_mfma_row(lane, v);
+      if constexpr (NB == 1) {
+        xb[0] = x_s[row * LDX + col];
+      } else if constexpr (NB == 2) {
+        const float2 t = *reinterpret_cast<const float2*>(&x_s[row * LDX + col * 2]);
+        xb[0] = t.x; xb[1] = t.y;
+      } else {
+#pragma unroll
+        for (int q = 0; q < NB / 4; ++q) {
+          const float4 t = *reinterpret_cast<const float4*>(&x_s[row * LDX + col * NB + 4 * q]);
+          xb[4 * q] = t.x; xb[4 * q + 1] = t.y; xb[4 * q + 2] = t.z; xb[4 * q + 3] = t.w;
+        }
+      }
+    };
+    float xb[NB];
+    ldsb(0, xb);
+    __builtin_amdgcn_sched_group_barrier(0x100, NB == 8 ? 2 : 1, 0);  // the first read has its own slot
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      float xn[NB];
+      if (v + 1 < 16) ldsb(v + 1, xn);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x2f32(c[v], c[v], gAA, 0, 0, 0);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) gAX[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c[v], xb[nb], gAX[nb], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, NB == 8 ? 2 : 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, NB + 1, 0);
+      if (v + 1 < 16) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xb[nb] = xn[nb];
+      }
+    }
+    pf_wave_sync();  // this wave's reads of the tile precede its next staging writes
+  }
+  __syncthreads();  // every wave is done with its tile (and with Mt): the LDS is reused below
+
+  // reduce the waves' tiles through LDS, one 32 x 32 block at a time
+  const int ne = r * (r + d);
+  float* out = part + ((int64_t)h * S + s) * ne;
+  for (int blk = 0; blk <= NB; ++blk) {
+    float* mine = sm + wave * 1024;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      float val = gAA[v];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        if (blk == nb + 1) val = gAX[nb][v];
+      mine[pf_mfma_row(lane, v) * 32 + col] = val;
+    }
+    __syncthreads();
+    for (int e = tid; e < 1024; e += NT) {
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v += sm[w * 1024 + e];
+      const int m = e >> 5, n = e & 31;
+      if (blk == 0) {
+        if (m < r && n < r) out[m * (r + d) + n] = v;
+      } else {
+        const int cx = n * NB + (blk - 1);
+        if (m < r && cx < d) out[m * (r + d) + r + cx] = v;
+      }
+    }
+    __syncthreads();
+  }
+  if (apply) {
+    dsum = wave_sum(dsum);
+    if (lane == 0) red[wave] = dsum;
+    __syncthreads();
+    if (tid == 0) {
+      float t = 0.0f;
+      for (int w = 0; w < NW; ++w) t += red[w];
+      delta_part[(int64_t)h * S + s] = t;
+    }
+  }
+}
+
+// ---- small per-head systems, r <= 32: every thread keeps one column of the augmented matrix
+// [G (32 x 32, identity beyond r) | RHS (32 x d)] in registers; per pivot the pivot column is
+// broadcast through LDS.  No pivoting: G is a Gram matrix (plus B B^T), positive definite.
+struct PfSmallShared {
+  __align__(16) float cbuf[2][32];
+};
+
+// col[i], i < 32: this thread's column.  On return the RHS columns hold G^-1 RHS.
+__device__ __forceinline__ void pf_solve32(float (&colv)[32], PfSmallShared& sh) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int p = 0; p < 32; ++p) {
+    float4* cb4 = reinterpret_cast<float4*>(sh.cbuf[p & 1]);
+    if (tid == p) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) cb4[i] = make_float4(colv[4 * i], colv[4 * i + 1], colv[4 * i + 2], colv[4 * i + 3]);
+    }
+    __syncthreads();
+    float cb[32];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float4 t = cb4[i];
+      cb[4 * i] = t.x; cb[4 * i + 1] = t.y; cb[4 * i + 2] = t.z; cb[4 * i + 3] = t.w;
+    }
+    const float inv = 1.0f / cb[p];
+    const float mp = colv[p] * inv;
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+      if (i != p) colv[i] = fmaf(-cb[i], mp, colv[i]);
+    colv[p] = mp;
+  }
+  __syncthreads();
+}
+
+// sum of the S partial [r][r+d] blocks; 16 elements x 8 partials of loads in flight per thread
+__device__ __forceinline__ void pf_reduce_part(const float* __restrict__ part, int S, int ne, float* dst) {
+  constexpr int EB = 16;
+  for (int e0 = threadIdx.x; e0 < ne; e0 += EB * kPfSmallThreads) {
+    float v[EB];
+#pragma unroll
+    for (int q = 0; q < EB; ++q) v[q] = 0.0f;
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      float x[EB][8];
+#pragma unroll
+      for (int q = 0; q < EB; ++q)
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          x[q][u] = part[(int64_t)min(s0 + u, S - 1) * ne + min(e0 + q * kPfSmallThreads, ne - 1)];
+#pragma unroll
+      for (int q = 0; q < EB; ++q)
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < S) v[q] += x[q][u];
+    }
+#pragma unroll
+    for (int q = 0; q < EB; ++q)
+      if (e0 + q * kPfSmallThreads < ne) dst[e0 + q * kPfSmallThreads] = v[q];
+  }
+}
+
+// Column `tid` of [G | RHS] from a packed [r][r+d] block G0 (+ optional additions), identity-padded.
+__device__ __forceinline__ void pf_load_col(const float* G0, int r, int d, float (&colv)[32]) {
+  const int j = threadIdx.x;  // < 32: system column, else RHS column j - 32
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    float v = 0.0f;
+    if (j < 32) {
+      if (i < r && j < r) v = G0[i * (r + d) + j];
+      else if (i == j) v = 1.0f;
+    } else if (j - 32 < d && i < r) {
+      v = G0[i * (r + d) + r + (j - 32)];
+    }
+    colv[i] = v;
+  }
+}
+
+// G0[i][c] (packed [r][r+d]) <- G[i][c] + (c < r ? (B B^T)[i][c] : B[i][c-r]),  B in LDS [r][d+4], d % 4 == 0
+__device__ __forceinline__ void pf_add_bbt(const float* G, const float* Bs, int r, int d, float* G0) {
+  const int ldb = d + 4;
+  // right-hand side block
+  for (int e = threadIdx.x; e < r * d; e += kPfSmallThreads) {
+    const int i = e / d, c = e - i * d;
+    G0[i * (r + d) + r + c] = G[i * (r + d) + r + c] + Bs[i * ldb + c];
+  }
+  // Gram block: lanes run over c (16-byte reads, conflict-free at this row stride), i is wave-uniform
+  for (int o = threadIdx.x; o < 32 * r; o += kPfSmallThreads) {
+    const int i = o >> 5, c = o & 31;
+    if (c < r) {
+      const float4* bi = reinterpret_cast<const float4*>(Bs + i * ldb);
+      const float4* bc = reinterpret_cast<const float4*>(Bs + c * ldb);
+      float g0 = 0.0f, g1 = 0.0f;
+      for (int x = 0; x < d / 4; ++x) {
+        const float4 a = bi[x], b = bc[x];
+        g0 = fmaf(a.x, b.x, g0); g1 = fmaf(a.y, b.y, g1);
+        g0 = fmaf(a.z, b.z, g0); g1 = fmaf(a.w, b.w, g1);
+      }
+      G0[i * (r + d) + c] = G[i * (r + d) + c] + (g0 + g1);
+    }
+  }
+}
+
+// stage 0: (stopping test) B_Q, B_K from the current Grams, then Mt for the A_Q update
+// stage 1: Mt for the A_K update from the new A_Q Grams
+// stage 2: final B_Q, B_K
+__global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, int it, const float* __restrict__ partQ,
+                                                                     const float* __restrict__ partK, int S, int bh,
+                                                                     int r, int d, int64_t l, float tol,
+                                                                     const float* __restrict__ delta_all,
+                                                                     int* __restrict__ flags, float* __restrict__ Mt,
+                                                                     float* __restrict__ b_q, float* __restrict__ b_k) {
+  extern __shared__ __align__(16) float sm[];
+  const int ne = r * (r + d);
+  float* G1 = sm;            // [r][r+d] packed
+  float* G2 = G1 + ne;       // [r][r+d] packed
+  float* G0 = G2 + ne;       // [r][r+d] packed, system being solved
+  float* Bs = sm + ((3 * ne + 3) & ~3);  // [r][d+4], 16-byte aligned
+  __shared__ PfSmallShared sh;
+  __shared__ int s_done;
+  __shared__ float s_red[kPfSmallThreads / kWave][2];
+  const int tid = threadIdx.x;
+  const int h = blockIdx.x;
+  float colv[32];
+
+  if (stage == 0) {
+    int done = 0;
+    if (it > 0) {
+      done = flags[it - 1];
+      if (!done) {
+        const float* dq = delta_all + ((int64_t)(it - 1) * 2 + 0) * bh * S;
+        const float* dk = delta_all + ((int64_t)(it - 1) * 2 + 1) * bh * S;
+        float sq = 0.0f, sk = 0.0f;
+        for (int i = tid; i < bh * S; i += kPfSmallThreads) {
+          sq += dq[i];
+          sk += dk[i];
+        }
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        if (lane_id() == 0) {
+          s_red[wave_id()][0] = sq;
+          s_red[wave_id()][1] = sk;
+        }
+        __syncthreads();
+        if (tid == 0) {
+          float tq = 0.0f, tk = 0.0f;
+          for (int w = 0; w < kPfSmallThreads / kWave; ++w) {
+            tq += s_red[w][0];
+            tk += s_red[w][1];
+          }
+          const float n = (float)bh * (float)l * (float)r;
+          s_done = fmaxf(tq / n, tk / n) < tol;
+        }
+        __syncthreads();
+        done = s_done;
+      }
+    }
+    // every head computes the same decision from data that no launch of this iteration overwrites
+    if (h == 0 && tid == 0) flags[it] = done;
+    if (done) return;
+  } else if (stage == 1) {
+    if (flags[it]) return;
+  }
+
+  const float* pq = partQ + (int64_t)h * S * ne;
+  const float* pk = partK + (int64_t)h * S * ne;
+  if (stage == 0 || stage == 2) {
+    pf_reduce_part(pq, S, ne, G1);
+    pf_reduce_part(pk, S, ne, G2);
+    __syncthreads();
+    // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q
+    pf_load_col(G1, r, d, colv);
+    pf_solve32(colv, sh);
+    if (tid >= 32 && tid - 32 < d) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        if (i < r) {
+          Bs[i * (d + 4) + tid - 32] = colv[i];
+          b_q[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
+        }
+    }
+    // B_K
+    pf_load_col(G2, r, d, colv);
+    pf_solve32(colv, sh);
+    if (tid >= 32 && tid - 32 < d) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        if (i < r) b_k[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
+    }
+    if (stage == 2) return;
+    __syncthreads();
+    // Mt_Q = (A_K^T A_K + B_Q B_Q^T)^-1 (A_K^T K + B_Q)
+    pf_add_bbt(G2, Bs, r, d, G0);
+  } else {
+    // stage 1: Mt_K = (A_Q^T A_Q + B_K B_K^T)^-1 (A_Q^T Q + B_K)
+    pf_reduce_part(pq, S, ne, G1);
+    for (int e = tid; e < r * d; e += kPfSmallThreads) Bs[(e / d) * (d + 4) + e % d] = b_k[(int64_t)h * r * d + e];
+    __syncthreads();
+    pf_add_bbt(G1, Bs, r, d, G0);
+  }
+  __syncthreads();
+  pf_load_col(G0, r, d, colv);
+  pf_solve32(colv, sh);
+  if (tid >= 32 && tid - 32 < d) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+      if (i < r) Mt[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
+  }
+}
+
+template <typename T>
+using PfPassFn = void (*)(const T*, int, int, int64_t, int, int, const float*, float*, float*, float*, const int*, int);
+
 template <typename T>
 static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q, float* a_k, float* b_q, float* b_k,
                         int b, int hq, int hkv, int64_t l, int r, int d, int max_iter, float tol, hipStream_t st) {
+  constexpr int VEC = Vec16<T>::N;
   const int bh = b * hq;
   const int ne = r * (r + d);
-  LRQK_REQUIRE(ne <= kPfThreads * kPfMaxPer, LRQK_ELIMIT, "r*(r+d)=%d exceeds %d", ne, kPfThreads * kPfMaxPer);
-  int S = (int)std::min<int64_t>(64, (l + 255) / 256);
-  if (S < 1) S = 1;
+  const bool mfma = r <= 32 && d % VEC == 0 && d <= 256 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)k % 16 == 0);
+  const bool small32 = r <= 32 && d <= kPfSmallThreads - 32 && d % 4 == 0;
+  LRQK_REQUIRE(mfma || ne <= kPfThreads * kPfMaxPer, LRQK_ELIMIT, "r*(r+d)=%d exceeds %d", ne, kPfThreads * kPfMaxPer);
+  // splits of the long axis: about one workgroup per CU (a pass keeps one wave per SIMD busy), but
+  // at least 128 rows per split
+  int S = std::max(1, std::min(64, 256 / bh));
+  S = (int)std::max<int64_t>(1, std::min<int64_t>(S, (l + 127) / 128));
   const int iters = max_iter > 0 ? max_iter : 0;
   // workspace: partQ, partK, Mt, deltas[iters][2][bh][S], flags[iters+1]
   const size_t n_part = (size_t)bh * S * ne;
@@ -272,37 +745,47 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   int* flags = (int*)(deltas + n_delta);
   LRQK_HIP_CHECK(hipMemsetAsync(flags, 0, (size_t)(iters + 1) * sizeof(int), st));
 
-  const size_t smem_pass = ((size_t)kPfTile * (d + 1) + (size_t)kPfTile * (r + 1) + (size_t)r * (d + 1)) * sizeof(float);
-  const size_t smem_small = ((size_t)2 * ne + (size_t)r * (r + d + 1) + (size_t)r * (d + 1)) * sizeof(float);
-  if (smem_pass > 48 * 1024)
-    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)pf_pass_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem_pass));
-  if (smem_small > 48 * 1024)
-    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)pf_small_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem_small));
+  PfPassFn<T> pass = pf_pass_generic_kernel<T>;
+  size_t smem_pass = ((size_t)kPfTile * (d + 1) + (size_t)kPfTile * (r + 1) + (size_t)r * (d + 1)) * sizeof(float);
+  int pass_threads = kPfThreads;
+  if (mfma) {
+    const int nb = d <= 32 ? 1 : d <= 64 ? 2 : d <= 128 ? 4 : 8;
+    pass = nb == 1 ? pf_pass_mfma_kernel<T, 1, 8, true> : nb == 2 ? pf_pass_mfma_kernel<T, 2, 8, true>
+         : nb == 4 ? pf_pass_mfma_kernel<T, 4, 8, true> : pf_pass_mfma_kernel<T, 8, 4, false>;
+    const int nw = nb == 8 ? 4 : 8;
+    pass_threads = nw * kWave;
+    smem_pass = std::max((size_t)(nw + (nb == 8 ? 0 : 1)) * 32 * (32 * nb + 4), (size_t)nw * 1024) * sizeof(float);
+  }
+  auto small = small32 ? pf_small32_kernel : pf_small_generic_kernel;
+  const size_t smem_small = small32 ? ((size_t)3 * ne + 4 + (size_t)r * (d + 4)) * sizeof(float)
+                                    : ((size_t)2 * ne + (size_t)r * (r + d + 1) + (size_t)r * (d + 1)) * sizeof(float);
   LRQK_REQUIRE(smem_small <= 160 * 1024 && smem_pass <= 160 * 1024, LRQK_ELIMIT, "r=%d d=%d need too much LDS", r, d);
-  const dim3 grid((unsigned)S, (unsigned)bh), blk(kPfThreads);
+  if (smem_pass > 48 * 1024)
+    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)pass, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
+  if (smem_small > 48 * 1024)
+    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)small, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_small));
+  const dim3 grid((unsigned)S, (unsigned)bh), blk((unsigned)pass_threads), sblk(small32 ? kPfSmallThreads : kPfThreads);
   const T* Q = (const T*)q;
   const T* K = (const T*)k;
-  hipLaunchKernelGGL((pf_pass_kernel<T>), grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
+  hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
                      (float*)nullptr, (const int*)nullptr, S);
-  hipLaunchKernelGGL((pf_pass_kernel<T>), grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
+  hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
                      (float*)nullptr, (const int*)nullptr, S);
   LRQK_HIP_CHECK(hipGetLastError());
   for (int it = 0; it < iters; ++it) {
     float* dq = deltas + ((size_t)it * 2 + 0) * bh * S;
     float* dk = deltas + ((size_t)it * 2 + 1) * bh * S;
-    hipLaunchKernelGGL(pf_small_kernel, dim3((unsigned)bh), blk, smem_small, st, 0, it, partQ, partK, S, bh, r, d, l, tol,
+    hipLaunchKernelGGL(small, dim3((unsigned)bh), sblk, smem_small, st, 0, it, partQ, partK, S, bh, r, d, l, tol,
                        deltas, flags, Mt, b_q, b_k);
-    hipLaunchKernelGGL((pf_pass_kernel<T>), grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)Mt, a_q, partQ, dq,
+    hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)Mt, a_q, partQ, dq,
                        (const int*)(flags + it), S);
-    hipLaunchKernelGGL(pf_small_kernel, dim3((unsigned)bh), blk, smem_small, st, 1, it, partQ, partK, S, bh, r, d, l, tol,
+    hipLaunchKernelGGL(small, dim3((unsigned)bh), sblk, smem_small, st, 1, it, partQ, partK, S, bh, r, d, l, tol,
                        deltas, flags, Mt, b_q, b_k);
-    hipLaunchKernelGGL((pf_pass_kernel<T>), grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)Mt, a_k, partK, dk,
+    hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)Mt, a_k, partK, dk,
                        (const int*)(flags + it), S);
     LRQK_HIP_CHECK(hipGetLastError());
   }
-  hipLaunchKernelGGL(pf_small_kernel, dim3((unsigned)bh), blk, smem_small, st, 2, iters, partQ, partK, S, bh, r, d, l, tol,
+  hipLaunchKernelGGL(small, dim3((unsigned)bh), sblk, smem_small, st, 2, iters, partQ, partK, S, bh, r, d, l, tol,
                      deltas, flags, Mt, b_q, b_k);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;

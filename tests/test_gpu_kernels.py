@@ -361,7 +361,9 @@ def test_als_decode_prefix_branch(ops, ws, oracle):
 @pytest.mark.parametrize("dtype,hq,hkv,l,d,r,iters,tol",
                          [(torch.float32, 4, 2, 40, 16, 4, 2, 0.0), (torch.float32, 4, 2, 700, 16, 4, 0, 0.0),
                           (torch.float32, 28, 4, 1024, 128, 16, 1, 1e-2), (torch.bfloat16, 8, 2, 3000, 128, 32, 3, 0.0),
-                          (torch.float32, 2, 1, 333, 8, 3, 6, 1e30), (torch.float32, 2, 1, 333, 8, 3, 6, 5e-2)])
+                          (torch.float32, 2, 1, 333, 8, 3, 6, 1e30), (torch.float32, 2, 1, 333, 8, 3, 6, 5e-2),
+                          (torch.bfloat16, 4, 2, 1500, 64, 8, 2, 0.0), (torch.bfloat16, 2, 2, 777, 256, 32, 2, 0.0),
+                          (torch.bfloat16, 2, 1, 500, 12, 4, 2, 0.0), (torch.float32, 2, 1, 4500, 96, 24, 2, 0.0)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
