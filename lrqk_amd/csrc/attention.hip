@@ -3,65 +3,67 @@
 // partial (max, sum, accumulator) triples.  (A device-scope fence per workgroup, which a
 // single-launch "last arrival combines" scheme needs, costs more than the second launch:
 // the L2 is per XCD.)
+//
+// Inside the decode step the partial pass shares its launch with the miss fetch: the
+// workgroups that copy the missed rows from the host store are bound by the host link,
+// the others meanwhile run the attention over the slots that stay resident; the combine
+// kernel then adds the freshly fetched slots of its head before merging.
 #include <math.h>
 
 #include "common.hpp"
 #include "ctx.hpp"
+#include "rows.hpp"
 
 namespace lrqk {
 
-constexpr int kAttnThreads = 256;
+constexpr int kAttnThreads = 256;          // partial pass
 constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kCombThreads = 1024;         // combine: wide enough to take a head's refetched rows in one pass
+constexpr int kCombWaves = kCombThreads / kWave;
 
-// Partial layout per (head, split): [m, l, acc[d]] fp32.
-// Each K/V row of d elements is read as d*sizeof(T)/16 chunks by `lpr` adjacent lanes, so a
-// wave covers 64/lpr rows per load instruction with fully coalesced 16-byte accesses.
-template <typename T>
-__global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __restrict__ q, const T* __restrict__ K,
-                                                                    const T* __restrict__ V, int n_slots, int n_valid,
-                                                                    int d, int lpr_log2, float scale_log2e,
-                                                                    float* __restrict__ part, int S) {
+// Online-softmax state of one lane group: running max, sum and the accumulator slice.
+template <int VEC>
+struct AttnAcc {
+  float m, l;
+  float acc[VEC];
+  __device__ __forceinline__ void init() {
+    m = -INFINITY;
+    l = 0.0f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+  }
+};
+
+// Items begin..end-1 of a sequence; row_of(i, valid) gives the slot row of item i (always a
+// readable row; `valid` says whether it counts).  Each K/V row of d elements is read as
+// d*sizeof(T)/16 chunks by `lpr` adjacent lanes, so a wave covers 64/lpr rows per load
+// instruction with fully coalesced 16-byte accesses; four row groups per pass have their loads
+// issued together (one memory latency), unconditionally, and are masked afterwards.
+template <typename T, int NW, typename RowOf>
+__device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__ Kh, const T* __restrict__ Vh, int d,
+                                          int lpr_log2, int begin, int end, RowOf row_of,
+                                          AttnAcc<Vec16<T>::N>& st) {
   constexpr int VEC = Vec16<T>::N;
-  __shared__ float red[kAttnWaves][2 + 256];
-  const int h = blockIdx.y, s = blockIdx.x;
   const int lane = lane_id(), wave = wave_id();
   const int lpr = 1 << lpr_log2;
   const int sub = lane & (lpr - 1);
   const int grp = lane >> lpr_log2;
   const int gpw = kWave >> lpr_log2;  // row groups per wave
-  const int rows_per_iter = gpw * kAttnWaves;
-  const int rows_per_split = (n_valid + S - 1) / S;
-  const int r0 = s * rows_per_split;
-  const int r1 = min(n_valid, r0 + rows_per_split);
-
-  float qf[VEC];
-  {
-    Vec16<T> qv;
-    qv.load(q + (int64_t)h * d + sub * VEC);
-    qv.unpack(qf);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) qf[e] *= scale_log2e;
-  }
-  const T* Kh = K + (int64_t)h * n_slots * d;
-  const T* Vh = V + (int64_t)h * n_slots * d;
-
-  float m_run = -INFINITY, l_run = 0.0f;
-  float acc[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
-
-  // four row groups per pass: their K and V loads are issued together (one memory latency)
-  for (int base = r0; base < r1; base += 4 * rows_per_iter) {
+  const int rows_per_iter = gpw * NW;
+  for (int base = begin; base < end; base += 4 * rows_per_iter) {
     Vec16<T> kv[4], vv[4];
+    bool ok[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int rr = min(base + u * rows_per_iter + wave * gpw + grp, r1 - 1);
+      const int i = base + u * rows_per_iter + wave * gpw + grp;
+      bool valid;
+      const int rr = row_of(min(i, end - 1), valid);
+      ok[u] = valid && i < end;
       kv[u].load(Kh + (int64_t)rr * d + sub * VEC);
       vv[u].load(Vh + (int64_t)rr * d + sub * VEC);
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const bool valid = base + u * rows_per_iter + wave * gpw + grp < r1;
       float kf[VEC], vf[VEC];
       kv[u].unpack(kf);
       vv[u].unpack(vf);
@@ -69,99 +71,214 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sc = fmaf(kf[e], qf[e], sc);
       for (int off = 1; off < lpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);
-      if (!valid) sc = -INFINITY;
-      const float m_new = fmaxf(m_run, sc);
+      if (!ok[u]) sc = -INFINITY;
+      const float m_new = fmaxf(st.m, sc);
       // exp2 of (-inf) - (-inf) must not produce NaN: while nothing valid was seen keep zeros
-      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(m_run - m_new);
+      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
       const float p = (m_new == -INFINITY) ? 0.0f : exp2f(sc - m_new);
-      l_run = l_run * alpha + p;
+      st.l = st.l * alpha + p;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc[e] = acc[e] * alpha + p * vf[e];
-      m_run = m_new;
+      for (int e = 0; e < VEC; ++e) st.acc[e] = st.acc[e] * alpha + p * vf[e];
+      st.m = m_new;
     }
-  }
-  // merge the row groups of this wave
-  for (int off = lpr; off < kWave; off <<= 1) {
-    const float m_o = __shfl_xor(m_run, off, kWave);
-    const float l_o = __shfl_xor(l_run, off, kWave);
-    const float m_new = fmaxf(m_run, m_o);
-    const float a = (m_new == -INFINITY) ? 0.0f : exp2f(m_run - m_new);
-    const float b = (m_new == -INFINITY) ? 0.0f : exp2f(m_o - m_new);
-    l_run = l_run * a + l_o * b;
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      const float o = __shfl_xor(acc[e], off, kWave);
-      acc[e] = acc[e] * a + o * b;
-    }
-    m_run = m_new;
-  }
-  if (grp == 0) {
-    if (sub == 0) {
-      red[wave][0] = m_run;
-      red[wave][1] = l_run;
-    }
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) red[wave][2 + sub * VEC + e] = acc[e];
-  }
-  __syncthreads();
-  float* pout = part + ((int64_t)h * S + s) * (d + 2);
-  float M = -INFINITY;
-#pragma unroll
-  for (int w = 0; w < kAttnWaves; ++w) M = fmaxf(M, red[w][0]);
-  for (int c = threadIdx.x; c < d + 2; c += kAttnThreads) {
-    float v = 0.0f;
-    if (c == 0) {
-      v = M;
-    } else {
-#pragma unroll
-      for (int w = 0; w < kAttnWaves; ++w) {
-        const float f = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
-        v += red[w][c] * f;
-      }
-    }
-    pout[c] = v;
   }
 }
 
-// One workgroup per head merges the S partial triples.  d is a power of two <= 256: thread ->
-// (column c, split group tg); every batch of loads is independent, so it costs one latency.
+// Merges the lane groups of a wave, then the waves of the workgroup; afterwards threads c < d + 2
+// hold element c of the workgroup's (m, l, acc[d]) triple in the return value.
+// red: [NW][2 + 256] floats of LDS.
+template <int VEC, int NW>
+__device__ __forceinline__ float attn_block_merge(AttnAcc<VEC>& st, int lpr_log2, int d, float (*red)[2 + 256]) {
+  const int lane = lane_id(), wave = wave_id();
+  const int lpr = 1 << lpr_log2;
+  const int sub = lane & (lpr - 1);
+  const int grp = lane >> lpr_log2;
+  for (int off = lpr; off < kWave; off <<= 1) {
+    const float m_o = __shfl_xor(st.m, off, kWave);
+    const float l_o = __shfl_xor(st.l, off, kWave);
+    const float m_new = fmaxf(st.m, m_o);
+    const float a = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
+    const float b = (m_new == -INFINITY) ? 0.0f : exp2f(m_o - m_new);
+    st.l = st.l * a + l_o * b;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float o = __shfl_xor(st.acc[e], off, kWave);
+      st.acc[e] = st.acc[e] * a + o * b;
+    }
+    st.m = m_new;
+  }
+  if (grp == 0) {
+    if (sub == 0) {
+      red[wave][0] = st.m;
+      red[wave][1] = st.l;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) red[wave][2 + sub * VEC + e] = st.acc[e];
+  }
+  __syncthreads();
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, red[w][0]);
+  float v = 0.0f;
+  const int c = threadIdx.x;
+  if (c == 0) {
+    v = M;
+  } else if (c < d + 2) {
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float f = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
+      v += red[w][c] * f;
+    }
+  }
+  return v;
+}
+
 template <typename T>
-__global__ __launch_bounds__(kAttnThreads) void attn_combine_kernel(const float* __restrict__ part, int S, int d,
-                                                                    T* __restrict__ out) {
-  __shared__ float red[kAttnThreads];
+__device__ __forceinline__ void load_query(const T* q, int h, int d, int lpr_log2, float scale_log2e, float* qf) {
+  constexpr int VEC = Vec16<T>::N;
+  const int sub = lane_id() & ((1 << lpr_log2) - 1);
+  Vec16<T> qv;
+  qv.load(q + (int64_t)h * d + sub * VEC);
+  qv.unpack(qf);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) qf[e] *= scale_log2e;
+}
+
+// Partial layout per (head, split): [m, l, acc[d]] fp32; `stride_s` triples per head.
+// skip (optional): u8 [bh][k_skip], slots s < k_skip with skip != 0 are left out.
+template <typename T>
+__device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const T* __restrict__ K,
+                                                  const T* __restrict__ V, int n_slots, int n_valid, int d,
+                                                  int lpr_log2, float scale_log2e, float* __restrict__ part, int S,
+                                                  int stride_s, const uint8_t* __restrict__ skip, int k_skip, int h,
+                                                  int s) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ float red[kAttnWaves][2 + 256];
+  const int rows_per_split = (n_valid + S - 1) / S;
+  const int r0 = s * rows_per_split;
+  const int r1 = min(n_valid, r0 + rows_per_split);
+  float qf[VEC];
+  load_query<T>(q, h, d, lpr_log2, scale_log2e, qf);
+  const T* Kh = K + (int64_t)h * n_slots * d;
+  const T* Vh = V + (int64_t)h * n_slots * d;
+  AttnAcc<VEC> st;
+  st.init();
+  if (skip) {
+    const uint8_t* sk = skip + (int64_t)h * k_skip;
+    attn_scan<T, kAttnWaves>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
+      valid = sk[min(i, k_skip - 1)] == 0 || i >= k_skip;
+      return i;
+    }, st);
+  } else {
+    attn_scan<T, kAttnWaves>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
+      valid = true;
+      return i;
+    }, st);
+  }
+  const float v = attn_block_merge<VEC, kAttnWaves>(st, lpr_log2, d, red);
+  if ((int)threadIdx.x < d + 2) part[((int64_t)h * stride_s + s) * (d + 2) + threadIdx.x] = v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __restrict__ q, const T* __restrict__ K,
+                                                                    const T* __restrict__ V, int n_slots, int n_valid,
+                                                                    int d, int lpr_log2, float scale_log2e,
+                                                                    float* __restrict__ part, int S) {
+  attn_partial_body<T>(q, K, V, n_slots, n_valid, d, lpr_log2, scale_log2e, part, S, S, nullptr, 0, blockIdx.y,
+                       blockIdx.x);
+}
+
+// Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their
+// slots; the others run the partial attention over the slots that are not being replaced.
+template <typename T>
+__global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
+    const uint4* __restrict__ store, int64_t cap, int32_t* __restrict__ hit, int64_t hit_stride,
+    const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
+    int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
+    int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S) {
+  const int h = blockIdx.y;
+  if ((int)blockIdx.x < n_fetch) {
+    fetch_rows_body(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k,
+                    h, blockIdx.x, n_fetch);
+    return;
+  }
+  attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + 1, evict, k, h,
+                       (int)blockIdx.x - n_fetch);
+}
+
+// One workgroup per head merges the S partial triples (rows of `stride_s` triples per head).
+// With miss_slots != nullptr it first computes triple number S itself: the attention over
+// the head's refetched slots (their slot list, the partial triples and the rows are all
+// requested up front so that the kernel pays two memory latencies, not one per stage).
+// d is a power of two <= 256: thread -> (column c, split group tg).
+template <typename T>
+__global__ __launch_bounds__(kCombThreads) void attn_combine_kernel(float* __restrict__ part, int S, int stride_s,
+                                                                    int d, T* __restrict__ out,
+                                                                    const T* __restrict__ q, const T* __restrict__ K,
+                                                                    const T* __restrict__ V, int n_slots,
+                                                                    int lpr_log2, float scale_log2e,
+                                                                    const int32_t* __restrict__ miss_slots,
+                                                                    const int32_t* __restrict__ miss_count, int k) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ float red[kCombWaves][2 + 256];
+  __shared__ float ms_s[65], ls_s[65];  // S + 1 <= 65
+  __shared__ float extra[2 + 256];
   const int h = blockIdx.x;
-  const float* p = part + (int64_t)h * S * (d + 2);
-  __shared__ float ms_s[64], ls_s[64];  // S <= 64
-  if (threadIdx.x < 64) {
+  const float* p = part + (int64_t)h * stride_s * (d + 2);
+  const int c = threadIdx.x & (d - 1);
+  const int ntg = kCombThreads / d;
+  const int tg = threadIdx.x / d;
+  // the partial triples of this thread: splits tg, tg + ntg, ... (at most 8 with S <= 64, ntg >= 4... 16)
+  float x[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) x[u] = p[(int64_t)min(tg + u * ntg, S - 1) * (d + 2) + 2 + c];
+  float mv = 0.0f, lv = 0.0f;
+  if (threadIdx.x < 65) {
     const int t = min((int)threadIdx.x, S - 1);
-    const float mv = p[(int64_t)t * (d + 2)], lv = p[(int64_t)t * (d + 2) + 1];
+    mv = p[(int64_t)t * (d + 2)];
+    lv = p[(int64_t)t * (d + 2) + 1];
+  }
+  int n_tr = S;
+  if (miss_slots) {
+    const int cnt = miss_count[h];
+    const int32_t* ms = miss_slots + (int64_t)h * k;
+    float qf[VEC];
+    load_query<T>(q, h, d, lpr_log2, scale_log2e, qf);
+    AttnAcc<VEC> st;
+    st.init();
+    attn_scan<T, kCombWaves>(qf, K + (int64_t)h * n_slots * d, V + (int64_t)h * n_slots * d, d, lpr_log2, 0, cnt,
+                             [&](int i, bool& valid) {
+                               const int slot = ms[max(i, 0)];
+                               valid = slot >= 0 && slot < k;
+                               return valid ? slot : 0;
+                             }, st);
+    const float v = attn_block_merge<VEC, kCombWaves>(st, lpr_log2, d, red);
+    if ((int)threadIdx.x < d + 2) extra[threadIdx.x] = v;
+    n_tr = S + 1;
+  }
+  if (threadIdx.x < 65) {
     ms_s[threadIdx.x] = mv;
     ls_s[threadIdx.x] = lv;
   }
   __syncthreads();
-  float Mh = -INFINITY;
-  for (int t = 0; t < S; ++t) Mh = fmaxf(Mh, ms_s[t]);
-  float L = 0.0f;
-  for (int t = 0; t < S; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
-  // d is a power of two <= 256: thread -> (column c, split group tg)
-  const int c = threadIdx.x & (d - 1);
-  const int ntg = kAttnThreads / d;
-  const int tg = threadIdx.x / d;
-  float v = 0.0f;
-  for (int t0 = tg; t0 < S; t0 += 8 * ntg) {
-    float x[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int t = t0 + u * ntg;
-      x[u] = p[(int64_t)min(t, S - 1) * (d + 2) + 2 + c];  // unconditional (clamped), masked below
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int t = t0 + u * ntg;
-      if (t < S && ms_s[t] != -INFINITY) v = fmaf(x[u], exp2f(ms_s[t] - Mh), v);
-    }
+  if (miss_slots && threadIdx.x == 0) {
+    ms_s[S] = extra[0];
+    ls_s[S] = extra[1];
   }
-  float* comb = red;
+  __syncthreads();
+  float Mh = -INFINITY;
+  for (int t = 0; t < n_tr; ++t) Mh = fmaxf(Mh, ms_s[t]);
+  float L = 0.0f;
+  for (int t = 0; t < n_tr; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
+  float v = 0.0f;
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int t = tg + u * ntg;
+    if (t < S && ms_s[t] != -INFINITY) v = fmaf(x[u], exp2f(ms_s[t] - Mh), v);
+  }
+  if (miss_slots && tg == 0 && ms_s[S] != -INFINITY) v = fmaf(extra[2 + c], exp2f(ms_s[S] - Mh), v);
+  float* comb = &red[0][0];
+  __syncthreads();
   comb[threadIdx.x] = v;
   __syncthreads();
   if (tg == 0) {
@@ -171,29 +288,84 @@ __global__ __launch_bounds__(kAttnThreads) void attn_combine_kernel(const float*
   }
 }
 
+static int attn_shape(int d, int vec, int* lpr_log2) {
+  const int lpr = d / vec;
+  int lg = 0;
+  while ((1 << lg) < lpr) ++lg;
+  LRQK_REQUIRE(d % vec == 0 && (1 << lg) == lpr && lpr <= kWave && d <= 256, LRQK_ELIMIT,
+               "head_dim %d unsupported (need a power-of-two number of 16-byte chunks, <= 256 elements)", d);
+  *lpr_log2 = lg;
+  return LRQK_OK;
+}
+
 template <typename T>
 static int attention_impl(lrqk_ctx* ctx, const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
                           void* out, int bh, int d, hipStream_t st) {
-  constexpr int VEC = Vec16<T>::N;
-  const int lpr = d / VEC;
   int lpr_log2 = 0;
-  while ((1 << lpr_log2) < lpr) ++lpr_log2;
-  LRQK_REQUIRE(d % VEC == 0 && (1 << lpr_log2) == lpr && lpr <= kWave && d <= 256, LRQK_ELIMIT,
-               "head_dim %d unsupported (need a power-of-two number of 16-byte chunks, <= 256 elements)", d);
+  int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
+  if (rc) return rc;
   int S = (n_valid + 63) / 64;
   if (S < 1) S = 1;
   if (S > 64) S = 64;
-  int rc = ctx->attn_part.ensure((size_t)bh * S * (d + 2) * sizeof(float));
-  if (rc) return rc;
+  if ((rc = ctx->attn_part.ensure((size_t)bh * (S + 1) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   hipLaunchKernelGGL((attn_partial_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kAttnThreads), 0, st,
                      (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, n_valid, d, lpr_log2, scale_log2e,
                      (float*)ctx->attn_part.p, S);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kAttnThreads), 0, st,
-                     (const float*)ctx->attn_part.p, S, d, (T*)out);
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (float*)ctx->attn_part.p,
+                     S, S, d, (T*)out, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr, 0, 0, 0.0f,
+                     (const int32_t*)nullptr, (const int32_t*)nullptr, 0);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
+}
+
+template <typename T>
+static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t cap, void* k_act, void* v_act,
+                                int n_slots, int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
+                                const int32_t* miss_count, const uint8_t* evict, int b, int hq, int hkv, int d, int k,
+                                const void* q, void* out, hipStream_t st) {
+  const int bh = b * hq;
+  int lpr_log2 = 0;
+  int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
+  if (rc) return rc;
+  const int cpr = d * (int)sizeof(T) / 16;
+  LRQK_REQUIRE(2 * cpr <= kAttnThreads, LRQK_ELIMIT, "row of %d bytes too long", 2 * cpr * 16);
+  int S = (n_slots + 63) / 64;
+  if (S > 64) S = 64;
+  const int rpb = kAttnThreads / (2 * cpr);
+  const int n_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));  // sized for a miss rate of 1/8
+  if ((rc = ctx->attn_part.ensure((size_t)bh * (S + 1) * (d + 2) * sizeof(float)))) return rc;
+  const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
+  hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S), (unsigned)bh), dim3(kAttnThreads), 0,
+                     st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count, evict, hq, hkv, cpr, k,
+                     n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2, scale_log2e,
+                     (float*)ctx->attn_part.p, S);
+  LRQK_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (float*)ctx->attn_part.p,
+                     S, S + 1, d, (T*)out, (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, lpr_log2,
+                     scale_log2e, miss_slots, miss_count, k);
+  LRQK_HIP_CHECK(hipGetLastError());
+  return LRQK_OK;
+}
+
+// Miss fetch overlapped with the attention over the slots that stay resident, then the
+// refetched slots and the merge.  Same result as lrqk_fetch_rows followed by lrqk_attention.
+int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
+                    int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
+                    const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
+                    hipStream_t st) {
+  const void* dev_store = nullptr;
+  int rc = resolve_store(kv_store, &dev_store);
+  if (rc) return rc;
+  LRQK_REQUIRE(((uintptr_t)dev_store % 16 == 0) && ((uintptr_t)q % 16 == 0) && ((uintptr_t)k_act % 16 == 0) &&
+                   ((uintptr_t)v_act % 16 == 0),
+               LRQK_EINVAL, "pointers must be 16-byte aligned");
+  if (dtype == LRQK_F32)
+    return fetch_attention_impl<float>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
+                                       miss_count, evict, b, hq, hkv, d, k, q, out, st);
+  return fetch_attention_impl<bf16_t>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
+                                      miss_count, evict, b, hq, hkv, d, k, q, out, st);
 }
 
 }  // namespace lrqk

@@ -66,4 +66,10 @@ namespace lrqk {
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st);
+// Miss fetch overlapped with the attention over the slots that stay resident (one launch), then
+// the attention over the refetched slots and the merge (second launch).
+int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
+                    int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
+                    const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
+                    hipStream_t st);
 }  // namespace lrqk

@@ -1,7 +1,10 @@
 // Hit/miss diff against the GPU-resident active set, miss fetch from the [K|V] store,
 // on-device row gather, ring append and ring flush.
+#include <algorithm>
+
 #include "common.hpp"
 #include "ctx.hpp"
+#include "rows.hpp"
 
 namespace lrqk {
 
@@ -95,31 +98,14 @@ __global__ __launch_bounds__(256) void replace_all_kernel(const int32_t* __restr
 // --------------------------------------------------------------------------- row movers
 // Rows are copied as 16-byte chunks; `cpr` chunks per K (or V) row.
 
-// Missed rows: store row (b, h/groups, token) = [K row | V row] -> active-set slot rows.
 __global__ __launch_bounds__(256) void fetch_rows_kernel(const uint4* __restrict__ store, int64_t cap,
                                                          uint4* __restrict__ k_act, uint4* __restrict__ v_act,
                                                          int n_slots, const int32_t* __restrict__ hit,
                                                          int64_t hit_stride, const int32_t* __restrict__ miss_slots,
                                                          const int32_t* __restrict__ miss_count, int hq, int hkv,
-                                                         int cpr, int k, int rows_per_block) {
-  const int h = blockIdx.y;  // flattened (b, head)
-  const int cnt = miss_count[h];
-  const int j0 = blockIdx.x * rows_per_block;
-  if (j0 >= cnt) return;
-  const int b = h / hq, head = h % hq;
-  const int kvh = head / (hq / hkv);
-  const int chunks = 2 * cpr;  // per store row
-  for (int w = threadIdx.x; w < rows_per_block * chunks; w += blockDim.x) {
-    const int j = j0 + w / chunks;
-    const int c = w % chunks;
-    if (j >= cnt) break;
-    const int slot = miss_slots[(int64_t)h * k + j];
-    const int32_t tok = hit[(int64_t)h * hit_stride + slot];
-    if (slot < 0 || slot >= k || tok < 0 || tok >= cap) continue;
-    const uint4 val = store[(((int64_t)b * hkv + kvh) * cap + tok) * chunks + c];
-    const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
-    if (c < cpr) k_act[dst + c] = val; else v_act[dst + (c - cpr)] = val;
-  }
+                                                         int cpr, int k) {
+  fetch_rows_body(store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k,
+                  blockIdx.y, blockIdx.x, gridDim.x);
 }
 
 // dst[bh][j][:] = src[b][h/groups][idx[bh][j]][:]
@@ -184,6 +170,20 @@ static int check_rows(int b, int hq, int hkv, int d, int dtype, int* cpr) {
 
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
+int resolve_store(const void* kv_store, const void** dev_store) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, kv_store) != hipSuccess) {
+    (void)hipGetLastError();
+    return set_error(LRQK_EINVAL, "kv_store is neither device memory nor pinned host memory");
+  }
+  *dev_store = kv_store;
+  if (attr.type == hipMemoryTypeHost) {
+    LRQK_REQUIRE(attr.devicePointer != nullptr, LRQK_EINVAL, "host store is not mapped into the device");
+    *dev_store = attr.devicePointer;
+  }
+  return LRQK_OK;
+}
+
 }  // namespace lrqk
 
 using namespace lrqk;
@@ -227,23 +227,14 @@ extern "C" int lrqk_fetch_rows(const void* kv_store, int64_t cap, void* k_act, v
   if (rc) return rc;
   LRQK_REQUIRE(kv_store && k_act && v_act && hit && miss_slots && miss_count, LRQK_EINVAL, "null pointer");
   LRQK_REQUIRE(k > 0 && k <= n_slots && hit_stride >= k && cap > 0, LRQK_EINVAL, "bad sizes k=%d n_slots=%d", k, n_slots);
-  const void* dev_store = kv_store;
-  hipPointerAttribute_t attr;
-  if (hipPointerGetAttributes(&attr, kv_store) == hipSuccess) {
-    if (attr.type == hipMemoryTypeHost) {
-      LRQK_REQUIRE(attr.devicePointer != nullptr, LRQK_EINVAL, "host store is not mapped into the device");
-      dev_store = attr.devicePointer;
-    }
-  } else {
-    (void)hipGetLastError();
-    return set_error(LRQK_EINVAL, "kv_store is neither device memory nor pinned host memory");
-  }
+  const void* dev_store = nullptr;
+  if ((rc = resolve_store(kv_store, &dev_store))) return rc;
   LRQK_REQUIRE(aligned16(dev_store) && aligned16(k_act) && aligned16(v_act), LRQK_EINVAL, "pointers must be 16-byte aligned");
-  const int rows_per_block = 8;
-  dim3 grid((unsigned)((k + rows_per_block - 1) / rows_per_block), (unsigned)(b * hq));
+  LRQK_REQUIRE(2 * cpr <= 256, LRQK_ELIMIT, "row of %d bytes too long", 2 * cpr * 16);
+  const int rpb = 256 / (2 * cpr);
+  dim3 grid((unsigned)std::min(256, (k + rpb - 1) / rpb), (unsigned)(b * hq));
   hipLaunchKernelGGL(fetch_rows_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint4*)dev_store, cap,
-                     (uint4*)k_act, (uint4*)v_act, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k,
-                     rows_per_block);
+                     (uint4*)k_act, (uint4*)v_act, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
