@@ -31,7 +31,6 @@ constexpr int kGramWaves = kGramThreads / kWave;
 constexpr int kGramChunk = 32;  // tokens per wave per chunk = 16 MFMA steps
 constexpr int kGramNe = 32 * 32 + 32;
 constexpr int kSolveThreads = 256;
-constexpr int kSolveWaves = kSolveThreads / kWave;
 constexpr int kFinThreads = 256;
 
 // C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
@@ -148,65 +147,69 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
 constexpr int kLdm = 65;  // row stride of an augmented [G | I] matrix (64 columns)
 constexpr int kLdi = 33;  // row stride of an inverse
 
-// Gauss-Jordan inversion of two SPD 32 x 32 matrices side by side in LDS, no pivoting, 256
-// threads.  Mx: two augmented matrices [G | I] (row stride kLdm), the second at 32*kLdm.  In
-// step p only columns p+1 .. p+32 of a row change (the identity half is lower triangular so
-// far), so a thread owns one column offset and 8 rows.  On return
-// inv{0,1}[i][c] = Mx[i][32+c] / Mx[i][i].
-__device__ __forceinline__ void invert_pair_lds(float* Mx, float* inv0, float* inv1) {
+// Gauss-Jordan inversion of two SPD 32 x 32 matrices at once, no pivoting.  Threads 0..127:
+// thread (mat, j) keeps column j of the augmented matrix [G | I] of matrix `mat` in registers
+// (colv, rows 0..31); per pivot the pivot column is broadcast through LDS (cbuf: [2][2][32]
+// floats, 16-byte aligned) and the pivot row is normalised, so on return the identity half
+// holds the inverse: inv{0,1}[i][c] = colv[i] of thread (mat, 32 + c).  Every thread of the
+// workgroup must call it (one barrier per pivot).
+__device__ __forceinline__ void invert_pair_regs(float (&colv)[32], float* cbuf, float* inv0, float* inv1) {
   const int tid = threadIdx.x;
-  const int cw = tid & 31;
-  const int mat = (tid >> 5) & 1;
-  const int rc = tid >> 6;  // row class 0..3: rows rc + 4u
-  float* M = Mx + mat * 32 * kLdm;
-  for (int p = 0; p < 32; ++p) {
-    const float invp = 1.0f / M[p * kLdm + p];
-    const int c = p + 1 + cw;
-    const float mpc = M[p * kLdm + c];
-    float mip[8], mic[8];
+  const int mat = (tid >> 6) & 1, j = tid & 63;
+  const bool act = tid < 128;
+  // The rows are rotated by one after every pivot, so the pivot is always element 0 and the
+  // loop body is the same code for every p (a rolled loop: straight-line code for 32 pivots
+  // would be executed once per workgroup from a cold instruction cache).
+  // Each matrix belongs to one wave (64 columns), so the exchange needs no workgroup barrier.
+  // Four pivots per trip with static register indices, then one rotation by four rows.
+  if (act) {
+#pragma unroll 1
+    for (int p0 = 0; p0 < 32; p0 += 4) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      mip[u] = M[(rc + 4 * u) * kLdm + p];
-      mic[u] = M[(rc + 4 * u) * kLdm + c];
-    }
+      for (int q = 0; q < 4; ++q) {
+        // the pivot column lives in lane p0 + q of this wave: broadcast it lane -> scalar registers
+        float cb[32];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      if (rc + 4 * u != p) M[(rc + 4 * u) * kLdm + c] = fmaf(-(mip[u] * invp), mpc, mic[u]);
+        for (int i = 0; i < 32; ++i)
+          cb[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(colv[i]), p0 + q));
+        // reciprocal of the pivot: hardware estimate + one Newton step (error below 1 ulp)
+        float rc = __builtin_amdgcn_rcpf(cb[q]);
+        rc = fmaf(fmaf(-cb[q], rc, 1.0f), rc, rc);
+        const float mp = colv[q] * rc;
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+          if (i != q) colv[i] = fmaf(-cb[i], mp, colv[i]);
+        colv[q] = mp;
+      }
+      float t0 = colv[0], t1 = colv[1], t2 = colv[2], t3 = colv[3];
+#pragma unroll
+      for (int i = 0; i < 28; ++i) colv[i] = colv[i + 4];
+      colv[28] = t0; colv[29] = t1; colv[30] = t2; colv[31] = t3;
     }
-    __syncthreads();
   }
-  float* inv = mat ? inv1 : inv0;
+  if (act && j >= 32) {
+    float* inv = mat ? inv1 : inv0;
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
-    const int i = rc + 4 * u;
-    inv[i * kLdi + cw] = M[i * kLdm + 32 + cw] / M[i * kLdm + i];
+    for (int i = 0; i < 32; ++i) inv[i * kLdi + (j - 32)] = colv[i];
   }
   __syncthreads();
 }
 
-// out[j] = sum_i v[i] * Minv[i][j], 32 terms
-__device__ __forceinline__ float row_times32(const float* v, const float* Minv, int j) {
-  float s0 = 0.0f, s1 = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 32; i += 2) {
-    s0 = fmaf(v[i], Minv[i * kLdi + j], s0);
-    s1 = fmaf(v[i + 1], Minv[(i + 1) * kLdi + j], s1);
-  }
-  return s0 + s1;
+// Sum of x over lanes 0..31 of the wave with data-parallel-primitive moves (no LDS round trips):
+// butterflies inside each row of 16 lanes, then lane 15 of row 0 is added into row 1; the total
+// is read from lane 31.  Every lane of the wave must call it.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
+  return v + __int_as_float(t);
 }
-
-// x = b (G + v^T v)^-1 from G^-1 (Sherman-Morrison): x = y - (y.v / (1 + z.v)) z with
-// y = b G^-1, z = v G^-1.  Executed by the first wave; b, v, x are LDS vectors of 32.
-__device__ __forceinline__ void rank1_solve_wave(const float* b, const float* v, const float* Ginv, float* x) {
-  const int j = threadIdx.x & 31;  // caller guarantees threadIdx.x < 64; both halves compute the same
-  const float y = row_times32(b, Ginv, j);
-  const float z = row_times32(v, Ginv, j);
-  float yv = (threadIdx.x < 32) ? y * v[j] : 0.0f;
-  float zv = (threadIdx.x < 32) ? z * v[j] : 0.0f;
-  yv = wave_sum(yv);
-  zv = wave_sum(zv);
-  const float alpha = yv / (1.0f + zv);
-  if (threadIdx.x < 32) x[j] = fmaf(-alpha, z, y);
+__device__ __forceinline__ float sum_lanes_0_31(float x) {
+  x = dpp_add<0xB1, 0xf>(x);   // quad_perm [1,0,3,2]
+  x = dpp_add<0x4E, 0xf>(x);   // quad_perm [2,3,0,1]
+  x = dpp_add<0x141, 0xf>(x);  // row_half_mirror
+  x = dpp_add<0x140, 0xf>(x);  // row_mirror
+  x = dpp_add<0x142, 0xa>(x);  // row_bcast15 into rows 1 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 31));
 }
 
 // iter_out per head: [max_iter][2r] (q_hat then k_hat of each iteration);
@@ -233,7 +236,7 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
   float* qv = BK + 32 * ld;         // [d]
   float* kv = qv + d;               // [d]
   float* G = kv + d;                // [kGramNe] summed A^T [A | w]
-  float* Mx = G + kGramNe;          // 2 x [32][kLdm]: [G_K | I] then [G_Q | I]
+  float* Mx = G + kGramNe;          // pivot-column exchange buffers of the inversion (16-byte aligned)
   float* GKi = Mx + 2 * 32 * kLdm;  // [32][kLdi]
   float* GQi = GKi + 32 * kLdi;     // [32][kLdi]
   float* rhs_q = GQi + 32 * kLdi;   // 6 vectors of 32
@@ -344,57 +347,74 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
     if (lane == 0) s_qk = v;
   }
   __syncthreads();
-  // [G_K | I], [G_Q | I], identity-padded beyond r
+  // columns of [G_K | I] (threads 0..63) and [G_Q | I] (threads 64..127), identity-padded beyond r
   {
-    float* MK = Mx;
-    float* MQ = Mx + 32 * kLdm;
+    float colv[32];
+    const int mat = (tid >> 6) & 1, j = tid & 63;
+    // all LDS reads first (independent, so they pipeline), then the selects
+    const float* c0 = cred + (mat ? 0 : 2048);
+    const float gsel = mat ? 1.0f : 0.0f;
+    const int jj = j & 31;
+    float a0[32], a1[32], gg[32];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int e = tid + u * kSolveThreads;
-      const int i = e >> 5, j = e & 31;
-      const bool in = i < r && j < r;
-      const float eye = (i == j) ? 1.0f : 0.0f;
-      MQ[i * kLdm + j] = in ? (cred[e] + cred[1024 + e]) + G[e] : eye;
-      MK[i * kLdm + j] = in ? cred[2048 + e] + cred[3072 + e] : eye;
-      MQ[i * kLdm + 32 + j] = eye;
-      MK[i * kLdm + 32 + j] = eye;
+    for (int i = 0; i < 32; ++i) {
+      a0[i] = c0[i * 32 + jj];
+      a1[i] = c0[1024 + i * 32 + jj];
+      gg[i] = G[i * 32 + jj];
     }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const float g = fmaf(gsel, gg[i], a0[i] + a1[i]);
+      const float eye = (i == jj) ? 1.0f : 0.0f;
+      colv[i] = j < 32 ? ((i < r && j < r) ? g : eye) : eye;
+    }
+    (void)gsum;
+    invert_pair_regs(colv, Mx, GKi, GQi);
   }
-  (void)gsum;
-  __syncthreads();
-  invert_pair_lds(Mx, GKi, GQi);
-  // k_hat_0 = kB G_K^-1
-  if (tid < 32) hat_k[tid] = row_times32(kB, GKi, tid);
-  __syncthreads();
-  for (int it = 0; it < max_iter; ++it) {
-    // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
-    if (tid < 32) tmp[tid] = fmaf(s_qk, hat_k[tid], rhs_q[tid]);
-    __syncthreads();
-    if (tid < kWave) rank1_solve_wave(tmp, hat_k, GQi, hat_q);
-    __syncthreads();
-    // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat
-    if (tid < 32) tmp[tid] = fmaf(s_qk, hat_q[tid], kB[tid]);
-    __syncthreads();
-    if (tid < kWave) {
-      rank1_solve_wave(tmp, hat_q, GKi, new_k);
-      float dsq = 0.0f;
-      if (tid < r) {
-        const float df = hat_k[tid] - new_k[tid];  // each lane reads back only what it wrote
-        dsq = df * df;
-      }
-      dsq = wave_sum(dsq);
-      if (tid == 0) deltas[(int64_t)h * max_iter + it] = dsq;
+  // ---- k_hat_0 and the alternating rank-1 solves, all inside the first wave: lane c (and c + 32)
+  // holds column c of both inverses and element c of every vector; a vector element is
+  // broadcast with readlane, so the chain of small solves needs no barrier and no LDS round trip.
+  if (wave == 0) {
+    const int c = lane & 31;
+    float cK[32], cQ[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      cK[i] = GKi[i * kLdi + c];
+      cQ[i] = GQi[i * kLdi + c];
     }
-    __syncthreads();
-    float* o = iter_out + ((int64_t)h * max_iter + it) * 2 * r;
-    if (tid < 32) {
-      if (tid < r) {
-        o[tid] = hat_q[tid];
-        o[r + tid] = new_k[tid];
+    const float rq = rhs_q[c], kb = kB[c], sqk = s_qk;
+    // y_c = sum_i b_i col[i]  (b lane-distributed)
+    auto vecmat = [&](float bvec, const float (&col)[32]) {
+      float y0 = 0.0f, y1 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; i += 2) {
+        y0 = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(bvec), i)), col[i], y0);
+        y1 = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(bvec), i + 1)), col[i + 1], y1);
       }
-      hat_k[tid] = new_k[tid];
+      return y0 + y1;
+    };
+    auto dot32 = [&](float a, float bb) { return sum_lanes_0_31(a * bb); };
+    // x = b (G + v^T v)^-1 from G^-1 (Sherman-Morrison): x = y - (y.v / (1 + z.v)) z, y = b G^-1, z = v G^-1
+    auto rank1 = [&](float bvec, float v, const float (&col)[32]) {
+      const float y = vecmat(bvec, col);
+      const float z = vecmat(v, col);
+      const float alpha = dot32(y, v) / (1.0f + dot32(z, v));
+      return fmaf(-alpha, z, y);
+    };
+    float hk = vecmat(kb, cK);  // k_hat_0 = kB G_K^-1
+    for (int it = 0; it < max_iter; ++it) {
+      const float hq = rank1(fmaf(sqk, hk, rq), hk, cQ);  // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
+      const float nk = rank1(fmaf(sqk, hq, kb), hq, cK);  // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat
+      const float df = c < r ? hk - nk : 0.0f;
+      const float dsq = dot32(df, df);
+      if (lane == 0) deltas[(int64_t)h * max_iter + it] = dsq;
+      float* o = iter_out + ((int64_t)h * max_iter + it) * 2 * r;
+      if (lane < r) {
+        o[lane] = hq;
+        o[r + lane] = nk;
+      }
+      hk = nk;
     }
-    __syncthreads();
   }
 }
 
@@ -628,3 +648,4 @@ extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, i
   return als_decode_impl<bf16_t>(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q,
                                  k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, st);
 }
+

@@ -516,7 +516,10 @@ struct PfSmallShared {
 // col[i], i < 32: this thread's column.  On return the RHS columns hold G^-1 RHS.
 __device__ __forceinline__ void pf_solve32(float (&colv)[32], PfSmallShared& sh) {
   const int tid = threadIdx.x;
-#pragma unroll
+  // The rows are rotated by one after every pivot, so the pivot is always element 0 and the
+  // loop body is the same code for every p (a rolled loop keeps the code small: it runs once
+  // per workgroup, from a cold instruction cache).
+#pragma unroll 1
   for (int p = 0; p < 32; ++p) {
     float4* cb4 = reinterpret_cast<float4*>(sh.cbuf[p & 1]);
     if (tid == p) {
@@ -530,12 +533,10 @@ __device__ __forceinline__ void pf_solve32(float (&colv)[32], PfSmallShared& sh)
       const float4 t = cb4[i];
       cb[4 * i] = t.x; cb[4 * i + 1] = t.y; cb[4 * i + 2] = t.z; cb[4 * i + 3] = t.w;
     }
-    const float inv = 1.0f / cb[p];
-    const float mp = colv[p] * inv;
+    const float mp = colv[0] * (1.0f / cb[0]);
 #pragma unroll
-    for (int i = 0; i < 32; ++i)
-      if (i != p) colv[i] = fmaf(-cb[i], mp, colv[i]);
-    colv[p] = mp;
+    for (int i = 0; i < 31; ++i) colv[i] = fmaf(-cb[i + 1], mp, colv[i + 1]);
+    colv[31] = mp;
   }
   __syncthreads();
 }
