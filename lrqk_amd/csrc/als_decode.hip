@@ -195,21 +195,10 @@ __device__ __forceinline__ void invert_pair_regs(float (&colv)[32], float* cbuf,
   __syncthreads();
 }
 
-// Sum of x over lanes 0..31 of the wave with data-parallel-primitive moves (no LDS round trips):
-// butterflies inside each row of 16 lanes, then lane 15 of row 0 is added into row 1; the total
-// is read from lane 31.  Every lane of the wave must call it.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add(float v) {
-  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
-  return v + __int_as_float(t);
-}
+// Sum of x over lanes 0..31 of the wave (the first two rows of 16 lanes); every lane must call it.
 __device__ __forceinline__ float sum_lanes_0_31(float x) {
-  x = dpp_add<0xB1, 0xf>(x);   // quad_perm [1,0,3,2]
-  x = dpp_add<0x4E, 0xf>(x);   // quad_perm [2,3,0,1]
-  x = dpp_add<0x141, 0xf>(x);  // row_half_mirror
-  x = dpp_add<0x140, 0xf>(x);  // row_mirror
-  x = dpp_add<0x142, 0xa>(x);  // row_bcast15 into rows 1 and 3
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 31));
+  x = row_reduce(x, [](float a, float b) { return a + b; });
+  return lane_bcast(x, 0) + lane_bcast(x, 16);
 }
 
 // iter_out per head: [max_iter][2r] (q_hat then k_hat of each iteration);

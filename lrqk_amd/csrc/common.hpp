@@ -119,25 +119,52 @@ __device__ __forceinline__ int wave_rank(bool pred, int& total) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
-// inclusive wave scan (sum) via shuffles
+// Cross-lane moves of the data-parallel-primitive kind (no LDS round trip, unlike a shuffle).
+// Lanes that the row / bank mask disables, or whose source lies outside the row, receive 0.
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ int dpp_mov0(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, BANK_MASK, false);
+}
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kDppRowShr1 = 0x111, kDppRowShr2 = 0x112, kDppRowShr3 = 0x113, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+constexpr int kDppRowMirror = 0x140, kDppRowHalfMirror = 0x141;
+constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143;
+
+// inclusive wave scan (sum): three shifted copies of the input, then doubling steps inside each
+// row of 16 lanes, then the row totals are passed on (lane 15 -> next row, lane 31 -> rows 2, 3)
 __device__ __forceinline__ int wave_inclusive_sum(int v) {
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    int t = __shfl_up(v, off, kWave);
-    if (lane_id() >= off) v += t;
-  }
-  return v;
+  int x = v + dpp_mov0<kDppRowShr1, 0xf, 0xf>(v);
+  x += dpp_mov0<kDppRowShr2, 0xf, 0xf>(v);
+  x += dpp_mov0<kDppRowShr3, 0xf, 0xf>(v);
+  x += dpp_mov0<kDppRowShr4, 0xf, 0xe>(x);
+  x += dpp_mov0<kDppRowShr8, 0xf, 0xc>(x);
+  x += dpp_mov0<kDppRowBcast15, 0xa, 0xf>(x);
+  x += dpp_mov0<kDppRowBcast31, 0xc, 0xf>(x);
+  return x;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+// Butterflies inside each row of 16 lanes; afterwards every lane of a row holds the row's result.
+template <typename Op>
+__device__ __forceinline__ float row_reduce(float v, Op op) {
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), kDppQuadXor1, 0xf, 0xf, false)));
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), kDppQuadXor2, 0xf, 0xf, false)));
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), kDppRowHalfMirror, 0xf, 0xf, false)));
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), kDppRowMirror, 0xf, 0xf, false)));
   return v;
 }
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// result in every lane
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row_reduce(v, [](float a, float b) { return a + b; });
+  return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  v = row_reduce(v, [](float a, float b) { return fmaxf(a, b); });
+  return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
 }
 
 // Workgroup-wide rank of a predicate in thread order.  `scratch` needs blockDim/64 + 1

@@ -222,15 +222,7 @@ constexpr int kFusedDiffMaxK = 4096;          // LDS budget of the in-kernel dif
 
 // Inclusive block scan of two counters at once.  scratch: 2 * kSelWaves ints.  Two barriers.
 __device__ __forceinline__ void block_inclusive_sum2(int& a, int& b, int* scratch, int& tot_a, int& tot_b) {
-  int ia = a, ib = b;
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const int ta = __shfl_up(ia, off, kWave), tb = __shfl_up(ib, off, kWave);
-    if (lane_id() >= off) {
-      ia += ta;
-      ib += tb;
-    }
-  }
+  const int ia = wave_inclusive_sum(a), ib = wave_inclusive_sum(b);
   if (lane_id() == kWave - 1) {
     scratch[wave_id()] = ia;
     scratch[kSelWaves + wave_id()] = ib;
@@ -250,6 +242,35 @@ __device__ __forceinline__ void block_inclusive_sum2(int& a, int& b, int* scratc
   __syncthreads();
   a = base_a + ia;
   b = base_b + ib;
+  tot_a = ta;
+  tot_b = tb;
+}
+
+// Workgroup-wide exclusive ranks of two predicates in thread order (ballots, no scan).
+// scratch: 2 * kSelWaves ints.  Two barriers.
+__device__ __forceinline__ void block_rank2(bool pa, bool pb, int* scratch, int& rank_a, int& rank_b, int& tot_a,
+                                            int& tot_b) {
+  int wa, wb;
+  const int ra = wave_rank(pa, wa), rb = wave_rank(pb, wb);
+  if (lane_id() == 0) {
+    scratch[wave_id()] = wa;
+    scratch[kSelWaves + wave_id()] = wb;
+  }
+  __syncthreads();
+  int base_a = 0, base_b = 0, ta = 0, tb = 0;
+#pragma unroll
+  for (int w = 0; w < kSelWaves; ++w) {
+    const int ca = scratch[w], cb = scratch[kSelWaves + w];
+    if (w < wave_id()) {
+      base_a += ca;
+      base_b += cb;
+    }
+    ta += ca;
+    tb += cb;
+  }
+  __syncthreads();
+  rank_a = base_a + ra;
+  rank_b = base_b + rb;
   tot_a = ta;
   tot_b = tb;
 }
@@ -335,6 +356,16 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   const uint2* cand = cand_all + (int64_t)h * cand_cap;
   int32_t* out = out_all + (int64_t)h * out_stride;
 
+  // the resident token ids of the fused diff do not depend on the selection: requested now,
+  // used at the end (items tid*kDiffIpt .. +kDiffIpt-1, contiguous per thread to keep slot order)
+  constexpr int kDiffIpt = kFusedDiffMaxK / kSelThreads;
+  const int ipt = (k + kSelThreads - 1) / kSelThreads;  // items per thread actually in use (<= kDiffIpt)
+  int32_t hv[kDiffIpt];
+  if (df.hit != nullptr && !df.replace_all) {
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u)
+      hv[u] = df.hit[(int64_t)h * df.hit_stride + min(tid * ipt + u, k - 1)];
+  }
   bool fast = false;
   int64_t N = m;
   uint32_t lo = 0;
@@ -502,9 +533,15 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   for (int64_t c0 = 0; c0 < m; c0 += kChunkBits) {
     const int span = (int)min((int64_t)kChunkBits, m - c0);
     const int words = (span + 31) >> 5;
-    for (int i = tid; i < words; i += kSelThreads) {
-      gt[i] = 0;
-      eq[i] = 0;
+    // each thread owns W consecutive words (4 or 8: whole 16-byte vectors, read once into registers)
+    const int W = (((words + kSelThreads - 1) / kSelThreads) + 3) & ~3;
+    {
+      uint4* g4 = reinterpret_cast<uint4*>(gt);
+      uint4* e4 = reinterpret_cast<uint4*>(eq);
+      for (int i = tid; i < W * kSelThreads / 4; i += kSelThreads) {
+        g4[i] = make_uint4(0, 0, 0, 0);
+        e4[i] = make_uint4(0, 0, 0, 0);
+      }
     }
     __syncthreads();
     for_each([&](uint32_t key, int64_t idx) {
@@ -512,28 +549,42 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       if (key >= Tk && rel >= 0 && rel < span) atomicOr(key > Tk ? &gt[rel >> 5] : &eq[rel >> 5], 1u << (rel & 31));
     });
     __syncthreads();
-    const int W = (words + kSelThreads - 1) / kSelThreads;
     const int w0 = tid * W;
+    uint32_t gwr[8], ewr[8];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      uint4 a = make_uint4(0, 0, 0, 0), b = a;
+      if (q * 4 < W) {
+        a = reinterpret_cast<const uint4*>(gt)[(w0 >> 2) + q];
+        b = reinterpret_cast<const uint4*>(eq)[(w0 >> 2) + q];
+      }
+      gwr[4 * q] = a.x; gwr[4 * q + 1] = a.y; gwr[4 * q + 2] = a.z; gwr[4 * q + 3] = a.w;
+      ewr[4 * q] = b.x; ewr[4 * q + 1] = b.y; ewr[4 * q + 2] = b.z; ewr[4 * q + 3] = b.w;
+    }
     int cg = 0, ce = 0;
-    for (int w = w0; w < min(words, w0 + W); ++w) {
-      cg += __popc(gt[w]);
-      ce += __popc(eq[w]);
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      cg += __popc(gwr[x]);
+      ce += __popc(ewr[x]);
     }
     int g_incl = cg, e_incl = ce, g_tot, e_tot;
     block_inclusive_sum2(g_incl, e_incl, scratch, g_tot, e_tot);
     int e_run = eq_seen + e_incl - ce;  // equal keys before this thread's words (all chunks)
     int pos = out_pos + (g_incl - cg) + (min(e_run, need_eq) - min(eq_seen, need_eq));
-    for (int w = w0; w < min(words, w0 + W); ++w) {
-      const uint32_t gw = gt[w], ew = eq[w];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const uint32_t gw = gwr[x], ew = ewr[x];
       uint32_t both = gw | ew;
+      uint32_t sel = gw;
       while (both) {
         const int bit = __ffs((int)both) - 1;
         both &= both - 1;
-        const int32_t idx = (int32_t)(c0 + (int64_t)w * 32 + bit);
+        const int32_t idx = (int32_t)(c0 + (int64_t)(w0 + x) * 32 + bit);
         bool take = true;
         if (!((gw >> bit) & 1u)) {
           take = e_run < need_eq;
           ++e_run;
+          if (take) sel |= 1u << bit;
         }
         if (take) {
           out[pos] = idx;
@@ -541,6 +592,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
           ++pos;
         }
       }
+      if (do_diff && sel != gw) gt[w0 + x] = sel;  // gt then marks exactly the selected tokens (used by the diff)
     }
     out_pos += g_tot + (min(eq_seen + e_tot, need_eq) - min(eq_seen, need_eq));
     eq_seen += e_tot;
@@ -564,32 +616,89 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   int32_t* miss_s = new_s + k;                                   // [k] missing tokens, ascending
   uint8_t* matched = reinterpret_cast<uint8_t*>(miss_s + k);     // [k]
   uint8_t* evict_s = matched + k;                                // [k]
-  for (int i = tid; i < k; i += kSelThreads) matched[i] = 0;
-  __syncthreads();
-  for (int s = tid; s < k; s += kSelThreads) {
-    const int32_t v = hit[s];
-    int lo_i = 0, hi_i = k;
-    while (lo_i < hi_i) {
-      const int mid = (lo_i + hi_i) >> 1;
-      if (new_s[mid] < v) lo_i = mid + 1; else hi_i = mid;
+  if (m <= kChunkBits) {
+    // One chunk: gt[] still marks the selected tokens.  eq[] becomes the bitmap of the resident
+    // tokens; membership either way is one bit test.
+    const int words = (int)((m + 31) >> 5);
+    for (int i = tid; i < words; i += kSelThreads) eq[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u) {
+      const int s = tid * ipt + u;
+      if (u < ipt && s < k) {
+        const int32_t v = hv[u];
+        const bool in_range = v >= 0 && v < m;
+        if (in_range) atomicOr(&eq[v >> 5], 1u << (v & 31));
+        const bool found = in_range && ((gt[in_range ? (v >> 5) : 0] >> (v & 31)) & 1u);
+        evict_s[s] = found ? 0 : 1;
+      }
     }
-    const bool found = lo_i < k && new_s[lo_i] == v;
-    if (found) matched[lo_i] = 1;
-    evict_s[s] = found ? 0 : 1;
+    __syncthreads();
+    for (int i = tid; i < k; i += kSelThreads) {
+      const int32_t t = new_s[i];
+      matched[i] = (uint8_t)((eq[t >> 5] >> (t & 31)) & 1u);
+    }
+  } else {
+    for (int i = tid; i < k; i += kSelThreads) matched[i] = 0;
+    __syncthreads();
+    // lower bound of every resident id in new_s; the searches of a thread's items advance in step
+    int lo_i[kDiffIpt], len[kDiffIpt];
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u) {
+      lo_i[u] = 0;
+      len[u] = k;
+    }
+    for (int step = 32 - __clz(k); step > 0; --step) {
+      int32_t probe[kDiffIpt];
+#pragma unroll
+      for (int u = 0; u < kDiffIpt; ++u)
+        if (u < ipt) probe[u] = new_s[min(lo_i[u] + (len[u] >> 1), k - 1)];
+#pragma unroll
+      for (int u = 0; u < kDiffIpt; ++u) {
+        const int half = len[u] >> 1;
+        if (u < ipt && len[u] > 0) {
+          if (probe[u] < hv[u]) {
+            lo_i[u] += half + 1;
+            len[u] -= half + 1;
+          } else {
+            len[u] = half;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u) {
+      const int s = tid * ipt + u;
+      if (u < ipt && s < k) {
+        const bool found = lo_i[u] < k && new_s[min(lo_i[u], k - 1)] == hv[u];
+        if (found) matched[lo_i[u]] = 1;
+        evict_s[s] = found ? 0 : 1;
+      }
+    }
   }
   __syncthreads();
   // both ordered compactions in one sweep: rank of missing tokens and of evicted slots
-  int n_missing = 0, n_evict = 0;
-  for (int base = 0; base < k; base += kSelThreads) {
-    const int i = base + tid;
-    const bool miss = i < k && matched[i] == 0;
-    const bool ev = i < k && evict_s[i] != 0;
-    int a = miss ? 1 : 0, b2 = ev ? 1 : 0, ta, tb;
-    block_inclusive_sum2(a, b2, scratch, ta, tb);
-    if (miss) miss_s[n_missing + a - 1] = new_s[i];
-    if (ev) reinterpret_cast<int32_t*>(gt)[n_evict + b2 - 1] = i;  // evicted slots, ascending (bitmaps are free now)
-    n_missing += ta;
-    n_evict += tb;
+  int n_missing, n_evict;
+  {
+    bool miss[kDiffIpt], ev[kDiffIpt];
+    int a = 0, b2 = 0;
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u) {
+      const int i = tid * ipt + u;
+      miss[u] = u < ipt && i < k && matched[min(i, k - 1)] == 0;
+      ev[u] = u < ipt && i < k && evict_s[min(i, k - 1)] != 0;
+      a += miss[u] ? 1 : 0;
+      b2 += ev[u] ? 1 : 0;
+    }
+    int ia = a, ib = b2;
+    block_inclusive_sum2(ia, ib, scratch, n_missing, n_evict);
+    int pa = ia - a, pb = ib - b2;
+#pragma unroll
+    for (int u = 0; u < kDiffIpt; ++u) {
+      const int i = tid * ipt + u;
+      if (miss[u]) miss_s[pa++] = new_s[i];
+      if (ev[u]) reinterpret_cast<int32_t*>(gt)[pb++] = i;  // evicted slots, ascending (bitmaps are free now)
+    }
   }
   __syncthreads();
   const int n_pair = min(n_missing, n_evict);
@@ -839,3 +948,4 @@ extern "C" int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads
   if (reset) LRQK_HIP_CHECK(hipMemset(stats, 0, sizeof(v)));
   return LRQK_OK;
 }
+
