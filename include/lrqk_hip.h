@@ -30,7 +30,7 @@ extern "C" {
 #define LRQK_EHIP (-2)     /* a HIP runtime call failed */
 #define LRQK_ELIMIT (-3)   /* size beyond what the kernels support */
 
-#define LRQK_MAX_R 64
+#define LRQK_MAX_R 64          /* scan / select; the factor updates (lrqk_als_*) take r <= 32 */
 #define LRQK_MAX_TOPK 8192
 #define LRQK_MAX_DECODE_ITERS 16
 
@@ -86,6 +86,15 @@ int lrqk_select_stats_detail(lrqk_ctx* ctx, int* list_short, int* list_overflow)
 int lrqk_diff(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t hit_stride, int bh, int k,
               uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, void* stream);
 
+/* py:1235-1273 + py:1275-1315 in one pass -- lrqk_score_select followed by lrqk_diff, with the
+ * diff done by the select kernel while the selection is still on chip (m > topk required).
+ * new_idx: [bh][topk] receives the ascending selection; hit / evict / miss_slots / miss_count
+ * as in lrqk_diff (evict may be NULL). */
+int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh,
+                           int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit,
+                           int64_t hit_stride, uint8_t* evict, int32_t* miss_slots, int32_t* miss_count,
+                           void* stream);
+
 /* py:1752, 1762-1773 (LightAttentionIndicesNoHitMiss) -- the ablation without hit/miss
  * bookkeeping: hit <- new_idx, every slot marked evicted (all k rows are refetched). */
 int lrqk_replace_all(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t hit_stride, int bh, int k,
@@ -139,9 +148,10 @@ int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head
 /* py:772-800 cast_lrqk_prefill -> py:319-423 _lrqk_prefill_inv_w1 -- joint rank-r ALS fit.
  * q: [b][hq][l][d], k: [b][hkv][l][d] storage dtype (query head h uses KV head h/groups);
  * a_q,a_k: [bh][l][r] fp32 work buffers holding the initial factors on entry and the
- * result on return; b_q,b_k out: [bh][r][d] fp32.  Synchronises the stream once per
- * iteration to evaluate the stopping test on the host.  Returns the number of
- * iterations run (>= 0). */
+ * result on return; b_q,b_k out: [bh][r][d] fp32.  The stopping test (batch-wide mean squared
+ * change of A_Q and A_K below tol) is evaluated on the device: once it fires the remaining
+ * launches return at once, and the host never waits.  r <= 32 and head dimensions that are a
+ * multiple of 16 bytes run on fp32 MFMA tiles, other shapes on a generic kernel.  Returns 0. */
 int lrqk_als_prefill(lrqk_ctx* ctx, const void* q, const void* k, float* a_q, float* a_k, float* b_q,
                      float* b_k, int b, int hq, int hkv, int64_t l, int r, int d, int max_iter, float tol,
                      int dtype, void* stream);

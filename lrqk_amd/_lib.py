@@ -45,6 +45,7 @@ def _sig(lib):
         "lrqk_ctx_reserve": ([vp, i32, i64, i32, i32, i32, i32], i32),
         "lrqk_proxy_scores": ([vp, i64, vp, i32, i64, i32, i32, i32, vp, vp], i32),
         "lrqk_score_select": ([vp, vp, i64, vp, i32, i64, i32, i32, i32, i32, vp, i64, vp], i32),
+        "lrqk_score_select_diff": ([vp, vp, i64, vp, i32, i64, i32, i32, i32, i32, vp, vp, i64, vp, vp, vp, vp], i32),
         "lrqk_select_from_scores": ([vp, vp, i32, i64, i32, vp, i64, vp], i32),
         "lrqk_diff": ([vp, i64, vp, i64, i32, i32, vp, vp, vp, vp], i32),
         "lrqk_replace_all": ([vp, i64, vp, i64, i32, i32, vp, vp, vp, vp], i32),

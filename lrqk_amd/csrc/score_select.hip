@@ -905,6 +905,23 @@ extern "C" int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_st
   return rc ? rc : topk;
 }
 
+extern "C" int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh,
+                                      int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* new_idx,
+                                      int32_t* hit, int64_t hit_stride, uint8_t* evict, int32_t* miss_slots,
+                                      int32_t* miss_count, void* stream) {
+  LRQK_REQUIRE(a_k && q_hat && new_idx && hit && miss_slots && miss_count, LRQK_EINVAL, "null pointer");
+  LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
+  LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_EINVAL, "r=%d", r);
+  LRQK_REQUIRE(m > topk, LRQK_EINVAL, "m=%lld must exceed topk=%d (no diff happens in the prefix branch)",
+               (long long)m, topk);
+  LRQK_REQUIRE(head_stride >= m * r && hit_stride >= topk, LRQK_EINVAL, "stride too small");
+  int rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_bf16, new_idx, hit, hit_stride,
+                             evict, miss_slots, miss_count, 0, (hipStream_t)stream);
+  if (rc < 0) return rc;
+  if (rc == 0) return lrqk_diff(new_idx, topk, hit, hit_stride, bh, topk, evict, miss_slots, miss_count, stream);
+  return LRQK_OK;
+}
+
 extern "C" int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int bh, int64_t m, int topk,
                                        int32_t* out_idx, int64_t out_stride, void* stream) {
   int rc = check_select_args(ctx, bh, m, topk, out_idx, out_stride);

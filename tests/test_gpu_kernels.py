@@ -172,6 +172,53 @@ def _check_diff(ops, oracle, now, new):
             assert torch.equal(slots[i, h, :c].cpu().long(), mask[i, h].nonzero()[:, 0])
 
 
+@pytest.mark.parametrize("m,cap,k,H,dtype", [(5000, 5008, 512, 3, torch.float32), (40000, 40000, 2048, 2, torch.bfloat16),
+                                             (300000, 300032, 2048, 2, torch.bfloat16),
+                                             (270000, 270000, 4096, 1, torch.bfloat16),
+                                             (20000, 20000, 4100, 1, torch.float32)])
+def test_score_select_diff_fused(ops, oracle, m, cap, k, H, dtype):
+    """Selection and hit/miss diff in one pass against the oracle's two stages: one bitmap chunk
+    (m <= 262144), several chunks, the largest fused k, and a k beyond it (separate diff launch).
+    Second round on the same workspace goes through the filtered path."""
+    _say("score_select_diff", m, k, H, dtype)
+    ws = ops.Workspace()
+    g = torch.Generator().manual_seed(m + k)
+    r = 16
+    A = torch.randn((1, H, cap, r), generator=g).to(dtype)
+    q = torch.randn((1, H, 1, r), generator=g).to(dtype)
+    # resident set: random unique tokens below m, in random order
+    hit = torch.stack([torch.randperm(m, generator=g)[:k] for _ in range(H)]).view(1, H, k).to(torch.int32)
+    Ad = A.to(DEV)
+    hit_d = hit.to(DEV).contiguous()
+    now = hit.long().unsqueeze(-1)
+    for rnd in range(2):
+        exp_new = oracle.compute_hit_indices(q, A[:, :, :m].contiguous(), k, True)
+        exp_upd, exp_ev = oracle.only_indices_in_cpu(now, exp_new)
+        new, evict, slots, count = ops.score_select_diff(ws, Ad, q.to(DEV), m, k, hit_d)
+        assert torch.equal(new.cpu().long(), exp_new[..., 0]), rnd
+        assert torch.equal(hit_d.cpu().long(), exp_upd[..., 0]), rnd
+        assert torch.equal(evict.cpu().bool(), exp_ev), rnd
+        assert torch.equal(count.cpu().long(), exp_ev.sum(-1)), rnd
+        for h in range(H):
+            c = int(count[0, h])
+            assert slots[0, h, :c].cpu().tolist() == exp_ev[0, h].nonzero().view(-1).tolist()
+        now = exp_upd
+        q = (q.float() + 0.05 * torch.randn(q.shape, generator=g)).to(dtype)
+
+
+def test_score_select_many_chunks(ops, ws, oracle):
+    """More candidates than one bitmap chunk covers (262144): the ordered output runs chunk by chunk."""
+    _say("score_select many chunks")
+    g = torch.Generator().manual_seed(5)
+    m, cap, r, k = 600000, 600000, 8, 2048
+    A = torch.randn((1, 2, cap, r), generator=g).bfloat16()
+    q = torch.randn((1, 2, 1, r), generator=g).bfloat16()
+    exp = oracle.compute_hit_indices(q, A, k, True)[..., 0].to(torch.int32)
+    for _ in range(2):   # second call: filtered path
+        got = ops.score_select(ws, A.to(DEV), q.to(DEV), m, k, True).cpu()
+        assert torch.equal(got, exp)
+
+
 def test_diff_docstring_vector(ops, oracle):
     _say("diff docstring")
     now = torch.tensor([0, 1, 2, 6, 7]).view(1, 1, 5)
