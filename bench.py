@@ -45,6 +45,8 @@ def parse():
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
+    p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
+                   help="miss fetch: the kernel reads the pinned store itself, or host gather + hipMemcpyAsync")
     p.add_argument("--mode", default="decode", choices=["decode", "prefill_als"],
                    help="prefill_als: time the prefill factorisation alone (workload llama8b_32k_prefill_als unless "
                         "--workload is given); a step is one whole factorisation")
@@ -160,6 +162,7 @@ def main():
               max_iter=w.max_iter, tol=w.tol, capacity=4096)
     eng.init_factors = A0
     eng.attn_in_step = not a.no_attn
+    eng.fetch_mode = a.fetch
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     eng.prefill(Q, K, V)
@@ -254,7 +257,7 @@ def main():
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
                    "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
-                   "variant": a.variant, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
+                   "variant": a.variant, "fetch": a.fetch, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round(n_miss / a.steps * row_bytes),

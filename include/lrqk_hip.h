@@ -111,6 +111,18 @@ int lrqk_fetch_rows(const void* kv_store, int64_t cap, void* k_act, void* v_act,
                     const int32_t* miss_count, int b, int hq, int hkv, int d, int k, int dtype,
                     void* stream);
 
+/* py:101-117 + py:1597-1608 as the reference stages it -- the same fetch through a staging block:
+ * the miss list is copied to the host (the call waits for the stream once), the host gathers the
+ * rows of the pinned store (cpp:13-124) into pinned staging memory owned by the ctx, one
+ * hipMemcpyAsync on the ctx's side stream moves them, the caller's stream waits on an event and a
+ * kernel scatters them into the slots.  kv_store must be pinned host memory. */
+int lrqk_fetch_rows_staged(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
+                           const int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
+                           const int32_t* miss_count, int b, int hq, int hkv, int d, int k, int dtype, void* stream);
+/* Which fetch lrqk_decode_step uses: 0 (default) lrqk_fetch_rows, 1 lrqk_fetch_rows_staged with
+ * host_threads gather threads (<= 0 keeps the current count).  No counterpart in the reference. */
+int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
+
 /* py:1339-1351 fetch_by_hit (same-device branch) -- k_act[bh][j][:] = src[b][h/groups][idx[bh][j]][:]
  * for j < count, src: [b][hkv][src_len][d] on the device. */
 int lrqk_gather_rows(const void* src, int64_t src_len, const int32_t* idx, int64_t idx_stride, int count,

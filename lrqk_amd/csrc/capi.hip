@@ -10,6 +10,7 @@
 
 #include "common.hpp"
 #include "ctx.hpp"
+#include "hostpar.hpp"
 
 namespace lrqk {
 
@@ -21,24 +22,6 @@ int set_error(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
-}
-
-template <typename F>
-static void parallel_ranges(int64_t n, int threads, int64_t min_chunk, F&& fn) {
-  if (threads < 1) threads = 1;
-  int64_t parts = std::min<int64_t>(threads, (n + min_chunk - 1) / std::max<int64_t>(min_chunk, 1));
-  if (parts <= 1) {
-    fn(0, n);
-    return;
-  }
-  std::vector<std::thread> pool;
-  int64_t step = (n + parts - 1) / parts;
-  for (int64_t p = 0; p < parts; ++p) {
-    int64_t lo = p * step, hi = std::min(n, lo + step);
-    if (lo >= hi) break;
-    pool.emplace_back([=, &fn] { fn(lo, hi); });
-  }
-  for (auto& t : pool) t.join();
 }
 
 }  // namespace lrqk
@@ -68,6 +51,10 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->prefill_ws.release();
   ctx->new_idx.release();
   ctx->misc.release();
+  ctx->stage_dev.release();
+  if (ctx->stage_host) (void)hipHostFree(ctx->stage_host);
+  if (ctx->stage_ev) (void)hipEventDestroy(ctx->stage_ev);
+  if (ctx->side) (void)hipStreamDestroy(ctx->side);
   if (ctx->tev) {
     for (int i = 0; i < 2 * ctx->tev_pairs; ++i) (void)hipEventDestroy(ctx->tev[i]);
     delete[] ctx->tev;

@@ -52,6 +52,14 @@ struct lrqk_ctx {
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
   lrqk::DevBuf misc;        // evict mask, miss lists, counters of the fused step
+  // staged miss fetch: pinned host staging, its device twin, side stream and event (created on first use)
+  lrqk::DevBuf stage_dev;
+  void* stage_host = nullptr;
+  size_t stage_host_bytes = 0;
+  hipStream_t side = nullptr;
+  hipEvent_t stage_ev = nullptr;
+  int fetch_mode = 0;  // 0: the kernel reads the pinned store directly; 1: host gather + hipMemcpyAsync on the side stream
+  int host_threads = 8;
   // optional event timing of the proxy-score kernel (two events per launch)
   hipEvent_t* tev = nullptr;
   int tev_pairs = 0;   // capacity in pairs

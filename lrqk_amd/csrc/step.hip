@@ -48,6 +48,13 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
       rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
     if (rc) return rc;
   }
+  if (ctx->fetch_mode == 1) {
+    if ((rc = lrqk_fetch_rows_staged(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv,
+                                     d, topk, dtype, stream)))
+      return rc;
+    if (attn_out) return lrqk_attention(ctx, q, k_act, v_act, n, n, attn_out, bh, d, dtype, stream);
+    return LRQK_OK;
+  }
   if (attn_out && !no_hit_miss) {
     // the fetch is bound by the host link: the attention over the resident slots runs beside it
     return fetch_attention(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, ev, b, hq, hkv, d,

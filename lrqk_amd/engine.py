@@ -77,8 +77,20 @@ class LightAttentionIndicesFactory:
         self.last_miss_count = None   # int32 [b,Hq]
         self.last_attn = None
         self.attn_in_step = False     # compute attention inside the fused step (uses the step's q)
+        self._fetch_mode = "direct"
 
     # ------------------------------------------------------------------ small accessors
+    @property
+    def fetch_mode(self) -> str:
+        """'direct' (the fetch kernel reads the pinned store) or 'staged' (host gather into pinned staging +
+        hipMemcpyAsync on a side stream + scatter, the way lrqk_attention.py:1597-1608 moves its misses)."""
+        return self._fetch_mode
+
+    @fetch_mode.setter
+    def fetch_mode(self, mode: str):
+        self.ws.set_fetch_mode(mode)
+        self._fetch_mode = mode
+
     def __len__(self):
         return self.current_len
 
@@ -314,7 +326,11 @@ class LightAttentionIndicesFactory:
             evict = mask.to(torch.uint8).contiguous()
             slots, count = _slots_from_mask(evict)
         self.last_evict, self.last_miss_count = evict, count
-        ops.fetch_rows(self.KVcpu.data, self.Kgpu, self.Vgpu, self._active_idx, slots, count, evict.shape[2])
+        if self._fetch_mode == "staged":
+            ops.fetch_rows_staged(self.ws, self.KVcpu.data, self.Kgpu, self.Vgpu, self._active_idx, slots, count,
+                                  evict.shape[2])
+        else:
+            ops.fetch_rows(self.KVcpu.data, self.Kgpu, self.Vgpu, self._active_idx, slots, count, evict.shape[2])
         return self.Kgpu, self.Vgpu
 
     # ------------------------------------------------------------------ statistics

@@ -47,6 +47,11 @@ class Workspace:
     def reserve(self, bh, max_tokens, topk, n_active, r, d):
         check(_lib.load().lrqk_ctx_reserve(self._h, bh, max_tokens, topk, n_active, r, d))
 
+    def set_fetch_mode(self, mode: str, host_threads: int = 0):
+        """'direct': the fetch kernel reads the pinned store itself (default); 'staged': host gather +
+        hipMemcpyAsync on a side stream, as the reference stages its misses."""
+        check(_lib.load().lrqk_ctx_set_fetch_mode(self.handle, {"direct": 0, "staged": 1}[mode], int(host_threads)))
+
     def timing_enable(self, max_launches: int):
         check(_lib.load().lrqk_timing_enable(self._h, max_launches))
 
@@ -195,6 +200,22 @@ def fetch_rows(kv_store: torch.Tensor, k_act: torch.Tensor, v_act: torch.Tensor,
     check(_lib.load().lrqk_fetch_rows(kv_store.data_ptr(), cap, k_act.data_ptr(), v_act.data_ptr(), n, hit.data_ptr(),
                                       hit.shape[2], miss_slots.data_ptr(), miss_count.data_ptr(), b, hq, hkv, d, k,
                                       _dt(k_act), _stream(k_act)))
+
+
+def fetch_rows_staged(ws: Workspace, kv_store: torch.Tensor, k_act: torch.Tensor, v_act: torch.Tensor,
+                      hit: torch.Tensor, miss_slots: torch.Tensor, miss_count: torch.Tensor, k: int):
+    """Same result as fetch_rows, through host gather + hipMemcpyAsync on the workspace's side stream
+    (kv_store must be pinned host memory; waits for the stream once)."""
+    _need_cuda(k_act, v_act, hit, miss_slots, miss_count)
+    b, hkv, cap, d2 = kv_store.shape
+    _, hq, n, d = k_act.shape
+    assert d2 == 2 * d and kv_store.is_contiguous() and k_act.is_contiguous() and v_act.is_contiguous()
+    assert kv_store.dtype == k_act.dtype == v_act.dtype
+    if kv_store.is_cuda or not kv_store.is_pinned():
+        raise ValueError("the staged fetch needs the [K|V] store in pinned host memory")
+    check(_lib.load().lrqk_fetch_rows_staged(ws.handle, kv_store.data_ptr(), cap, k_act.data_ptr(), v_act.data_ptr(), n,
+                                             hit.data_ptr(), hit.shape[2], miss_slots.data_ptr(),
+                                             miss_count.data_ptr(), b, hq, hkv, d, k, _dt(k_act), _stream(k_act)))
 
 
 def gather_rows(src: torch.Tensor, idx: torch.Tensor, dst: torch.Tensor, count: int):

@@ -155,6 +155,21 @@ def test_edge_branch_then_main(lrqk, oracle):
               max_iter=(2, 2), tol=(1e-8, 1e-8), rho=3, capacity=8)
 
 
+def test_staged_fetch_trace(lrqk, oracle):
+    """The same lock-step trace with the misses moved by host gather + hipMemcpyAsync on the side
+    stream (buffer growth included: the pinned store is reallocated during the run)."""
+    _say("staged fetch trace")
+
+    class Staged(lrqk.LightAttentionIndicesFactory):
+        def __init__(self, *a, **kw):
+            super().__init__(*a, **kw)
+            self.fetch_mode = "staged"
+
+    _, _, n = _lockstep(lrqk, oracle, b=2, hq=4, hkv=2, d=16, l=40, r=4, k=8, L=4, steps=40, dtype=torch.float32,
+                        max_iter=(2, 2), tol=(1e-8, 1e-8), rho=4, capacity=16, cls=Staged)
+    assert n > 0
+
+
 def test_no_hit_miss_variant(lrqk, oracle):
     _say("no hit/miss trace")
     _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=16, l=40, r=4, k=8, L=4, steps=12, dtype=torch.float32,

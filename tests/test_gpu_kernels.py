@@ -292,6 +292,18 @@ def test_fetch_rows(ops, oracle, dtype, d, pinned):
     torch.cuda.synchronize()
     assert torch.equal(Kd.cpu(), expK) and torch.equal(Vd.cpu(), expV)
     assert torch.equal(hit[:, :, :k].cpu().long(), upd[..., 0])
+    if pinned:
+        # the staged path (host gather + hipMemcpyAsync on the side stream + scatter): same bytes, twice
+        # in a row on one workspace (the second call reuses the staging block)
+        ws = ops.Workspace()
+        for _ in range(2):
+            Kd2, Vd2 = Kg.to(DEV), Vg.to(DEV)
+            ops.fetch_rows_staged(ws, store_dev, Kd2, Vd2, hit, slots, cnt, k)
+            torch.cuda.synchronize()
+            assert torch.equal(Kd2.cpu(), expK) and torch.equal(Vd2.cpu(), expV)
+    else:
+        with pytest.raises(ValueError):
+            ops.fetch_rows_staged(ops.Workspace(), store_dev, Kd, Vd, hit, slots, cnt, k)
 
 
 def test_gather_append_flush(ops, oracle):
