@@ -43,6 +43,9 @@ def parse():
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--cpu-steps", type=int, default=3, help="oracle steps timed for cpu_baseline (0 = skip)")
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
+    p.add_argument("--event-every", type=int, default=8,
+                   help="bracket every n-th proxy-score launch of the timed region with HIP events (each pair "
+                        "of event packets delays its step by ~10 us, so every launch would inflate the step time)")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
@@ -190,7 +193,7 @@ def main():
     cap_before = (eng._A_K.capacity, eng.KVcpu.capacity)
     m_first = eng.lite_indices[eng.lite_len] - 1
 
-    eng.ws.timing_enable(a.steps)
+    eng.ws.timing_enable(a.steps, every=max(1, a.event_every))
     eng.ws.select_stats(reset=True)
     counts = []
     torch.cuda.synchronize()

@@ -192,6 +192,9 @@ int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t hea
  * lrqk_timing_read waits for them, returns the summed kernel time and the launch count, and
  * re-arms.  n = 0 switches timing off. */
 int lrqk_timing_enable(lrqk_ctx* ctx, int max_launches);
+/* Bracket only every `every`-th launch (default 1): the two event packets delay the kernels around
+ * them by a few microseconds, which a sampled measurement keeps out of most steps. */
+int lrqk_timing_stride(lrqk_ctx* ctx, int every);
 int lrqk_timing_read(lrqk_ctx* ctx, double* total_ms, int* launches);
 
 /* Host-side row gathers with the reference's native signatures (the staged fetch path

@@ -64,6 +64,7 @@ def _sig(lib):
         "lrqk_select_stats": ([vp, c.POINTER(i32), c.POINTER(i32), i32], i32),
         "lrqk_select_stats_detail": ([vp, c.POINTER(i32), c.POINTER(i32)], i32),
         "lrqk_timing_enable": ([vp, i32], i32),
+        "lrqk_timing_stride": ([vp, i32], i32),
         "lrqk_timing_read": ([vp, c.POINTER(c.c_double), c.POINTER(i32)], i32),
         "lrqk_d0_indices_select": ([vp, vp, vp, i64, i64, i64, i32], i32),
         "lrqk_take_along_dim_with_mask": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32], i64),

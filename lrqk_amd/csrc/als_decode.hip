@@ -36,14 +36,28 @@ constexpr int kFinThreads = 256;
 // C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
 __device__ __forceinline__ int mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
 
+// Ring append folded into the Gram pass: slot `slot` (>= 0) of every head is the new token.  The
+// pass takes its K row from k_new and its token id from `token` instead of the buffers, and the
+// wave that owns the slot writes k_new, v_new and the id into them.
+struct GramAppend {
+  const void* k_new;  // [b][hkv][d]
+  const void* v_new;  // [b][hkv][d]
+  void* v_act;        // [bh][kprev_slots][d]
+  int32_t* idx_out;   // active_idx, writable
+  int slot;           // -1: nothing to append
+  int32_t token;
+  int hq, hkv;
+};
+
 // Partial layout per (head, split): 32*32 floats of A^T A (row stride 32) then 32 floats of
 // A^T w.  Rows/columns >= r are zero.
 template <typename T>
 __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restrict__ a_k, int64_t head_stride,
                                                                 int64_t a_rows, const int32_t* __restrict__ active_idx,
-                                                                int64_t idx_stride, const T* __restrict__ k_prev,
+                                                                int64_t idx_stride, T* k_prev,
                                                                 int kprev_slots, int n, const T* __restrict__ q, int r,
-                                                                int d, int lpr_log2, float* __restrict__ part, int S) {
+                                                                int d, int lpr_log2, float* __restrict__ part, int S,
+                                                                GramAppend ap) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float w_all[kGramWaves][kGramChunk];
   __shared__ float red[kGramWaves][kGramNe];
@@ -63,6 +77,11 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
   const T* A = a_k + (int64_t)h * head_stride;
   const T* Kp = k_prev + (int64_t)h * kprev_slots * d;
   const int col = lane & 31, khalf = lane >> 5;
+  const T* knew_h = Kp;
+  if (ap.slot >= 0) {
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    knew_h = (const T*)ap.k_new + ((int64_t)bb * ap.hkv + kvh) * d;
+  }
 
   float qf[VEC];
   {
@@ -84,7 +103,8 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
 #pragma unroll
     for (int g = 0; g < kGramChunk / 2; ++g) {
       const int t = min(c0 + 2 * g + khalf, n - 1);
-      src[g] = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      const int id = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      src[g] = t == ap.slot ? ap.token : id;
     }
     // K rows of the chunk -> w
     for (int base0 = 0; base0 < kGramChunk; base0 += 8 * gpw) {
@@ -92,7 +112,7 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int row = min(c0 + base0 + u * gpw + grp, n - 1);
-        kv[u].load(Kp + (int64_t)row * d + sub * VEC);
+        kv[u].load((row == ap.slot ? knew_h : Kp + (int64_t)row * d) + sub * VEC);
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -128,6 +148,17 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
     __syncthreads();  // before the next chunk overwrites w_s
   }
   racc += __shfl_xor(racc, 32, kWave);
+  if (ap.slot >= w0 && ap.slot < w1 && lane < lpr) {  // this wave owns the new token's slot
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    const int64_t so = ((int64_t)bb * ap.hkv + kvh) * d + lane * VEC;
+    const int64_t dof = ((int64_t)h * kprev_slots + ap.slot) * d + lane * VEC;
+    Vec16<T> kx, vx;
+    kx.load((const T*)ap.k_new + so);
+    vx.load((const T*)ap.v_new + so);
+    *reinterpret_cast<decltype(kx.raw)*>(k_prev + dof) = kx.raw;
+    *reinterpret_cast<decltype(vx.raw)*>((T*)ap.v_act + dof) = vx.raw;
+    if (lane == 0) ap.idx_out[(int64_t)h * idx_stride + ap.slot] = ap.token;
+  }
   // ---- cross-wave reduction through LDS
 #pragma unroll
   for (int v = 0; v < 16; ++v) red[wave][mfma_row(lane, v) * 32 + col] = acc[v];
@@ -562,7 +593,7 @@ template <typename T>
 static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
                            const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots, int n,
                            const void* q, const void* k_new, int b, int hq, int hkv, int r, int d, int max_iter,
-                           float tol, void* q_hat, void* k_hat, int64_t append_row, hipStream_t st) {
+                           float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, hipStream_t st) {
   constexpr int VEC = Vec16<T>::N;
   const int bh = b * hq;
   const int lpr = d / VEC;
@@ -593,8 +624,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
     solve_allowed = smem_solve;
   }
   hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kGramThreads), 0, st, (const T*)a_k,
-                     head_stride, a_rows, active_idx, idx_stride, (const T*)k_prev, kprev_slots, n, (const T*)q, r, d,
-                     lpr_log2, part, S);
+                     head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q, r, d,
+                     lpr_log2, part, S, ap);
   LRQK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const T*)b_q,
                      (const T*)b_k, part, S, (const T*)q, (const T*)k_new, hq, hkv, r, d, lpr_log2, max_iter, iter_out,
@@ -607,15 +638,11 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   return LRQK_OK;
 }
 
-}  // namespace lrqk
-
-using namespace lrqk;
-
-extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
-                               const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots,
-                               int n, const void* q, const void* k_new, int b, int hq, int hkv, int r, int d,
-                               int max_iter, float tol, void* q_hat, void* k_hat, int64_t append_row, int dtype,
-                               void* stream) {
+static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
+                              const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots, int n,
+                              const void* q, const void* k_new, int b, int hq, int hkv, int r, int d, int max_iter,
+                              float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, int dtype,
+                              hipStream_t st) {
   LRQK_REQUIRE(ctx && b_q && b_k && a_k && k_prev && q && k_new && q_hat && k_hat, LRQK_EINVAL, "null pointer");
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(b > 0 && hq > 0 && hkv > 0 && hq % hkv == 0 && (int64_t)b * hq <= 65535, LRQK_EINVAL,
@@ -630,11 +657,38 @@ extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, i
   if (max_iter < 1) max_iter = 1;
   LRQK_REQUIRE(max_iter <= LRQK_MAX_DECODE_ITERS, LRQK_ELIMIT, "max_iter=%d > %d", max_iter, LRQK_MAX_DECODE_ITERS);
   LRQK_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)k_prev % 16 == 0), LRQK_EINVAL, "pointers must be 16-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
   if (dtype == LRQK_F32)
     return als_decode_impl<float>(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q,
-                                  k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, st);
+                                  k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, st);
   return als_decode_impl<bf16_t>(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q,
-                                 k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, st);
+                                 k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, st);
 }
 
+// The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
+// into its first kernel (same result as lrqk_append_token followed by lrqk_als_decode).
+int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
+                      int64_t idx_stride, void* k_act, void* v_act, int n_slots, const void* q, const void* k_new,
+                      const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
+                      void* k_hat, int64_t append_row, int slot, int32_t token, int dtype, hipStream_t st) {
+  LRQK_REQUIRE(active_idx && v_act && v_new, LRQK_EINVAL, "null pointer");
+  LRQK_REQUIRE(slot >= 0 && slot < n_slots, LRQK_EINVAL, "slot=%d outside 0..%d", slot, n_slots);
+  LRQK_REQUIRE(((uintptr_t)k_new % 16 == 0) && ((uintptr_t)v_new % 16 == 0) && ((uintptr_t)v_act % 16 == 0), LRQK_EINVAL,
+               "pointers must be 16-byte aligned");
+  GramAppend ap{k_new, v_new, v_act, active_idx, slot, token, hq, hkv};
+  return als_decode_checked(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_act, n_slots, n_slots, q, k_new, b,
+                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, dtype, st);
+}
+
+}  // namespace lrqk
+
+using namespace lrqk;
+
+extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
+                               const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots,
+                               int n, const void* q, const void* k_new, int b, int hq, int hkv, int r, int d,
+                               int max_iter, float tol, void* q_hat, void* k_hat, int64_t append_row, int dtype,
+                               void* stream) {
+  GramAppend ap{nullptr, nullptr, nullptr, nullptr, -1, 0, hq, hkv};
+  return als_decode_checked(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q, k_new, b,
+                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, dtype, (hipStream_t)stream);
+}

@@ -92,11 +92,18 @@ extern "C" int lrqk_timing_enable(lrqk_ctx* ctx, int max_launches) {
     delete[] ctx->tev;
     ctx->tev = nullptr;
   }
-  ctx->tev_pairs = ctx->tev_used = 0;
+  ctx->tev_pairs = ctx->tev_used = ctx->tev_seen = 0;
   if (max_launches == 0) return LRQK_OK;
   ctx->tev = new hipEvent_t[2 * (size_t)max_launches];
   for (int i = 0; i < 2 * max_launches; ++i) LRQK_HIP_CHECK(hipEventCreate(&ctx->tev[i]));
   ctx->tev_pairs = max_launches;
+  return LRQK_OK;
+}
+
+extern "C" int lrqk_timing_stride(lrqk_ctx* ctx, int every) {
+  LRQK_REQUIRE(ctx != nullptr && every >= 1, LRQK_EINVAL, "bad arguments");
+  ctx->tev_every = every;
+  ctx->tev_seen = 0;
   return LRQK_OK;
 }
 

@@ -64,6 +64,8 @@ struct lrqk_ctx {
   hipEvent_t* tev = nullptr;
   int tev_pairs = 0;   // capacity in pairs
   int tev_used = 0;    // pairs recorded since the last read
+  int tev_every = 1;   // only every n-th launch is bracketed (the event packets cost a few us each)
+  int tev_seen = 0;    // launches seen since timing was enabled
   int sel_bh = 0;      // head count the selector state (t_low, counters) was initialised for
   int last_short = 0, last_overflow = 0;  // split of the rescans seen by the last lrqk_select_stats
 };
@@ -74,6 +76,12 @@ namespace lrqk {
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st);
+// The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
+// into its first kernel.
+int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
+                      int64_t idx_stride, void* k_act, void* v_act, int n_slots, const void* q, const void* k_new,
+                      const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
+                      void* k_hat, int64_t append_row, int slot, int32_t token, int dtype, hipStream_t st);
 // Miss fetch overlapped with the attention over the slots that stay resident (one launch), then
 // the attention over the refetched slots and the merge (second launch).
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,

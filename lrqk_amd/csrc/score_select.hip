@@ -790,7 +790,7 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
                                        (int)smem));
     smem_allowed = smem;
   }
-  const bool timed = ctx->tev && ctx->tev_used < ctx->tev_pairs;
+  const bool timed = ctx->tev && ctx->tev_used < ctx->tev_pairs && (ctx->tev_seen++ % ctx->tev_every) == 0;
   if (timed) LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used], st));
   dim3 grid((unsigned)((m + kFiltRows - 1) / kFiltRows), (unsigned)bh);
   hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), 0, st, (const T*)a_k, head_stride,

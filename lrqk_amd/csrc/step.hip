@@ -28,16 +28,16 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   int32_t* mcount = miss_count ? miss_count : miss_slots + (size_t)bh * topk;
   uint8_t* ev = evict ? evict : (uint8_t*)(miss_slots + (size_t)bh * topk + bh);
 
-  if ((rc = lrqk_append_token(k_new, v_new, k_act, v_act, n, topk + ring_slot, active_idx, n, token, b, hq, hkv, d, dtype,
-                              stream)))
+  // ring append folded into the first kernel of the factor update; the flush of a full ring
+  // (which reads the slot just written) follows it
+  if ((rc = als_decode_append(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq, hkv,
+                              r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, dtype,
+                              (hipStream_t)stream)))
     return rc;
   if (flush_row0 >= 0) {
     if ((rc = lrqk_flush_ring(k_act, v_act, n, topk, lite, kv_store, cap, flush_row0, b, hq, hkv, d, dtype, stream)))
       return rc;
   }
-  if ((rc = lrqk_als_decode(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, n, n, q, k_new, b, hq, hkv, r, d,
-                            max_iter, tol, q_hat, k_hat, token, dtype, stream)))
-    return rc;
   rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, active_idx, n, ev,
                          miss_slots, mcount, no_hit_miss, (hipStream_t)stream);
   if (rc < 0) return rc;

@@ -52,8 +52,10 @@ class Workspace:
         hipMemcpyAsync on a side stream, as the reference stages its misses."""
         check(_lib.load().lrqk_ctx_set_fetch_mode(self.handle, {"direct": 0, "staged": 1}[mode], int(host_threads)))
 
-    def timing_enable(self, max_launches: int):
+    def timing_enable(self, max_launches: int, every: int = 1):
+        """Bracket (every `every`-th of) the next proxy-score launches with HIP events, at most max_launches."""
         check(_lib.load().lrqk_timing_enable(self._h, max_launches))
+        check(_lib.load().lrqk_timing_stride(self._h, every))
 
     def timing_read(self):
         """(summed proxy-score kernel time in ms, launches) since the last read."""
