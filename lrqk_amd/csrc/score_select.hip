@@ -146,7 +146,14 @@ __device__ __forceinline__ uint32_t rescaled_bound(uint32_t t_low, float q_norm_
 
 // --------------------------------------------------------------------------- score + filter
 constexpr int kFiltThreads = 256;
-constexpr int kFiltRPT = 8;  // rows per thread
+#ifndef LRQK_FILT_RPT
+#define LRQK_FILT_RPT 8
+#endif
+constexpr int kFiltRPT = LRQK_FILT_RPT;  // rows per thread and tile
+#ifndef LRQK_FILT_TILES
+#define LRQK_FILT_TILES 2
+#endif
+constexpr int kFiltTiles = LRQK_FILT_TILES;  // tiles per workgroup: one global list reservation for all of them
 constexpr int kFiltRows = kFiltThreads * kFiltRPT;
 
 template <typename T, int R>
@@ -154,7 +161,8 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
                                                                     const T* __restrict__ q_hat, int64_t m, int r,
                                                                     int round_bf16, SelState st,
                                                                     uint2* __restrict__ cand, int cand_cap) {
-  __shared__ uint2 lc[kFiltRows];
+  extern __shared__ __align__(16) uint32_t filt_dyn[];
+  uint2* lc = reinterpret_cast<uint2*>(filt_dyn);  // [kFiltRows * kFiltTiles]
   __shared__ int l_count, g_base;
   const int h = blockIdx.y;
   const int tid = threadIdx.x, lane = lane_id();
@@ -165,39 +173,46 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
   rs.init(q_hat + (int64_t)h * r, r, round_bf16);
   const uint32_t t_prev = st.t_low[h];
   const float qn_prev = st.q_norm[h];
-  const int64_t base = (int64_t)blockIdx.x * kFiltRows;
-  // pure streaming part: 8 rows per thread, loads unconditional (clamped), hits kept as a mask;
-  // the bound is derived after the row loads were issued so that its own loads overlap them
-  uint32_t keys[kFiltRPT];
-#pragma unroll
-  for (int it = 0; it < kFiltRPT; ++it) {
-    const int64_t i = base + it * kFiltThreads + tid;
-    keys[it] = score_key(rs.score(A, min(i, m - 1)));
-  }
-  const float qn = rs.q_norm();
-  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn);
-  if (tid == 0 && blockIdx.x == 0) {
-    st.t_used[h] = tl;
-    st.q_cur[h] = qn;
-  }
-  uint32_t mask = 0;
-#pragma unroll
-  for (int it = 0; it < kFiltRPT; ++it) {
-    const int64_t i = base + it * kFiltThreads + tid;
-    if (i < m && keys[it] >= tl) mask |= 1u << it;
-  }
-  // one LDS allocation per wave for all of its hits
-  const int cnt = __popc(mask);
-  const int incl = wave_inclusive_sum(cnt);
-  const int wtot = __shfl(incl, kWave - 1, kWave);
-  if (wtot) {
-    int wbase = 0;
-    if (lane == kWave - 1) wbase = atomicAdd(&l_count, wtot);
-    wbase = __shfl(wbase, kWave - 1, kWave);
-    int pos = wbase + incl - cnt;
+  uint32_t tl = 0;
+#pragma unroll 1
+  for (int tile = 0; tile < kFiltTiles; ++tile) {
+    const int64_t base = ((int64_t)blockIdx.x * kFiltTiles + tile) * kFiltRows;
+    if (base >= m) break;
+    // pure streaming part: loads unconditional (clamped), hits kept as a mask; the bound is
+    // derived after the first row loads were issued so that its own loads overlap them
+    uint32_t keys[kFiltRPT];
 #pragma unroll
     for (int it = 0; it < kFiltRPT; ++it) {
-      if ((mask >> it) & 1u) lc[pos++] = make_uint2(keys[it], (uint32_t)(base + it * kFiltThreads + tid));
+      const int64_t i = base + it * kFiltThreads + tid;
+      keys[it] = score_key(rs.score(A, min(i, m - 1)));
+    }
+    if (tile == 0) {
+      const float qn = rs.q_norm();
+      tl = rescaled_bound(t_prev, qn_prev, qn);
+      if (tid == 0 && blockIdx.x == 0) {
+        st.t_used[h] = tl;
+        st.q_cur[h] = qn;
+      }
+    }
+    uint32_t mask = 0;
+#pragma unroll
+    for (int it = 0; it < kFiltRPT; ++it) {
+      const int64_t i = base + it * kFiltThreads + tid;
+      if (i < m && keys[it] >= tl) mask |= 1u << it;
+    }
+    // one LDS allocation per wave for all of its hits
+    const int cnt = __popc(mask);
+    const int incl = wave_inclusive_sum(cnt);
+    const int wtot = __shfl(incl, kWave - 1, kWave);
+    if (wtot) {
+      int wbase = 0;
+      if (lane == kWave - 1) wbase = atomicAdd(&l_count, wtot);
+      wbase = __shfl(wbase, kWave - 1, kWave);
+      int pos = wbase + incl - cnt;
+#pragma unroll
+      for (int it = 0; it < kFiltRPT; ++it) {
+        if ((mask >> it) & 1u) lc[pos++] = make_uint2(keys[it], (uint32_t)(base + it * kFiltThreads + tid));
+      }
     }
   }
   __syncthreads();
@@ -792,8 +807,15 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
   }
   const bool timed = ctx->tev && ctx->tev_used < ctx->tev_pairs && (ctx->tev_seen++ % ctx->tev_every) == 0;
   if (timed) LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used], st));
-  dim3 grid((unsigned)((m + kFiltRows - 1) / kFiltRows), (unsigned)bh);
-  hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), 0, st, (const T*)a_k, head_stride,
+  constexpr size_t filt_smem = (size_t)kFiltRows * kFiltTiles * sizeof(uint2);
+  static bool filt_attr = false;
+  if (!filt_attr && filt_smem > 48 * 1024) {
+    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)score_filter_kernel<T, R>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)filt_smem));
+    filt_attr = true;
+  }
+  dim3 grid((unsigned)((m + (int64_t)kFiltRows * kFiltTiles - 1) / ((int64_t)kFiltRows * kFiltTiles)), (unsigned)bh);
+  hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), filt_smem, st, (const T*)a_k, head_stride,
                      (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap);
   LRQK_HIP_CHECK(hipGetLastError());
   if (timed) {
