@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the proxy-score kernel read from hardware counters (rocprofv3 --pmc FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB device copy: x2.000 and x1.000), per
 # workload at its default context.  The summary of those runs is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"llama8b_128k_bf16": (131206.3 * 2.000 + 1106.6 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"llama8b_128k_bf16": (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
 
 
 def parse():
