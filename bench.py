@@ -50,9 +50,14 @@ def parse():
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
                    help="miss fetch: the kernel reads the pinned store itself, or host gather + hipMemcpyAsync")
-    p.add_argument("--mode", default="decode", choices=["decode", "prefill_als"],
+    p.add_argument("--mode", default="decode", choices=["decode", "prefill_als", "decoder"],
                    help="prefill_als: time the prefill factorisation alone (workload llama8b_32k_prefill_als unless "
-                        "--workload is given); a step is one whole factorisation")
+                        "--workload is given); a step is one whole factorisation.  decoder: greedy decoding with a "
+                        "full Llama-3-8B-shaped stack around the cache (end-to-end tokens/s)")
+    p.add_argument("--layers", type=int, default=32, help="decoder mode: number of layers")
+    p.add_argument("--batch", type=int, default=4, help="decoder mode: sequences")
+    p.add_argument("--prompt", type=int, default=65536, help="decoder mode: prompt tokens per sequence")
+    p.add_argument("--new-tokens", type=int, default=128, help="decoder mode: tokens decoded per sequence")
     p.add_argument("--calib-copy-mb", type=int, default=0,
                    help="after the timed region, run one plain device copy of this many MiB (a known-size "
                         "kernel to scale hardware counters by)")
@@ -137,6 +142,42 @@ def prefill_als(a):
     print(json.dumps(out))
 
 
+def decoder(a):
+    """End-to-end greedy decoding: random-init Llama-3-8B-shaped stack, random token ids, LRQK cache in
+    every layer (r 32, k 2048, lite 64).  tokens/s = batch * new_tokens / wall time of the decode phase."""
+    from lrqk_amd.decoder import LlamaShapeDecoder, DecoderConfig
+    cfg = DecoderConfig(layers=a.layers)
+    dev = torch.device("cuda:0")
+    t0 = time.perf_counter()
+    model = LlamaShapeDecoder(cfg, torch.bfloat16, dev, seed=a.seed)
+    model.progress = lambda msg: print(msg, file=sys.stderr, flush=True)
+    g = torch.Generator(device=dev).manual_seed(a.seed + 1)
+    ids = torch.randint(0, cfg.vocab, (a.batch, a.prompt), generator=g, device=dev)
+    cache = model.new_cache(r=32, num_active_tokens=2048, lite_tokens=64, max_iter=(2, 2), tol=(1e-2, 1e-2))
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    toks, t_prefill, t_decode, steps = model.generate(ids, a.new_tokens, cache)
+    n_dec = a.new_tokens - 1
+    tps = a.batch * n_dec / t_decode
+    miss = sel = 0
+    for li in range(cfg.layers):
+        m_, s_, _ = cache.lwattn[li].miss_stats()
+        miss += m_
+        sel += s_
+    out = {"metric": "lrqk_decoder_tokens_per_s", "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1,
+           "steps": n_dec, "warmup": 0, "ms_per_step": round(t_decode / n_dec * 1e3, 3), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": f"llama3_8b_shape_decoder@{a.prompt}", "layers": cfg.layers, "batch": a.batch,
+                      "prompt_tokens": a.prompt, "new_tokens": a.new_tokens, "r": 32, "k": 2048, "lite": 64,
+                      "max_iter": [2, 2]},
+           "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3), "setup_s": round(setup_s, 2),
+           "reference_style_tokens_per_s": round(a.batch * len(steps) / max(sum(steps), 1e-9), 2),
+           "us_per_layer_step": round(t_decode / n_dec / cfg.layers * 1e6, 1),
+           "last_step_hit_rate": round(1.0 - miss / max(sel, 1), 4),
+           "roofline": None, "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -152,6 +193,8 @@ def main():
     _lib.load()  # fail loudly if the HIP library is missing
     if a.mode == "prefill_als":
         return prefill_als(a)
+    if a.mode == "decoder":
+        return decoder(a)
 
     dev = torch.device("cuda:0")
     w = synth.WORKLOADS[a.workload]
