@@ -20,18 +20,17 @@
 
 #include "common.hpp"
 #include "ctx.hpp"
+#include "als_finish.hpp"
 
 namespace lrqk {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kAlsMaxR = 32;  // one 32x32 MFMA tile
 constexpr int kGramThreads = 256;
 constexpr int kGramWaves = kGramThreads / kWave;
 constexpr int kGramChunk = 32;  // tokens per wave per chunk = 16 MFMA steps
 constexpr int kGramNe = 32 * 32 + 32;
 constexpr int kSolveThreads = 256;
-constexpr int kFinThreads = 256;
 
 // C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
 __device__ __forceinline__ int mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
@@ -438,162 +437,17 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
   }
 }
 
-// One workgroup per head.  B_Q and B_K of the head are held in registers as 16-byte vectors
-// (vector vi = tid + 256 u covers row vi >> vshift, columns (vi & (vpr-1)) * VEC ..).
 template <typename T>
-__global__ __launch_bounds__(kFinThreads) void als_finish_kernel(T* __restrict__ b_q, T* __restrict__ b_k,
-                                                                 const T* __restrict__ q, const T* __restrict__ k_new,
-                                                                 const float* __restrict__ iter_out,
-                                                                 const float* __restrict__ deltas, int bh, int hq,
-                                                                 int hkv, int r, int d, int vshift, int max_iter,
-                                                                 float tol, T* __restrict__ q_hat_out,
-                                                                 T* __restrict__ k_hat_out, T* __restrict__ a_k,
-                                                                 int64_t head_stride, int64_t append_row) {
-  constexpr int VEC = Vec16<T>::N;
-  constexpr int kMaxVec = 8;  // vectors per thread per matrix: r * d / VEC <= 2048
-  __shared__ float hat[2][kAlsMaxR];
-  __shared__ float err[2][256];
-  __shared__ float red[kFinThreads / kWave][2][256];
-  __shared__ float dsum[LRQK_MAX_DECODE_ITERS];
-  __shared__ int s_it;
-  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
-  const int h = blockIdx.x;
-  const int b = h / hq, head = h % hq;
-  const int kvh = head / (hq / hkv);
-  const int vpr = 1 << vshift;  // vectors per row, a power of two <= 64
-  const int nvec = r << vshift;
-  // B tiles -> registers (independent loads, issued first)
-  Vec16<T> vq[kMaxVec], vk[kMaxVec];
-#pragma unroll
-  for (int u = 0; u < kMaxVec; ++u) {
-    const int vi = min(tid + u * kFinThreads, nvec - 1);
-    vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
-    vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
-  }
-  const float qreg = ld_f32<T>(q, (int64_t)h * d + min(tid, d - 1));
-  const float kreg = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + min(tid, d - 1));
-  // batch-wide stopping test: wave `it` adds the heads' terms of iteration `it` in a fixed
-  // lane-strided order (the loads of one wave are in flight together)
-  for (int it = wave; it < max_iter; it += kFinThreads / kWave) {
-    float sacc = 0.0f;
-    for (int hh = lane; hh < bh; hh += kWave) sacc += deltas[(int64_t)hh * max_iter + it];
-    sacc = wave_sum(sacc);
-    if (lane == 0) dsum[it] = sacc;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int chosen = max_iter - 1;
-    for (int it = 0; it < max_iter; ++it) {
-      if (dsum[it] / (float)((int64_t)bh * r) < tol) {
-        chosen = it;
-        break;
-      }
-    }
-    s_it = chosen;
-  }
-  __syncthreads();
-  const float* o = iter_out + ((int64_t)h * max_iter + s_it) * 2 * r;
-  if (tid < 2 * r) hat[tid >= r ? 1 : 0][tid >= r ? tid - r : tid] = o[tid];
-  __syncthreads();
-  // column sums  sum_i hat[i] B[i][c]  for this thread's column group, both matrices
-  const int cg = tid & (vpr - 1);  // vpr divides 256, so the column group is fixed per thread
-  float pq[VEC], pk[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) pq[e] = pk[e] = 0.0f;
-#pragma unroll
-  for (int u = 0; u < kMaxVec; ++u) {
-    const int vi = tid + u * kFinThreads;
-    if (vi < nvec) {
-      const int row = vi >> vshift;
-      float fq[VEC], fk[VEC];
-      vq[u].unpack(fq);
-      vk[u].unpack(fk);
-      const float hq_ = hat[0][row], hk_ = hat[1][row];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        pq[e] = fmaf(hq_, fq[e], pq[e]);
-        pk[e] = fmaf(hk_, fk[e], pk[e]);
-      }
-    }
-  }
-  // lanes of a wave that share a column group differ in the lane-id bits >= vshift
-  for (int off = vpr; off < kWave; off <<= 1) {
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      pq[e] += __shfl_xor(pq[e], off, kWave);
-      pk[e] += __shfl_xor(pk[e], off, kWave);
-    }
-  }
-  if (lane < vpr) {
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      red[wave][0][cg * VEC + e] = pq[e];
-      red[wave][1][cg * VEC + e] = pk[e];
-    }
-  }
-  __syncthreads();
-  float en0 = 0.0f, en1 = 0.0f;
-  if (tid < d) {
-    float eq = -qreg, ek = -kreg;
-#pragma unroll
-    for (int w = 0; w < kFinThreads / kWave; ++w) {
-      eq += red[w][0][tid];
-      ek += red[w][1][tid];
-    }
-    err[0][tid] = eq;
-    err[1][tid] = ek;
-    en0 = eq * eq;
-    en1 = ek * ek;
-  }
-  en0 = wave_sum(en0);
-  en1 = wave_sum(en1);
-  __syncthreads();  // everyone is done reading red
-  if (lane == 0) {
-    red[wave][0][0] = en0;
-    red[wave][1][0] = en1;
-  }
-  __syncthreads();
-  float e2q = 0.0f, e2k = 0.0f, hnq = 0.0f, hnk = 0.0f;
-  for (int w = 0; w < kFinThreads / kWave; ++w) {
-    e2q += red[w][0][0];
-    e2k += red[w][1][0];
-  }
-  for (int i = 0; i < r; ++i) {
-    hnq = fmaf(hat[0][i], hat[0][i], hnq);
-    hnk = fmaf(hat[1][i], hat[1][i], hnk);
-  }
-  // dB = hat^T e : |dB|^2 = |hat|^2 |e|^2 ; hat dB = |hat|^2 e : |hat dB|^2 = |hat|^4 |e|^2
-  const float lrq = (hnq * e2q) / (hnq * hnq * e2q + 1e-6f);
-  const float lrk = (hnk * e2k) / (hnk * hnk * e2k + 1e-6f);
-#pragma unroll
-  for (int u = 0; u < kMaxVec; ++u) {
-    const int vi = tid + u * kFinThreads;
-    if (vi < nvec) {
-      const int row = vi >> vshift;
-      float fq[VEC], fk[VEC];
-      vq[u].unpack(fq);
-      vk[u].unpack(fk);
-      const float sq = lrq * hat[0][row], sk = lrk * hat[1][row];
-      const int64_t off = (int64_t)h * r * d + (int64_t)vi * VEC;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        st_f32<T>(b_q, off + e, fq[e] - sq * err[0][cg * VEC + e]);
-        st_f32<T>(b_k, off + e, fk[e] - sk * err[1][cg * VEC + e]);
-      }
-    }
-  }
-  if (tid < r) {
-    st_f32<T>(q_hat_out, (int64_t)h * r + tid, hat[0][tid]);
-    st_f32<T>(k_hat_out, (int64_t)h * r + tid, hat[1][tid]);
-    if (append_row >= 0) st_f32<T>(a_k, (int64_t)h * head_stride + append_row * r + tid, hat[1][tid]);
-  }
+__global__ __launch_bounds__(kFinThreads) void als_finish_kernel(FinishArgs fa) {
+  als_finish_body<T>(fa, blockIdx.x);
 }
 
 template <typename T>
 static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
                            const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots, int n,
                            const void* q, const void* k_new, int b, int hq, int hkv, int r, int d, int max_iter,
-                           float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, hipStream_t st) {
+                           float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, bool defer_finish,
+                           hipStream_t st) {
   constexpr int VEC = Vec16<T>::N;
   const int bh = b * hq;
   const int lpr = d / VEC;
@@ -631,9 +485,17 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                      (const T*)b_k, part, S, (const T*)q, (const T*)k_new, hq, hkv, r, d, lpr_log2, max_iter, iter_out,
                      deltas);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((als_finish_kernel<T>), dim3((unsigned)bh), dim3(kFinThreads), 0, st, (T*)b_q, (T*)b_k,
-                     (const T*)q, (const T*)k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol,
-                     (T*)q_hat, (T*)k_hat, (T*)a_k, head_stride, append_row);
+  FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
+                head_stride, append_row};
+  if (defer_finish) {
+    // the caller lets later launches of the step absorb the finish stage (flush_pending_finish otherwise)
+    ctx->fin = fa;
+    ctx->fin_dtype = sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16;
+    ctx->fin_pending = true;   // B update, outputs and the A_K row still to be done
+    ctx->qhat_pending = true;  // q_hat has not been written yet: consumers take the iterate from iter_out
+    return LRQK_OK;
+  }
+  hipLaunchKernelGGL((als_finish_kernel<T>), dim3((unsigned)bh), dim3(kFinThreads), 0, st, fa);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -641,8 +503,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
 static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
                               const int32_t* active_idx, int64_t idx_stride, const void* k_prev, int kprev_slots, int n,
                               const void* q, const void* k_new, int b, int hq, int hkv, int r, int d, int max_iter,
-                              float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, int dtype,
-                              hipStream_t st) {
+                              float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, bool defer_finish,
+                              int dtype, hipStream_t st) {
   LRQK_REQUIRE(ctx && b_q && b_k && a_k && k_prev && q && k_new && q_hat && k_hat, LRQK_EINVAL, "null pointer");
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(b > 0 && hq > 0 && hkv > 0 && hq % hkv == 0 && (int64_t)b * hq <= 65535, LRQK_EINVAL,
@@ -659,9 +521,9 @@ static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, in
   LRQK_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)k_prev % 16 == 0), LRQK_EINVAL, "pointers must be 16-byte aligned");
   if (dtype == LRQK_F32)
     return als_decode_impl<float>(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q,
-                                  k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, st);
+                                  k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, defer_finish, st);
   return als_decode_impl<bf16_t>(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q,
-                                 k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, st);
+                                 k_new, b, hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, defer_finish, st);
 }
 
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
@@ -669,14 +531,28 @@ static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, in
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
                       int64_t idx_stride, void* k_act, void* v_act, int n_slots, const void* q, const void* k_new,
                       const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
-                      void* k_hat, int64_t append_row, int slot, int32_t token, int dtype, hipStream_t st) {
+                      void* k_hat, int64_t append_row, int slot, int32_t token, bool defer_finish, int dtype,
+                      hipStream_t st) {
   LRQK_REQUIRE(active_idx && v_act && v_new, LRQK_EINVAL, "null pointer");
   LRQK_REQUIRE(slot >= 0 && slot < n_slots, LRQK_EINVAL, "slot=%d outside 0..%d", slot, n_slots);
   LRQK_REQUIRE(((uintptr_t)k_new % 16 == 0) && ((uintptr_t)v_new % 16 == 0) && ((uintptr_t)v_act % 16 == 0), LRQK_EINVAL,
                "pointers must be 16-byte aligned");
   GramAppend ap{k_new, v_new, v_act, active_idx, slot, token, hq, hkv};
   return als_decode_checked(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_act, n_slots, n_slots, q, k_new, b,
-                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, dtype, st);
+                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, defer_finish, dtype, st);
+}
+
+// Runs a deferred finish stage as its own launch (when no later launch of the step took it over).
+int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st) {
+  if (!ctx->fin_pending) return LRQK_OK;
+  ctx->fin_pending = false;
+  ctx->qhat_pending = false;
+  if (ctx->fin_dtype == LRQK_F32)
+    hipLaunchKernelGGL((als_finish_kernel<float>), dim3((unsigned)ctx->fin.bh), dim3(kFinThreads), 0, st, ctx->fin);
+  else
+    hipLaunchKernelGGL((als_finish_kernel<bf16_t>), dim3((unsigned)ctx->fin.bh), dim3(kFinThreads), 0, st, ctx->fin);
+  LRQK_HIP_CHECK(hipGetLastError());
+  return LRQK_OK;
 }
 
 }  // namespace lrqk
@@ -690,5 +566,5 @@ extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, i
                                void* stream) {
   GramAppend ap{nullptr, nullptr, nullptr, nullptr, -1, 0, hq, hkv};
   return als_decode_checked(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q, k_new, b,
-                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, dtype, (hipStream_t)stream);
+                            hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, false, dtype, (hipStream_t)stream);
 }

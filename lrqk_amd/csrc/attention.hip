@@ -13,6 +13,7 @@
 #include "common.hpp"
 #include "ctx.hpp"
 #include "rows.hpp"
+#include "als_finish.hpp"
 
 namespace lrqk {
 
@@ -189,14 +190,21 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
 }
 
 // Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their
-// slots; the others run the partial attention over the slots that are not being replaced.
+// slots; the next S run the partial attention over the slots that are not being replaced; one
+// more (with_finish) runs the finish stage of this step's factor update, which nothing in this
+// launch depends on.  The copy is bound by the host link, so the other roles ride along.
 template <typename T>
 __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     const uint4* __restrict__ store, int64_t cap, int32_t* __restrict__ hit, int64_t hit_stride,
     const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
     int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
-    int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S) {
+    int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
+    FinishArgs fa) {
   const int h = blockIdx.y;
+  if (with_finish && (int)blockIdx.x == n_fetch + S) {
+    als_finish_body<T>(fa, h);
+    return;
+  }
   if ((int)blockIdx.x < n_fetch) {
     fetch_rows_body(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k,
                     h, blockIdx.x, n_fetch);
@@ -337,10 +345,20 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   const int n_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));  // sized for a miss rate of 1/8
   if ((rc = ctx->attn_part.ensure((size_t)bh * (S + 1) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
-  hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S), (unsigned)bh), dim3(kAttnThreads), 0,
-                     st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count, evict, hq, hkv, cpr, k,
-                     n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2, scale_log2e,
-                     (float*)ctx->attn_part.p, S);
+  static_assert(kAttnThreads == kFinThreads, "the finish stage rides in an attention-sized workgroup");
+  int with_finish = 0;
+  if (ctx->fin_pending) {
+    if (ctx->fin.bh == bh && ctx->fin_dtype == (sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16) && !ctx->qhat_pending) {
+      with_finish = 1;
+      ctx->fin_pending = false;
+    } else if ((rc = flush_pending_finish(ctx, st))) {
+      return rc;
+    }
+  }
+  hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish), (unsigned)bh),
+                     dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
+                     evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
+                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin);
   LRQK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (float*)ctx->attn_part.p,
                      S, S + 1, d, (T*)out, (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, lpr_log2,

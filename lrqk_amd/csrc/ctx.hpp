@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
+#include "als_finish.hpp"
 
 namespace lrqk {
 
@@ -52,6 +53,11 @@ struct lrqk_ctx {
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
   lrqk::DevBuf misc;        // evict mask, miss lists, counters of the fused step
+  // finish stage of the factor update deferred into later launches of the decode step
+  lrqk::FinishArgs fin{};
+  int fin_dtype = 0;
+  bool fin_pending = false;   // B update / outputs / A_K row not done yet
+  bool qhat_pending = false;  // q_hat not written yet
   // staged miss fetch: pinned host staging, its device twin, side stream and event (created on first use)
   lrqk::DevBuf stage_dev;
   void* stage_host = nullptr;
@@ -81,7 +87,10 @@ int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
                       int64_t idx_stride, void* k_act, void* v_act, int n_slots, const void* q, const void* k_new,
                       const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
-                      void* k_hat, int64_t append_row, int slot, int32_t token, int dtype, hipStream_t st);
+                      void* k_hat, int64_t append_row, int slot, int32_t token, bool defer_finish, int dtype,
+                      hipStream_t st);
+// Runs a deferred finish stage as its own launch (no-op if none is pending).
+int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st);
 // Miss fetch overlapped with the attention over the slots that stay resident (one launch), then
 // the attention over the refetched slots and the merge (second launch).
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,

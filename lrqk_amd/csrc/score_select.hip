@@ -22,6 +22,7 @@
 //                  key == T) and, when asked, diffed in place against the resident set.
 #include "common.hpp"
 #include "ctx.hpp"
+#include "als_finish.hpp"
 
 namespace lrqk {
 
@@ -41,6 +42,41 @@ struct RowScorer {
 #pragma unroll
       for (int j = 0; j < R; ++j) qf[j] = ld_f32<T>(q_head, j);
     }
+  }
+  // the proxy query from a lane-distributed fp32 vector (lane j holds element j of an iterate of
+  // the factor update), rounded to the storage type and broadcast to every lane
+  __device__ __forceinline__ void init_from_lanes(float qv, int r_, int round_) {
+    qh = nullptr;
+    r = r_;
+    round_bf16 = round_;
+    if (sizeof(T) == 2) qv = round_to_bf16_f32(qv);
+    if (R > 0) {
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+        qf[j] = j < r_ ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qv), j)) : 0.0f;
+    }
+  }
+  // a row as 16-byte vectors (R > 0 only): requested now, scored later
+  struct Row {
+    Vec16<T> v[R / VEC > 0 ? R / VEC : 1];
+  };
+  __device__ __forceinline__ void load_row(const T* A, int64_t i, Row& row) const {
+    const T* p = A + i * R;
+#pragma unroll
+    for (int c = 0; c < R / VEC; ++c) row.v[c].load(p + c * VEC);
+  }
+  __device__ __forceinline__ float score_row(const Row& row) const {
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < R / VEC; ++c) {
+      float f[VEC];
+      row.v[c].unpack(f);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc = __builtin_fmaf(f[e], qf[c * VEC + e], acc);
+    }
+    if (round_bf16) acc = round_to_bf16_f32(acc);
+    if (acc == 0.0f) acc = 0.0f;
+    return acc;
   }
   __device__ __forceinline__ float q_norm() const {
     float s = 0.0f;
@@ -155,12 +191,25 @@ constexpr int kFiltRPT = LRQK_FILT_RPT;  // rows per thread and tile
 #endif
 constexpr int kFiltTiles = LRQK_FILT_TILES;  // tiles per workgroup: one global list reservation for all of them
 constexpr int kFiltRows = kFiltThreads * kFiltRPT;
+constexpr int kFiltMaxIt = 4;  // most iterations of the factor update whose pending iterate the filter can pick itself
+
+// Proxy query taken straight from the iterates of the factor update whose finish stage has not
+// run yet (iter_out == nullptr: q_hat is read instead).  Workgroup 0 of every head writes the
+// chosen, rounded iterate to q_hat_out.
+struct FilterQ {
+  const float* iter_out;  // [bh][max_iter][2r]
+  const float* deltas;    // [bh][max_iter]
+  int bh, max_iter;
+  float tol;
+  void* q_hat_out;        // [bh][r] storage dtype
+};
 
 template <typename T, int R>
 __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __restrict__ a_k, int64_t head_stride,
                                                                     const T* __restrict__ q_hat, int64_t m, int r,
                                                                     int round_bf16, SelState st,
-                                                                    uint2* __restrict__ cand, int cand_cap) {
+                                                                    uint2* __restrict__ cand, int cand_cap,
+                                                                    FilterQ fq) {
   extern __shared__ __align__(16) uint32_t filt_dyn[];
   uint2* lc = reinterpret_cast<uint2*>(filt_dyn);  // [kFiltRows * kFiltTiles]
   __shared__ int l_count, g_base;
@@ -170,21 +219,60 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
   RowScorer<T, R> rs;
   if (tid == 0) l_count = 0;
   __syncthreads();
-  rs.init(q_hat + (int64_t)h * r, r, round_bf16);
   const uint32_t t_prev = st.t_low[h];
   const float qn_prev = st.q_norm[h];
   uint32_t tl = 0;
+  // The small loads go first (memory returns in order: issued after the rows they would arrive
+  // last).  With a pending finish stage every wave fetches the stopping-test terms and element
+  // `lane` of every iterate, decides, and broadcasts the chosen iterate from its lanes (no barrier,
+  // no LDS); otherwise q_hat is read.
+  const bool pending = fq.iter_out != nullptr;
+  float sacc[kFiltMaxIt], oit[kFiltMaxIt];
+  if (pending) {
+    als_delta_sums<kFiltMaxIt>(fq.deltas, fq.bh, fq.max_iter, sacc);
+#pragma unroll
+    for (int it = 0; it < kFiltMaxIt; ++it)
+      oit[it] = fq.iter_out[((int64_t)h * fq.max_iter + min(it, fq.max_iter - 1)) * 2 * r + min(lane, r - 1)];
+  } else {
+    rs.init(q_hat + (int64_t)h * r, r, round_bf16);
+  }
 #pragma unroll 1
   for (int tile = 0; tile < kFiltTiles; ++tile) {
     const int64_t base = ((int64_t)blockIdx.x * kFiltTiles + tile) * kFiltRows;
     if (base >= m) break;
-    // pure streaming part: loads unconditional (clamped), hits kept as a mask; the bound is
-    // derived after the first row loads were issued so that its own loads overlap them
+    // pure streaming part: loads unconditional (clamped), hits kept as a mask
     uint32_t keys[kFiltRPT];
+    if constexpr (R > 0) {
+      // the first rows are requested before the pending iterate is resolved, so that its latency
+      // and theirs overlap
+      constexpr int kPre = 2;  // more would cost occupancy (16 registers per row)
+      typename RowScorer<T, R>::Row rows[kPre];
 #pragma unroll
-    for (int it = 0; it < kFiltRPT; ++it) {
-      const int64_t i = base + it * kFiltThreads + tid;
-      keys[it] = score_key(rs.score(A, min(i, m - 1)));
+      for (int it = 0; it < kPre; ++it) {
+        const int64_t i = base + it * kFiltThreads + tid;
+        rs.load_row(A, min(i, m - 1), rows[it]);
+      }
+      if (tile == 0 && pending) {
+        const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
+        float qv = oit[0];
+#pragma unroll
+        for (int it = 1; it < kFiltMaxIt; ++it) qv = chosen == it ? oit[it] : qv;
+        if (blockIdx.x == 0 && tid < r) st_f32<T>((T*)fq.q_hat_out, (int64_t)h * r + tid, qv);
+        rs.init_from_lanes(qv, r, round_bf16);
+      }
+#pragma unroll
+      for (int it = 0; it < kPre; ++it) keys[it] = score_key(rs.score_row(rows[it]));
+#pragma unroll
+      for (int it = kPre; it < kFiltRPT; ++it) {
+        const int64_t i = base + it * kFiltThreads + tid;
+        keys[it] = score_key(rs.score(A, min(i, m - 1)));
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kFiltRPT; ++it) {
+        const int64_t i = base + it * kFiltThreads + tid;
+        keys[it] = score_key(rs.score(A, min(i, m - 1)));
+      }
     }
     if (tile == 0) {
       const float qn = rs.q_norm();
@@ -814,9 +902,21 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)filt_smem));
     filt_attr = true;
   }
+  // a finish stage of the factor update that is still pending: the filter reads the iterate itself
+  FilterQ fq{nullptr, nullptr, 0, 0, 0.0f, nullptr};
+  if (ctx->qhat_pending) {
+    if (R > 0 && R <= 64 && ctx->fin.q_hat_out == q_hat && ctx->fin.r == r && ctx->fin.bh == bh &&
+        ctx->fin.max_iter <= kFiltMaxIt) {
+      fq = FilterQ{ctx->fin.iter_out, ctx->fin.deltas, bh, ctx->fin.max_iter, ctx->fin.tol, ctx->fin.q_hat_out};
+      ctx->qhat_pending = false;
+    } else {
+      int rcf = flush_pending_finish(ctx, st);
+      if (rcf) return rcf;
+    }
+  }
   dim3 grid((unsigned)((m + (int64_t)kFiltRows * kFiltTiles - 1) / ((int64_t)kFiltRows * kFiltTiles)), (unsigned)bh);
   hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), filt_smem, st, (const T*)a_k, head_stride,
-                     (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap);
+                     (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq);
   LRQK_HIP_CHECK(hipGetLastError());
   if (timed) {
     LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used + 1], st));

@@ -20,6 +20,7 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   const int bh = b * hq;
   const int n = topk + lite;
   int rc;
+  ctx->fin_pending = ctx->qhat_pending = false;  // nothing survives a call that failed half-way
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
   // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | evict u8 [bh][topk]
   if ((rc = ctx->misc.ensure((size_t)bh * topk * 5 + (size_t)bh * 4 + 64))) return rc;
@@ -28,11 +29,15 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   int32_t* mcount = miss_count ? miss_count : miss_slots + (size_t)bh * topk;
   uint8_t* ev = evict ? evict : (uint8_t*)(miss_slots + (size_t)bh * topk + bh);
 
+  // The finish stage of the factor update (B update, outputs, A_K row) is off the critical path: when
+  // the step ends with the fetch + attention launch it rides there, and the scan takes the proxy
+  // query from the iterates directly.  Any path that cannot absorb it flushes it as its own launch.
+  const bool defer_finish = attn_out != nullptr && !no_hit_miss && ctx->fetch_mode == 0;
   // ring append folded into the first kernel of the factor update; the flush of a full ring
   // (which reads the slot just written) follows it
   if ((rc = als_decode_append(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq, hkv,
-                              r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, dtype,
-                              (hipStream_t)stream)))
+                              r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, defer_finish,
+                              dtype, (hipStream_t)stream)))
     return rc;
   if (flush_row0 >= 0) {
     if ((rc = lrqk_flush_ring(k_act, v_act, n, topk, lite, kv_store, cap, flush_row0, b, hq, hkv, d, dtype, stream)))
@@ -41,12 +46,20 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, active_idx, n, ev,
                          miss_slots, mcount, no_hit_miss, (hipStream_t)stream);
   if (rc < 0) return rc;
+  if (ctx->qhat_pending) {  // no scan took the iterate over (cannot happen on the paths above; kept as a guard)
+    int rcf = flush_pending_finish(ctx, (hipStream_t)stream);
+    if (rcf) return rcf;
+  }
   if (rc == 0) {  // sizes outside the fused kernel's LDS budget: separate diff launch
     if (no_hit_miss)
       rc = lrqk_replace_all(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
     else
       rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
     if (rc) return rc;
+  }
+  if (!(attn_out && !no_hit_miss && ctx->fetch_mode == 0)) {
+    int rcf = flush_pending_finish(ctx, (hipStream_t)stream);
+    if (rcf) return rcf;
   }
   if (ctx->fetch_mode == 1) {
     if ((rc = lrqk_fetch_rows_staged(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv,
