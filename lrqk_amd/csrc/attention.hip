@@ -189,6 +189,111 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const T* __r
                        blockIdx.x);
 }
 
+// Fetch role of the decode step: like fetch_rows_body, and while a missed [K|V] row passes through
+// the registers of its 2*cpr lanes (cpr K chunks, then cpr V chunks) the lanes also form the row's
+// attention term, so the refetched slots never have to be read again.  The workgroup's rows are
+// merged into one (max, sum, acc) triple at `pout` (an empty triple if it had no row).
+template <typename T>
+__device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ store, int64_t cap,
+                                                     uint4* __restrict__ k_act, uint4* __restrict__ v_act, int n_slots,
+                                                     const int32_t* __restrict__ hit, int64_t hit_stride,
+                                                     const int32_t* __restrict__ miss_slots,
+                                                     const int32_t* __restrict__ miss_count, int hq, int hkv, int cpr,
+                                                     int k, int h, int blk, int nblk, const T* __restrict__ q, int d,
+                                                     float scale_log2e, float* __restrict__ pout) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ float accs[8][256 + 2];               // [row group][m, l, acc[d]] (at most 8 groups are merged at a time)
+  const int tid = threadIdx.x, lane = lane_id();
+  const int cnt = miss_count[h];
+  const int chunks = 2 * cpr;  // per store row; a power of two <= 64 here
+  const int rpb = kAttnThreads / chunks;
+  const int b = h / hq, head = h % hq;
+  const int kvh = head / (hq / hkv);
+  const int jl = tid / chunks, c = tid % chunks;
+  const bool is_k = c < cpr;
+  float qf[VEC];
+  {
+    Vec16<T> qv;
+    qv.load(q + (int64_t)h * d + (is_k ? c : 0) * VEC);
+    qv.unpack(qf);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) qf[e] *= scale_log2e;
+  }
+  AttnAcc<VEC> st;  // meaningful in the V lanes
+  st.init();
+  const int trips = (cnt + nblk * rpb - 1) / (nblk * rpb);  // uniform over the workgroup
+  for (int it = 0; it < trips; ++it) {
+    const int j = blk * rpb + jl + it * nblk * rpb;
+    bool ok = j < cnt;
+    int slot = 0;
+    int32_t tok = 0;
+    if (ok) {
+      slot = miss_slots[(int64_t)h * k + j];
+      ok = slot >= 0 && slot < k;
+      if (ok) {
+        tok = hit[(int64_t)h * hit_stride + slot];
+        ok = tok >= 0 && tok < cap;
+      }
+    }
+    uint4 val = make_uint4(0, 0, 0, 0);
+    if (ok) {
+      val = store[(((int64_t)b * hkv + kvh) * cap + tok) * chunks + c];
+      const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
+      if (is_k) k_act[dst + c] = val; else v_act[dst + (c - cpr)] = val;
+    }
+    Vec16<T> vv;
+    vv.raw = *reinterpret_cast<decltype(vv.raw)*>(&val);
+    float f[VEC];
+    vv.unpack(f);
+    float sc = 0.0f;
+    if (is_k) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sc = fmaf(f[e], qf[e], sc);
+    }
+    for (int off = 1; off < cpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);  // K lanes: the row's score
+    const float s_row = __shfl(sc, (lane & ~(chunks - 1)) | 0, kWave);           // first K lane of this row
+    if (!is_k) {
+      const float s_use = ok ? s_row : -INFINITY;
+      const float m_new = fmaxf(st.m, s_use);
+      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
+      const float p = (m_new == -INFINITY) ? 0.0f : exp2f(s_use - m_new);
+      st.l = st.l * alpha + p;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) st.acc[e] = st.acc[e] * alpha + p * f[e];
+      st.m = m_new;
+    }
+  }
+  // merge the row groups: V lane (jl, cv) owns columns cv*VEC .. of group jl
+  const int groups = rpb;  // <= 8 for rows of >= 512 bytes; larger counts are merged in rounds of 8
+  float M = -INFINITY, Lsum = 0.0f, col = 0.0f;  // thread t < d + 2 accumulates element t of the result
+  for (int g0 = 0; g0 < groups; g0 += 8) {
+    __syncthreads();
+    if (!is_k && jl >= g0 && jl < g0 + 8 && jl < groups) {
+      float* row = accs[jl - g0];
+      if (c == cpr) {
+        row[0] = st.m;
+        row[1] = st.l;
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) row[2 + (c - cpr) * VEC + e] = st.acc[e];
+    }
+    __syncthreads();
+    const int ng = min(8, groups - g0);
+    float Mg = M;
+    for (int g = 0; g < ng; ++g) Mg = fmaxf(Mg, accs[g][0]);
+    const float a_old = (Mg == -INFINITY) ? 0.0f : exp2f(M - Mg);
+    Lsum *= a_old;
+    col *= a_old;
+    for (int g = 0; g < ng; ++g) {
+      const float fg = (Mg == -INFINITY || accs[g][0] == -INFINITY) ? 0.0f : exp2f(accs[g][0] - Mg);
+      Lsum = fmaf(accs[g][1], fg, Lsum);
+      if (tid >= 2 && tid < d + 2) col = fmaf(accs[g][tid], fg, col);
+    }
+    M = Mg;
+  }
+  if (tid < d + 2) pout[tid] = tid == 0 ? M : (tid == 1 ? Lsum : col);
+}
+
 // Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their
 // slots; the next S run the partial attention over the slots that are not being replaced; one
 // more (with_finish) runs the finish stage of this step's factor update, which nothing in this
@@ -206,87 +311,48 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     return;
   }
   if ((int)blockIdx.x < n_fetch) {
-    fetch_rows_body(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv, cpr, k,
-                    h, blockIdx.x, n_fetch);
+    fetch_rows_attn_body<T>(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv,
+                            cpr, k, h, blockIdx.x, n_fetch, q, d, scale_log2e,
+                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2));
     return;
   }
-  attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + 1, evict, k, h,
+  attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
                        (int)blockIdx.x - n_fetch);
 }
 
-// One workgroup per head merges the S partial triples (rows of `stride_s` triples per head).
-// With miss_slots != nullptr it first computes triple number S itself: the attention over
-// the head's refetched slots (their slot list, the partial triples and the rows are all
-// requested up front so that the kernel pays two memory latencies, not one per stage).
-// d is a power of two <= 256: thread -> (column c, split group tg).
+// One workgroup per head merges its S partial (max, sum, acc) triples (S <= kCombMaxS).
+// d is a power of two <= 256: thread -> (column c, split group tg); all loads are issued up front.
+constexpr int kCombMaxS = 128;
 template <typename T>
-__global__ __launch_bounds__(kCombThreads) void attn_combine_kernel(float* __restrict__ part, int S, int stride_s,
-                                                                    int d, T* __restrict__ out,
-                                                                    const T* __restrict__ q, const T* __restrict__ K,
-                                                                    const T* __restrict__ V, int n_slots,
-                                                                    int lpr_log2, float scale_log2e,
-                                                                    const int32_t* __restrict__ miss_slots,
-                                                                    const int32_t* __restrict__ miss_count, int k) {
-  constexpr int VEC = Vec16<T>::N;
-  __shared__ float red[kCombWaves][2 + 256];
-  __shared__ float ms_s[65], ls_s[65];  // S + 1 <= 65
-  __shared__ float extra[2 + 256];
+__global__ __launch_bounds__(kCombThreads) void attn_combine_kernel(const float* __restrict__ part, int S, int d,
+                                                                    T* __restrict__ out) {
+  __shared__ float ms_s[kCombMaxS], ls_s[kCombMaxS];
+  __shared__ float comb[kCombThreads];
   const int h = blockIdx.x;
-  const float* p = part + (int64_t)h * stride_s * (d + 2);
+  const float* p = part + (int64_t)h * S * (d + 2);
   const int c = threadIdx.x & (d - 1);
-  const int ntg = kCombThreads / d;
+  const int ntg = kCombThreads / d;  // >= 4
   const int tg = threadIdx.x / d;
-  // the partial triples of this thread: splits tg, tg + ntg, ... (at most 8 with S <= 64, ntg >= 4... 16)
-  float x[16];
+  constexpr int kPer = kCombMaxS / 4;  // triples per thread at most
+  float x[kPer];
 #pragma unroll
-  for (int u = 0; u < 16; ++u) x[u] = p[(int64_t)min(tg + u * ntg, S - 1) * (d + 2) + 2 + c];
-  float mv = 0.0f, lv = 0.0f;
-  if (threadIdx.x < 65) {
+  for (int u = 0; u < kPer; ++u) x[u] = p[(int64_t)min(tg + u * ntg, S - 1) * (d + 2) + 2 + c];
+  if (threadIdx.x < kCombMaxS) {
     const int t = min((int)threadIdx.x, S - 1);
-    mv = p[(int64_t)t * (d + 2)];
-    lv = p[(int64_t)t * (d + 2) + 1];
-  }
-  int n_tr = S;
-  if (miss_slots) {
-    const int cnt = miss_count[h];
-    const int32_t* ms = miss_slots + (int64_t)h * k;
-    float qf[VEC];
-    load_query<T>(q, h, d, lpr_log2, scale_log2e, qf);
-    AttnAcc<VEC> st;
-    st.init();
-    attn_scan<T, kCombWaves>(qf, K + (int64_t)h * n_slots * d, V + (int64_t)h * n_slots * d, d, lpr_log2, 0, cnt,
-                             [&](int i, bool& valid) {
-                               const int slot = ms[max(i, 0)];
-                               valid = slot >= 0 && slot < k;
-                               return valid ? slot : 0;
-                             }, st);
-    const float v = attn_block_merge<VEC, kCombWaves>(st, lpr_log2, d, red);
-    if ((int)threadIdx.x < d + 2) extra[threadIdx.x] = v;
-    n_tr = S + 1;
-  }
-  if (threadIdx.x < 65) {
-    ms_s[threadIdx.x] = mv;
-    ls_s[threadIdx.x] = lv;
-  }
-  __syncthreads();
-  if (miss_slots && threadIdx.x == 0) {
-    ms_s[S] = extra[0];
-    ls_s[S] = extra[1];
+    ms_s[threadIdx.x] = p[(int64_t)t * (d + 2)];
+    ls_s[threadIdx.x] = p[(int64_t)t * (d + 2) + 1];
   }
   __syncthreads();
   float Mh = -INFINITY;
-  for (int t = 0; t < n_tr; ++t) Mh = fmaxf(Mh, ms_s[t]);
+  for (int t = 0; t < S; ++t) Mh = fmaxf(Mh, ms_s[t]);
   float L = 0.0f;
-  for (int t = 0; t < n_tr; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
+  for (int t = 0; t < S; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
   float v = 0.0f;
 #pragma unroll
-  for (int u = 0; u < 16; ++u) {
+  for (int u = 0; u < kPer; ++u) {
     const int t = tg + u * ntg;
     if (t < S && ms_s[t] != -INFINITY) v = fmaf(x[u], exp2f(ms_s[t] - Mh), v);
   }
-  if (miss_slots && tg == 0 && ms_s[S] != -INFINITY) v = fmaf(extra[2 + c], exp2f(ms_s[S] - Mh), v);
-  float* comb = &red[0][0];
-  __syncthreads();
   comb[threadIdx.x] = v;
   __syncthreads();
   if (tg == 0) {
@@ -315,15 +381,14 @@ static int attention_impl(lrqk_ctx* ctx, const void* q, const void* k_act, const
   int S = (n_valid + 63) / 64;
   if (S < 1) S = 1;
   if (S > 64) S = 64;
-  if ((rc = ctx->attn_part.ensure((size_t)bh * (S + 1) * (d + 2) * sizeof(float)))) return rc;
+  if ((rc = ctx->attn_part.ensure((size_t)bh * S * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   hipLaunchKernelGGL((attn_partial_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kAttnThreads), 0, st,
                      (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, n_valid, d, lpr_log2, scale_log2e,
                      (float*)ctx->attn_part.p, S);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (float*)ctx->attn_part.p,
-                     S, S, d, (T*)out, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr, 0, 0, 0.0f,
-                     (const int32_t*)nullptr, (const int32_t*)nullptr, 0);
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
+                     (const float*)ctx->attn_part.p, S, d, (T*)out);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -338,12 +403,12 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
   if (rc) return rc;
   const int cpr = d * (int)sizeof(T) / 16;
-  LRQK_REQUIRE(2 * cpr <= kAttnThreads, LRQK_ELIMIT, "row of %d bytes too long", 2 * cpr * 16);
+  LRQK_REQUIRE(2 * cpr <= kWave, LRQK_ELIMIT, "row of %d bytes does not fit one wave", 2 * cpr * 16);
   int S = (n_slots + 63) / 64;
   if (S > 64) S = 64;
   const int rpb = kAttnThreads / (2 * cpr);
   const int n_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));  // sized for a miss rate of 1/8
-  if ((rc = ctx->attn_part.ensure((size_t)bh * (S + 1) * (d + 2) * sizeof(float)))) return rc;
+  if ((rc = ctx->attn_part.ensure((size_t)bh * (S + n_fetch) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   static_assert(kAttnThreads == kFinThreads, "the finish stage rides in an attention-sized workgroup");
   int with_finish = 0;
@@ -360,9 +425,8 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
                      scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (float*)ctx->attn_part.p,
-                     S, S + 1, d, (T*)out, (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, lpr_log2,
-                     scale_log2e, miss_slots, miss_count, k);
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
+                     (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }

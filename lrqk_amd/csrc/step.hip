@@ -32,7 +32,10 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   // The finish stage of the factor update (B update, outputs, A_K row) is off the critical path: when
   // the step ends with the fetch + attention launch it rides there, and the scan takes the proxy
   // query from the iterates directly.  Any path that cannot absorb it flushes it as its own launch.
-  const bool defer_finish = attn_out != nullptr && !no_hit_miss && ctx->fetch_mode == 0;
+  // (a [K|V] row must fit the lanes of one wave for the fetch role to form its attention term)
+  const bool fused_tail = attn_out != nullptr && !no_hit_miss && ctx->fetch_mode == 0 &&
+                          2 * (size_t)d * elem_size(dtype) / 16 <= (size_t)kWave;
+  const bool defer_finish = fused_tail;
   // ring append folded into the first kernel of the factor update; the flush of a full ring
   // (which reads the slot just written) follows it
   if ((rc = als_decode_append(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq, hkv,
@@ -57,7 +60,7 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
       rc = lrqk_diff(new_idx, topk, active_idx, n, bh, topk, ev, miss_slots, mcount, stream);
     if (rc) return rc;
   }
-  if (!(attn_out && !no_hit_miss && ctx->fetch_mode == 0)) {
+  if (!fused_tail) {
     int rcf = flush_pending_finish(ctx, (hipStream_t)stream);
     if (rcf) return rcf;
   }
@@ -68,7 +71,7 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
     if (attn_out) return lrqk_attention(ctx, q, k_act, v_act, n, n, attn_out, bh, d, dtype, stream);
     return LRQK_OK;
   }
-  if (attn_out && !no_hit_miss) {
+  if (fused_tail) {
     // the fetch is bound by the host link: the attention over the resident slots runs beside it
     return fetch_attention(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, ev, b, hq, hkv, d,
                            topk, q, attn_out, dtype, (hipStream_t)stream);
