@@ -326,32 +326,57 @@ constexpr int kCombMaxS = 128;
 template <typename T>
 __global__ __launch_bounds__(kCombThreads) void attn_combine_kernel(const float* __restrict__ part, int S, int d,
                                                                     T* __restrict__ out) {
-  __shared__ float ms_s[kCombMaxS], ls_s[kCombMaxS];
+  __shared__ float sc_s[kCombMaxS];  // weight exp2(m_t - M) of triple t (0 for an empty one)
+  __shared__ float wred[2][4];
   __shared__ float comb[kCombThreads];
   const int h = blockIdx.x;
   const float* p = part + (int64_t)h * S * (d + 2);
   const int c = threadIdx.x & (d - 1);
   const int ntg = kCombThreads / d;  // >= 4
   const int tg = threadIdx.x / d;
+  // only as many loads as there are triples for this thread (S, ntg are uniform): batches of 8
+  const int per = (S - tg + ntg - 1) / ntg;
   constexpr int kPer = kCombMaxS / 4;  // triples per thread at most
   float x[kPer];
 #pragma unroll
-  for (int u = 0; u < kPer; ++u) x[u] = p[(int64_t)min(tg + u * ntg, S - 1) * (d + 2) + 2 + c];
+  for (int u0 = 0; u0 < kPer; u0 += 8) {
+    if (u0 < per) {
+#pragma unroll
+      for (int u = u0; u < u0 + 8; ++u) x[u] = p[(int64_t)min(tg + u * ntg, S - 1) * (d + 2) + 2 + c];
+    }
+  }
+  // the first two waves hold (m_t, l_t) of triple t = tid: block max, weights, weighted sum of l
+  float mt = -INFINITY, lt = 0.0f;
   if (threadIdx.x < kCombMaxS) {
     const int t = min((int)threadIdx.x, S - 1);
-    ms_s[threadIdx.x] = p[(int64_t)t * (d + 2)];
-    ls_s[threadIdx.x] = p[(int64_t)t * (d + 2) + 1];
+    const float mv = p[(int64_t)t * (d + 2)], lv = p[(int64_t)t * (d + 2) + 1];
+    if ((int)threadIdx.x < S) {
+      mt = mv;
+      lt = lv;
+    }
+    const float wm = wave_max(mt);
+    if (lane_id() == 0) wred[0][wave_id()] = wm;
   }
   __syncthreads();
-  float Mh = -INFINITY;
-  for (int t = 0; t < S; ++t) Mh = fmaxf(Mh, ms_s[t]);
-  float L = 0.0f;
-  for (int t = 0; t < S; ++t) L += (ms_s[t] == -INFINITY) ? 0.0f : ls_s[t] * exp2f(ms_s[t] - Mh);
+  const float Mh = fmaxf(wred[0][0], wred[0][1]);
+  if (threadIdx.x < kCombMaxS) {
+    const float w = (mt == -INFINITY) ? 0.0f : exp2f(mt - Mh);
+    sc_s[threadIdx.x] = w;
+    const float ws = wave_sum(lt * w);
+    if (lane_id() == 0) wred[1][wave_id()] = ws;
+  }
+  __syncthreads();
+  const float L = wred[1][0] + wred[1][1];
   float v = 0.0f;
 #pragma unroll
-  for (int u = 0; u < kPer; ++u) {
-    const int t = tg + u * ntg;
-    if (t < S && ms_s[t] != -INFINITY) v = fmaf(x[u], exp2f(ms_s[t] - Mh), v);
+  for (int u0 = 0; u0 < kPer; u0 += 8) {
+    if (u0 < per) {
+#pragma unroll
+      for (int u = u0; u < u0 + 8; ++u) {
+        const int t = tg + u * ntg;
+        if (t < S) v = fmaf(x[u], sc_s[t], v);
+      }
+    }
   }
   comb[threadIdx.x] = v;
   __syncthreads();
