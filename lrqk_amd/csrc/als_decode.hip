@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
         float wv = 0.0f;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) wv = fmaf(kf[e], qf[e], wv);
-        for (int off = 1; off < lpr; off <<= 1) wv += __shfl_xor(wv, off, kWave);
+        wv = group_sum(wv, lpr);
         if (sub == 0 && row < kGramChunk) w_s[row] = (c0 + row < w1) ? wv : 0.0f;
       }
     }
@@ -352,8 +352,7 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
     float v = 0.0f;
 #pragma unroll 8
     for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], B[c], v);
-    v += __shfl_xor(v, 1, kWave);
-    v += __shfl_xor(v, 2, kWave);
+    v = group_sum(v, 4);
     if (qtr == 0) {
       if (which == 0) rhs_q[row] = v + G[32 * 32 + row];
       else kB[row] = v;

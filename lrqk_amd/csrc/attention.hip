@@ -71,7 +71,7 @@ __device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__
       float sc = 0.0f;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sc = fmaf(kf[e], qf[e], sc);
-      for (int off = 1; off < lpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);
+      sc = group_sum(sc, lpr);
       if (!ok[u]) sc = -INFINITY;
       const float m_new = fmaxf(st.m, sc);
       // exp2 of (-inf) - (-inf) must not produce NaN: while nothing valid was seen keep zeros
@@ -250,7 +250,7 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sc = fmaf(f[e], qf[e], sc);
     }
-    for (int off = 1; off < cpr; off <<= 1) sc += __shfl_xor(sc, off, kWave);  // K lanes: the row's score
+    sc = group_sum(sc, cpr);  // K lanes: the row's score
     const float s_row = __shfl(sc, (lane & ~(chunks - 1)) | 0, kWave);           // first K lane of this row
     if (!is_k) {
       const float s_use = ok ? s_row : -INFINITY;

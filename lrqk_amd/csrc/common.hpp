@@ -157,6 +157,33 @@ __device__ __forceinline__ float lane_bcast(float v, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+// Sum over aligned groups of `n` adjacent lanes (n a power of two); every lane of a group gets
+// the group's sum.  Steps inside a row of 16 lanes are register moves, wider ones shuffles.
+template <int CTRL>
+__device__ __forceinline__ float dpp_self(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float group_sum(float v, int n) {
+  if (n > 1) v += dpp_self<kDppQuadXor1>(v);
+  if (n > 2) v += dpp_self<kDppQuadXor2>(v);
+  if (n > 4) v += dpp_self<kDppRowHalfMirror>(v);
+  if (n > 8) v += dpp_self<kDppRowMirror>(v);
+  if (n > 16) v += __shfl_xor(v, 16, kWave);
+  if (n > 32) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+// wave-wide reductions of unsigned values, result in every lane
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_reduce_u32(uint32_t v, Op op) {
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, kDppQuadXor1, 0xf, 0xf, false));
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, kDppQuadXor2, 0xf, 0xf, false));
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, kDppRowHalfMirror, 0xf, 0xf, false));
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, kDppRowMirror, 0xf, 0xf, false));
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+  return op(op(a, b), op(c, d));
+}
+
 // result in every lane
 __device__ __forceinline__ float wave_sum(float v) {
   v = row_reduce(v, [](float a, float b) { return a + b; });

@@ -539,8 +539,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     vmax = max(vmax, key);
   });
   if (!fast) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) vmin = min(vmin, (uint32_t)__shfl_xor((int)vmin, off, kWave));
+    vmin = wave_reduce_u32(vmin, [](uint32_t a, uint32_t b) { return a < b ? a : b; });
     if (lane == 0) wred[wave] = vmin;
     __syncthreads();
     vmin = 0xffffffffu;
@@ -550,11 +549,8 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     __syncthreads();
   }
   for_each([&](uint32_t key, int64_t) { vor |= key - lo; });
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    vmax = max(vmax, (uint32_t)__shfl_xor((int)vmax, off, kWave));
-    vor |= (uint32_t)__shfl_xor((int)vor, off, kWave);
-  }
+  vmax = wave_reduce_u32(vmax, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+  vor = wave_reduce_u32(vor, [](uint32_t a, uint32_t b) { return a | b; });
   if (lane == 0) {
     wred[wave] = vmax;
     wred[kSelWaves + wave] = vor;
