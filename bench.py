@@ -50,6 +50,8 @@ def parse():
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
                    help="miss fetch: the kernel reads the pinned store itself, or host gather + hipMemcpyAsync")
+    p.add_argument("--victim-rows", type=int, default=-1,
+                   help="rows per head of the device-side cache of evicted K/V rows (-1: k, 0: off)")
     p.add_argument("--mode", default="decode", choices=["decode", "prefill_als", "decoder"],
                    help="prefill_als: time the prefill factorisation alone (workload llama8b_32k_prefill_als unless "
                         "--workload is given); a step is one whole factorisation.  decoder: greedy decoding with a "
@@ -209,6 +211,8 @@ def main():
     eng.init_factors = A0
     eng.attn_in_step = not a.no_attn
     eng.fetch_mode = a.fetch
+    if a.victim_rows >= 0:
+        eng.victim_rows = a.victim_rows
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     eng.prefill(Q, K, V)
@@ -238,6 +242,7 @@ def main():
 
     eng.ws.timing_enable(a.steps, every=max(1, a.event_every))
     eng.ws.select_stats(reset=True)
+    eng.ws.victim_stats(reset=True)
     counts = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -250,6 +255,9 @@ def main():
     eng.ws.timing_enable(0)
     sel_fast, sel_full = eng.ws.select_stats()
     sel_short, sel_over = eng.ws.select_stats_detail()
+    host_rows = eng.ws.victim_stats()
+    vic_on = (eng.victim_rows if eng.victim_rows is not None else w.num_active_tokens) > 0 and a.fetch == "direct" \
+        and not a.no_attn and a.variant == "default"
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
 
@@ -306,7 +314,11 @@ def main():
                    "variant": a.variant, "fetch": a.fetch, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
-        "h2d_bytes_per_step": round(n_miss / a.steps * row_bytes),
+        "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
+        "missed_bytes_per_step": round(n_miss / a.steps * row_bytes),
+        "victim_cache": {"rows_per_head": (eng.victim_rows if eng.victim_rows is not None else w.num_active_tokens)
+                         if vic_on else 0,
+                         "served": round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0},
         "step_algorithmic_bytes": round(step_bytes),
         "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": "score_filter_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,

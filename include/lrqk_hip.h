@@ -123,6 +123,18 @@ int lrqk_fetch_rows_staged(lrqk_ctx* ctx, const void* kv_store, int64_t cap, voi
  * host_threads gather threads (<= 0 keeps the current count).  No counterpart in the reference. */
 int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
 
+/* Victim cache for lrqk_decode_step (no counterpart in the reference; off by default).  K/V rows
+ * that leave the top-k slots are kept in a per-head FIFO of rows_per_head rows on the device
+ * (tokens near the selection threshold return within a few steps); a missed row that is still
+ * there is copied from the FIFO instead of over the host link.  Results are identical: a token's
+ * row never changes.  The cache belongs to ONE sequence: call this again (any value) to drop its
+ * contents before the ctx is used for another prompt.  0 switches it off.  Memory: bh *
+ * rows_per_head rows of 2*d elements plus 2 bytes per (head, store row). */
+int lrqk_ctx_victim_cache(lrqk_ctx* ctx, int rows_per_head);
+/* Rows that lrqk_decode_step fetched over the host link since the last reset (the other missed
+ * rows came from the victim cache).  Synchronises.  Counts only while the victim cache is on. */
+int lrqk_victim_stats(lrqk_ctx* ctx, int64_t* host_rows, int reset);
+
 /* py:1339-1351 fetch_by_hit (same-device branch) -- k_act[bh][j][:] = src[b][h/groups][idx[bh][j]][:]
  * for j < count, src: [b][hkv][src_len][d] on the device. */
 int lrqk_gather_rows(const void* src, int64_t src_len, const int32_t* idx, int64_t idx_stride, int count,

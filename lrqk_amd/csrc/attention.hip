@@ -14,6 +14,7 @@
 #include "ctx.hpp"
 #include "rows.hpp"
 #include "als_finish.hpp"
+#include "victim.hpp"
 
 namespace lrqk {
 
@@ -200,7 +201,8 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
                                                      const int32_t* __restrict__ miss_slots,
                                                      const int32_t* __restrict__ miss_count, int hq, int hkv, int cpr,
                                                      int k, int h, int blk, int nblk, const T* __restrict__ q, int d,
-                                                     float scale_log2e, float* __restrict__ pout) {
+                                                     float scale_log2e, float* __restrict__ pout,
+                                                     const int32_t* __restrict__ miss_old, const VictimView& vic) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float accs[8][256 + 2];               // [row group][m, l, acc[d]] (at most 8 groups are merged at a time)
   const int tid = threadIdx.x, lane = lane_id();
@@ -237,8 +239,44 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
     }
     uint4 val = make_uint4(0, 0, 0, 0);
     if (ok) {
-      val = store[(((int64_t)b * hkv + kvh) * cap + tok) * chunks + c];
       const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
+      const uint4* src = store + (((int64_t)b * hkv + kvh) * cap + tok) * chunks + c;
+      if (vic.nv > 0) {
+        // Victim cache.  The row that leaves the slot goes to FIFO position base + j (unless the
+        // cache still holds it); the row that enters is taken from the FIFO if it is there and
+        // not being replaced in this very step.  All reads of the metadata come before the writes,
+        // and a row's lanes share one wave, so they decide alike.
+        const int nv = vic.nv;
+        const int base = vic.base[h];
+        const int n_ins = min(cnt, nv);
+        const int32_t old = miss_old[(int64_t)h * k + j];
+        const int p_ins = (base + j) % nv;
+        bool do_ins = j < nv && old >= 0 && old < vic.cap;
+        int q_old = -1;
+        if (do_ins) q_old = vic.pos[(int64_t)h * vic.cap + old];
+        int p_new = tok < vic.cap ? (int)vic.pos[(int64_t)h * vic.cap + tok] : -1;
+        if (q_old >= 0 && !victim_slot_in_flight(q_old, base, n_ins, nv) && vic.tok[(int64_t)h * nv + q_old] == old)
+          do_ins = false;
+        bool from_fifo = p_new >= 0 && !victim_slot_in_flight(p_new, base, n_ins, nv);
+        if (from_fifo) from_fifo = vic.tok[(int64_t)h * nv + p_new] == tok;
+        const int32_t prev = do_ins ? vic.tok[(int64_t)h * nv + p_ins] : -1;
+        int prev_pos = -1;
+        if (prev >= 0 && prev < vic.cap) prev_pos = vic.pos[(int64_t)h * vic.cap + prev];
+        if (from_fifo) src = vic.rows + ((int64_t)h * nv + p_new) * chunks + c;
+        const uint4 old_val = is_k ? k_act[dst + c] : v_act[dst + (c - cpr)];
+        val = *src;
+        if (do_ins) {
+          vic.rows[((int64_t)h * nv + p_ins) * chunks + c] = old_val;
+          if (c == 0) {
+            if (prev_pos == p_ins) vic.pos[(int64_t)h * vic.cap + prev] = -1;
+            vic.tok[(int64_t)h * nv + p_ins] = old;
+            vic.pos[(int64_t)h * vic.cap + old] = (int16_t)p_ins;
+          }
+        }
+        if (c == 0 && !from_fifo) atomicAdd(&vic.host_rows[h], 1);
+      } else {
+        val = *src;
+      }
       if (is_k) k_act[dst + c] = val; else v_act[dst + (c - cpr)] = val;
     }
     Vec16<T> vv;
@@ -304,7 +342,7 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
     int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
     int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
-    FinishArgs fa) {
+    FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic) {
   const int h = blockIdx.y;
   if (with_finish && (int)blockIdx.x == n_fetch + S) {
     als_finish_body<T>(fa, h);
@@ -313,7 +351,7 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
   if ((int)blockIdx.x < n_fetch) {
     fetch_rows_attn_body<T>(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv,
                             cpr, k, h, blockIdx.x, n_fetch, q, d, scale_log2e,
-                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2));
+                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic);
     return;
   }
   attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
@@ -422,8 +460,11 @@ template <typename T>
 static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t cap, void* k_act, void* v_act,
                                 int n_slots, int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
                                 const int32_t* miss_count, const uint8_t* evict, int b, int hq, int hkv, int d, int k,
-                                const void* q, void* out, hipStream_t st) {
+                                const void* q, void* out, hipStream_t st, const int32_t* miss_old,
+                                const VictimView* vicp) {
   const int bh = b * hq;
+  VictimView vic{};
+  if (vicp && miss_old && vicp->nv > 0) vic = *vicp;
   int lpr_log2 = 0;
   int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
   if (rc) return rc;
@@ -448,7 +489,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish), (unsigned)bh),
                      dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
-                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin);
+                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic);
   LRQK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
                      (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);
@@ -461,7 +502,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
-                    hipStream_t st) {
+                    hipStream_t st, const int32_t* miss_old, const VictimView* vic) {
   const void* dev_store = nullptr;
   int rc = resolve_store(kv_store, &dev_store);
   if (rc) return rc;
@@ -470,9 +511,9 @@ int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_ac
                LRQK_EINVAL, "pointers must be 16-byte aligned");
   if (dtype == LRQK_F32)
     return fetch_attention_impl<float>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                       miss_count, evict, b, hq, hkv, d, k, q, out, st);
+                                       miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic);
   return fetch_attention_impl<bf16_t>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                      miss_count, evict, b, hq, hkv, d, k, q, out, st);
+                                      miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic);
 }
 
 }  // namespace lrqk

@@ -52,6 +52,8 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->new_idx.release();
   ctx->misc.release();
   ctx->stage_dev.release();
+  ctx->vic_rows.release();
+  ctx->vic_meta.release();
   if (ctx->stage_host) (void)hipHostFree(ctx->stage_host);
   if (ctx->stage_ev) (void)hipEventDestroy(ctx->stage_ev);
   if (ctx->side) (void)hipStreamDestroy(ctx->side);

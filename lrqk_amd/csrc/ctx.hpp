@@ -4,6 +4,7 @@
 
 #include "common.hpp"
 #include "als_finish.hpp"
+#include "victim.hpp"
 
 namespace lrqk {
 
@@ -58,6 +59,12 @@ struct lrqk_ctx {
   int fin_dtype = 0;
   bool fin_pending = false;   // B update / outputs / A_K row not done yet
   bool qhat_pending = false;  // q_hat not written yet
+  // victim cache of the decode step (off unless lrqk_ctx_victim_cache asked for rows)
+  lrqk::DevBuf vic_rows, vic_meta;
+  lrqk::VictimView vic{};   // current view; nv == 0 while off or not yet built
+  int vic_req = 0;          // FIFO rows per head asked for
+  int vic_bh = 0, vic_chunks = 0;
+  bool vic_dirty = true;    // (re)initialise before the next use
   // staged miss fetch: pinned host staging, its device twin, side stream and event (created on first use)
   lrqk::DevBuf stage_dev;
   void* stage_host = nullptr;
@@ -81,7 +88,8 @@ namespace lrqk {
 // sizes allow.  Returns 1 if the diff ran, 0 if the caller still has to, negative on error.
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
-                      uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st);
+                      uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
+                      int32_t* miss_old = nullptr, const VictimView* vic = nullptr);
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
 // into its first kernel.
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
@@ -96,5 +104,7 @@ int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st);
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
-                    hipStream_t st);
+                    hipStream_t st, const int32_t* miss_old = nullptr, const VictimView* vic = nullptr);
+// Builds / resets the victim cache for the given geometry (no-op when it is current).
+int victim_prepare(lrqk_ctx* ctx, int bh, int64_t cap, int chunks, hipStream_t st);
 }  // namespace lrqk

@@ -78,6 +78,8 @@ class LightAttentionIndicesFactory:
         self.last_attn = None
         self.attn_in_step = False     # compute attention inside the fused step (uses the step's q)
         self._fetch_mode = "direct"
+        # rows per head of the device-side victim cache of evicted K/V rows (0 = off); None = attn_topk
+        self.victim_rows: Optional[int] = None
 
     # ------------------------------------------------------------------ small accessors
     @property
@@ -204,6 +206,8 @@ class LightAttentionIndicesFactory:
         self._active_idx = torch.full((bsz, nheads, self.gpu_capacity), -1, dtype=torch.int32, device=dev)
         self.prefill_length = seq_len
         self.current_len = seq_len
+        # a new sequence: whatever the victim cache holds belongs to the previous one
+        self.ws.victim_cache(self.attn_topk if self.victim_rows is None else self.victim_rows)
 
         from .factor import cast_lrqk_prefill
         A_Q, B_Q, A_K, B_K = cast_lrqk_prefill(query_states, key_states, r=self.r, lambda_Q=self.weights[0],

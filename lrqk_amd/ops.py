@@ -52,6 +52,16 @@ class Workspace:
         hipMemcpyAsync on a side stream, as the reference stages its misses."""
         check(_lib.load().lrqk_ctx_set_fetch_mode(self.handle, {"direct": 0, "staged": 1}[mode], int(host_threads)))
 
+    def victim_cache(self, rows_per_head: int):
+        """Size (and empty) the victim cache of the fused decode step; 0 switches it off."""
+        check(_lib.load().lrqk_ctx_victim_cache(self.handle, int(rows_per_head)))
+
+    def victim_stats(self, reset: bool = True) -> int:
+        """Rows the fused decode step fetched over the host link since the last reset."""
+        n = ctypes.c_int64()
+        check(_lib.load().lrqk_victim_stats(self.handle, ctypes.byref(n), 1 if reset else 0))
+        return n.value
+
     def timing_enable(self, max_launches: int, every: int = 1):
         """Bracket (every `every`-th of) the next proxy-score launches with HIP events, at most max_launches."""
         check(_lib.load().lrqk_timing_enable(self._h, max_launches))
