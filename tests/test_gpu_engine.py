@@ -170,6 +170,43 @@ def test_staged_fetch_trace(lrqk, oracle):
     assert n > 0
 
 
+def test_victim_cache_is_invisible(lrqk):
+    """The device-side cache of evicted rows only changes where a missed row comes from: two engines on
+    the same stream, one with the cache and one without, must hold bit-identical K/V slots, ids and
+    attention outputs after every step -- while a good part of the misses is served from the cache."""
+    _say("victim cache on/off")
+    from lrqk_amd import synth
+    wl = synth.Workload("v", 8, 2, 64, 1, torch.bfloat16, 3000, 16, 256, 16, (2, 2), (1e-2, 1e-2), 48, rho=16)
+    dev = torch.device(DEV)
+    Q, K, V, bases, gen = synth.prompt_qkv(wl, 5, 3000, device=dev)
+    A0 = synth.init_factors(wl, 3000, 6, device=dev)
+    engs = []
+    for rows in (0, 96):
+        e = lrqk.LightAttentionIndicesFactory(num_lite_tokens=16, attn_topk=256, num_key_value_groups=4, r=16,
+                                              max_iter=(2, 2), tol=(1e-2, 1e-2), capacity=1024)
+        e.victim_rows = rows
+        e.init_factors = (A0[0].clone(), A0[1].clone())
+        e.attn_in_step = True
+        e.prefill(Q, K, V)
+        engs.append(e)
+    stream = synth.DecodeStream(wl, Q[:, :, -1:], bases, gen)
+    missed = 0
+    engs[1].ws.victim_stats(reset=True)
+    for step in range(48):
+        q, k, v = [t.contiguous() for t in stream.next()]
+        for e in engs:
+            e.decode(q, k, v)
+        a, b = engs
+        assert torch.equal(a._active_idx, b._active_idx), step
+        assert torch.equal(a.Kgpu, b.Kgpu) and torch.equal(a.Vgpu, b.Vgpu), step
+        assert torch.equal(a.last_attn, b.last_attn), step
+        assert torch.equal(a.B_Q, b.B_Q) and torch.equal(a.last_evict, b.last_evict), step
+        missed += int(b.last_miss_count.sum())
+    host = engs[1].ws.victim_stats()
+    _say("missed rows", missed, "over the host link", host)
+    assert missed > 0 and 0 < host < 0.9 * missed
+
+
 def test_no_hit_miss_variant(lrqk, oracle):
     _say("no hit/miss trace")
     _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=16, l=40, r=4, k=8, L=4, steps=12, dtype=torch.float32,
