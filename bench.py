@@ -50,6 +50,8 @@ def parse():
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
                    help="miss fetch: the kernel reads the pinned store itself, or host gather + hipMemcpyAsync")
+    p.add_argument("--no-score-index", action="store_true",
+                   help="scan the bf16 A_K rows directly instead of their 8-bit score index")
     p.add_argument("--victim-rows", type=int, default=-1,
                    help="rows per head of the device-side cache of evicted K/V rows (-1: k, 0: off)")
     p.add_argument("--mode", default="decode", choices=["decode", "prefill_als", "decoder"],
@@ -211,6 +213,7 @@ def main():
     eng.init_factors = A0
     eng.attn_in_step = not a.no_attn
     eng.fetch_mode = a.fetch
+    eng.use_score_index = not a.no_score_index
     if a.victim_rows >= 0:
         eng.victim_rows = a.victim_rows
     torch.cuda.synchronize()
@@ -311,7 +314,7 @@ def main():
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
                    "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
-                   "variant": a.variant, "fetch": a.fetch, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
+                   "variant": a.variant, "fetch": a.fetch, "score_index": not a.no_score_index, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),

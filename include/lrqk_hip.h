@@ -123,6 +123,15 @@ int lrqk_fetch_rows_staged(lrqk_ctx* ctx, const void* kv_store, int64_t cap, voi
  * host_threads gather threads (<= 0 keeps the current count).  No counterpart in the reference. */
 int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
 
+/* Score index for the scan (no counterpart in the reference; off by default).  The ctx keeps an
+ * 8-bit copy of the A_K rows (one scale per row, 36 instead of 64 bytes per row for r = 32) and the
+ * scan of lrqk_score_select / lrqk_score_select_diff / lrqk_decode_step reads that copy: it bounds
+ * every row's score and rescores exactly, from a_k itself, only the rows whose bound reaches the
+ * filter threshold.  Results are identical.  The copy is built on demand for rows [0, m) and
+ * extended by the factor update's appended row; it is derived state: after changing rows of a_k
+ * in place call this again (any value) to drop it.  Applies to r = 16, 32, 64. */
+int lrqk_ctx_score_index(lrqk_ctx* ctx, int enable);
+
 /* Victim cache for lrqk_decode_step (no counterpart in the reference; off by default).  K/V rows
  * that leave the top-k slots are kept in a per-head FIFO of rows_per_head rows on the device
  * (tokens near the selection threshold return within a few steps); a missed row that is still

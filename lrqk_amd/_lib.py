@@ -52,6 +52,7 @@ def _sig(lib):
         "lrqk_fetch_rows": ([vp, i64, vp, vp, i32, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_fetch_rows_staged": ([vp, vp, i64, vp, vp, i32, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_ctx_set_fetch_mode": ([vp, i32, i32], i32),
+        "lrqk_ctx_score_index": ([vp, i32], i32),
         "lrqk_ctx_victim_cache": ([vp, i32], i32),
         "lrqk_victim_stats": ([vp, c.POINTER(c.c_int64), i32], i32),
         "lrqk_gather_rows": ([vp, i64, vp, i64, i32, vp, i32, i32, i32, i32, i32, i32, vp], i32),

@@ -438,7 +438,14 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
 
 template <typename T>
 __global__ __launch_bounds__(kFinThreads) void als_finish_kernel(FinishArgs fa) {
-  als_finish_body<T>(fa, blockIdx.x);
+  // workgroups [bh, 2 bh), if launched, encode the appended rows for the score index
+  if ((int)blockIdx.x < fa.bh)
+    als_finish_body<T>(fa, blockIdx.x);
+  else
+    als_index_append_body<T>(fa, (int)blockIdx.x - fa.bh);
+}
+static inline unsigned finish_grid(const FinishArgs& fa) {
+  return (unsigned)fa.bh * (fa.qa != nullptr && fa.append_row >= 0 ? 2u : 1u);
 }
 
 template <typename T>
@@ -485,7 +492,16 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                      deltas);
   LRQK_HIP_CHECK(hipGetLastError());
   FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
-                head_stride, append_row};
+                head_stride, append_row, nullptr, nullptr, nullptr, 0};
+  if (ctx->sidx_enabled && ctx->sidx_a_k == a_k && ctx->sidx_bh == bh && ctx->sidx_r == r && append_row >= 0 &&
+      ctx->sidx_head_rows == head_stride / r && ctx->sidx_dtype == (sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16)) {
+    // the appended row also goes into the score index; rows stay contiguous as long as rows are appended in order
+    fa.qa = (uint8_t*)ctx->sidx_qa.p;
+    fa.qs = (float*)ctx->sidx_qs.p;
+    fa.qw = (const float*)ctx->sidx_wm.p;
+    fa.q_head_rows = ctx->sidx_head_rows;
+    if (append_row == ctx->sidx_valid) ctx->sidx_valid = append_row + 1;  // (a gap is indexed on demand later)
+  }
   if (defer_finish) {
     // the caller lets later launches of the step absorb the finish stage (flush_pending_finish otherwise)
     ctx->fin = fa;
@@ -494,7 +510,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
     ctx->qhat_pending = true;  // q_hat has not been written yet: consumers take the iterate from iter_out
     return LRQK_OK;
   }
-  hipLaunchKernelGGL((als_finish_kernel<T>), dim3((unsigned)bh), dim3(kFinThreads), 0, st, fa);
+  hipLaunchKernelGGL((als_finish_kernel<T>), dim3(finish_grid(fa)), dim3(kFinThreads), 0, st, fa);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -547,9 +563,9 @@ int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st) {
   ctx->fin_pending = false;
   ctx->qhat_pending = false;
   if (ctx->fin_dtype == LRQK_F32)
-    hipLaunchKernelGGL((als_finish_kernel<float>), dim3((unsigned)ctx->fin.bh), dim3(kFinThreads), 0, st, ctx->fin);
+    hipLaunchKernelGGL((als_finish_kernel<float>), dim3(finish_grid(ctx->fin)), dim3(kFinThreads), 0, st, ctx->fin);
   else
-    hipLaunchKernelGGL((als_finish_kernel<bf16_t>), dim3((unsigned)ctx->fin.bh), dim3(kFinThreads), 0, st, ctx->fin);
+    hipLaunchKernelGGL((als_finish_kernel<bf16_t>), dim3(finish_grid(ctx->fin)), dim3(kFinThreads), 0, st, ctx->fin);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }

@@ -2,6 +2,7 @@
 // decode step (where it runs as extra workgroups of the fetch / attention launch).
 #pragma once
 #include "common.hpp"
+#include "score_index.hpp"
 
 namespace lrqk {
 
@@ -59,7 +60,39 @@ struct FinishArgs {
   void* k_hat_out;
   void* a_k;
   int64_t head_stride, append_row;
+  uint8_t* qa;       // score index (8-bit copy of A_K) to extend with the appended row, or nullptr
+  float* qs;
+  const float* qw;   // its per-head transforms [bh][r*r + r]
+  int64_t q_head_rows;
 };
+
+// The row that the finish stage appends to A_K (k_hat of the chosen iterate, as stored), encoded
+// into the score index.  Executed by one whole wave per head; it repeats the stopping decision, so
+// it does not depend on the finish stage and can run beside it.
+template <typename T, int R>
+__device__ __forceinline__ void als_index_append_rows(const FinishArgs& fa, int h) {
+  const int lane = lane_id();
+  float wcol[R];
+  score_index_load_wcol<R>(fa.qw + (int64_t)h * (R * R + R), lane, wcol);
+  const int chosen = als_choose_iterate(fa.deltas, fa.bh, fa.max_iter, R, fa.tol);
+  float v = fa.iter_out[((int64_t)h * fa.max_iter + chosen) * 2 * R + R + min(lane, R - 1)];
+  if (sizeof(T) == 2) v = round_to_bf16_f32(v);
+  if (lane >= R) v = 0.0f;
+  float scale;
+  const uint8_t u = score_index_encode_row<R>(v, wcol, &scale);
+  if (lane < R) fa.qa[((int64_t)h * fa.q_head_rows + fa.append_row) * R + lane] = u;
+  if (lane == 0) fa.qs[(int64_t)h * fa.q_head_rows + fa.append_row] = scale;
+}
+template <typename T>
+__device__ __forceinline__ void als_index_append_body(const FinishArgs& fa, int h) {
+  if (fa.qa == nullptr || fa.append_row < 0 || wave_id() != 0) return;
+  if (fa.r == 32)
+    als_index_append_rows<T, 32>(fa, h);
+  else if (fa.r == 16)
+    als_index_append_rows<T, 16>(fa, h);
+  else if (fa.r == 64)
+    als_index_append_rows<T, 64>(fa, h);
+}
 
 // One workgroup (kFinThreads threads) per head h: batch-wide stopping decision, line-search update
 // of B_Q and B_K (held in registers as 16-byte vectors: vector vi = tid + 256 u covers row

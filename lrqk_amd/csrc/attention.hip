@@ -335,7 +335,8 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
 // Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their
 // slots; the next S run the partial attention over the slots that are not being replaced; one
 // more (with_finish) runs the finish stage of this step's factor update, which nothing in this
-// launch depends on.  The copy is bound by the host link, so the other roles ride along.
+// launch depends on, and after it one that encodes the appended row for the score index (if there
+// is one).  The copy is bound by the host link, so the other roles ride along.
 template <typename T>
 __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     const uint4* __restrict__ store, int64_t cap, int32_t* __restrict__ hit, int64_t hit_stride,
@@ -344,8 +345,11 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
     FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic) {
   const int h = blockIdx.y;
-  if (with_finish && (int)blockIdx.x == n_fetch + S) {
-    als_finish_body<T>(fa, h);
+  if (with_finish && (int)blockIdx.x >= n_fetch + S) {
+    if ((int)blockIdx.x == n_fetch + S)
+      als_finish_body<T>(fa, h);
+    else
+      als_index_append_body<T>(fa, h);  // (one wave) the appended row's entry in the score index
     return;
   }
   if ((int)blockIdx.x < n_fetch) {
@@ -486,7 +490,8 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
       return rc;
     }
   }
-  hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish), (unsigned)bh),
+  const int index_role = with_finish && ctx->fin.qa != nullptr && ctx->fin.append_row >= 0 ? 1 : 0;
+  hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish + index_role), (unsigned)bh),
                      dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
                      scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic);

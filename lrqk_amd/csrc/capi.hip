@@ -53,6 +53,9 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->misc.release();
   ctx->stage_dev.release();
   ctx->vic_rows.release();
+  ctx->sidx_qa.release();
+  ctx->sidx_qs.release();
+  ctx->sidx_wm.release();
   ctx->vic_meta.release();
   if (ctx->stage_host) (void)hipHostFree(ctx->stage_host);
   if (ctx->stage_ev) (void)hipEventDestroy(ctx->stage_ev);

@@ -59,6 +59,13 @@ struct lrqk_ctx {
   int fin_dtype = 0;
   bool fin_pending = false;   // B update / outputs / A_K row not done yet
   bool qhat_pending = false;  // q_hat not written yet
+  // score index: 8-bit copy of the A_K rows for the scan (off unless lrqk_ctx_score_index enabled it)
+  lrqk::DevBuf sidx_qa, sidx_qs, sidx_wm;
+  bool sidx_enabled = false;
+  const void* sidx_a_k = nullptr;   // A_K buffer the index was built from
+  int64_t sidx_head_rows = 0, sidx_valid = 0;  // rows per head; rows [0, valid) are indexed
+  int sidx_r = 0, sidx_dtype = -1, sidx_bh = 0;
+  int64_t sidx_rows_hint = 0;  // rows of A_K known to be written (the decode step sets it); 0 = only the scanned ones
   // victim cache of the decode step (off unless lrqk_ctx_victim_cache asked for rows)
   lrqk::DevBuf vic_rows, vic_meta;
   lrqk::VictimView vic{};   // current view; nv == 0 while off or not yet built
@@ -105,6 +112,10 @@ int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_ac
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
                     hipStream_t st, const int32_t* miss_old = nullptr, const VictimView* vic = nullptr);
+// Makes the score index cover rows [0, m) of a_k (building or extending it as needed).  Returns 1 and
+// fills `view` if the scan may use it, 0 if the index is off or does not apply, negative on error.
+int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t m, int r, int dtype,
+                        hipStream_t st, ScoreIndexView* view);
 // Builds / resets the victim cache for the given geometry (no-op when it is current).
 int victim_prepare(lrqk_ctx* ctx, int bh, int64_t cap, int chunks, hipStream_t st);
 }  // namespace lrqk

@@ -1,0 +1,194 @@
+// Host side of the score index (8-bit copy of the A_K rows used by the scan): binding to an A_K
+// buffer, building / extending it, and the quantisation kernel.
+#include <algorithm>
+
+#include "common.hpp"
+#include "ctx.hpp"
+
+namespace lrqk {
+
+// W of one head from a strided sample of at most kSidxSample of the rows [0, rows): second-moment
+// matrix S of the sample (plus a small ridge), Cholesky factor S = L L^T, W = L^-T.  One workgroup of
+// 256 threads per head, everything in a fixed order (reproducible).  Anything degenerate (no rows,
+// zero or non-finite S, a non-positive pivot) gives W = I.
+constexpr int kSidxSample = 4096;
+constexpr int kSidxTile = 64;  // sample rows per LDS tile
+template <typename T, int R>
+__global__ __launch_bounds__(256) void score_index_whiten_kernel(const T* __restrict__ a_k, int64_t head_stride,
+                                                                 int64_t rows, float* __restrict__ wm) {
+  constexpr int LD = R + 1;
+  constexpr int EPT = (R * R + 255) / 256;  // entries of S per thread
+  __shared__ float tile[kSidxTile][LD];
+  __shared__ float S[R][LD];
+  __shared__ float X[R][LD];
+  __shared__ int bad;
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const T* A = a_k + (int64_t)h * head_stride;
+  float* W = wm + (int64_t)h * (R * R + R);
+  const int64_t step = rows > 0 ? (rows + kSidxSample - 1) / kSidxSample : 1;
+  const int64_t n = rows > 0 ? (rows + step - 1) / step : 0;
+  float acc[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) acc[e] = 0.0f;
+  if (tid == 0) bad = 0;
+  for (int64_t t0 = 0; t0 < n; t0 += kSidxTile) {
+    const int cnt = (int)min((int64_t)kSidxTile, n - t0);
+    __syncthreads();
+    for (int x = tid; x < kSidxTile * R; x += 256) {
+      const int rr = x / R, c = x % R;
+      tile[rr][c] = rr < cnt ? ld_f32<T>(A, (t0 + rr) * step * R + c) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int x = tid + e * 256;
+      if (x < R * R) {
+        const int i = x / R, j = x % R;
+        float s = acc[e];
+        for (int rr = 0; rr < kSidxTile; ++rr) s = fmaf(tile[rr][i], tile[rr][j], s);
+        acc[e] = s;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int x = tid + e * 256;
+    if (x < R * R) S[x / R][x % R] = n > 0 ? acc[e] / (float)n : 0.0f;
+  }
+  __syncthreads();
+  float tr = 0.0f;
+  for (int i = 0; i < R; ++i) tr += S[i][i];
+  const float ridge = 1e-4f * tr / (float)R;
+  if (!(tr > 0.0f && tr < INFINITY) && tid == 0) bad = 1;
+  __syncthreads();
+  if (tid < R) S[tid][tid] += ridge;
+  // Cholesky, column by column (lower triangle of S becomes L)
+  for (int c = 0; c < R; ++c) {
+    __syncthreads();
+    const float piv = S[c][c];
+    if (!(piv > 0.0f && piv < INFINITY)) {
+      if (tid == 0) bad = 1;
+      break;  // uniform: every thread reads the same pivot
+    }
+    const float d = sqrtf(piv);
+    __syncthreads();
+    if (tid == 0) S[c][c] = d;
+    if (tid > c && tid < R) S[tid][c] /= d;
+    __syncthreads();
+    for (int x = tid; x < R * R; x += 256) {
+      const int i = x / R, j = x % R;
+      if (j > c && i >= j) S[i][j] -= S[i][c] * S[j][c];
+    }
+  }
+  __syncthreads();
+  // X = L^-1 by forward substitution, one column per thread
+  if (!bad && tid < R) {
+    const int c = tid;
+    for (int i = 0; i < R; ++i) X[i][c] = 0.0f;
+    X[c][c] = 1.0f / S[c][c];
+    for (int i = c + 1; i < R; ++i) {
+      float s = 0.0f;
+      for (int k = c; k < i; ++k) s = fmaf(S[i][k], X[k][c], s);
+      X[i][c] = -s / S[i][i];
+    }
+    for (int i = c; i < R; ++i)
+      if (!(fabsf(X[i][c]) < INFINITY)) bad = 1;
+    if (!(X[c][c] > 0.0f)) bad = 1;
+  }
+  __syncthreads();
+  const bool ident = bad != 0;
+  // W[i][j] = X[j][i] for i <= j, zero below the diagonal; then 1 / W_jj
+  for (int x = tid; x < R * R; x += 256) {
+    const int i = x / R, j = x % R;
+    W[x] = ident ? (i == j ? 1.0f : 0.0f) : (i <= j ? X[j][i] : 0.0f);
+  }
+  if (tid < R) W[R * R + tid] = ident ? 1.0f : 1.0f / X[tid][tid];
+}
+
+// One wave per row: lane i holds element i of the row, and column `lane` of W stays in registers.
+template <typename T, int R>
+__global__ __launch_bounds__(256) void score_index_build_kernel(const T* __restrict__ a_k, int64_t head_stride,
+                                                                int64_t row0, int64_t row1, uint8_t* __restrict__ qa,
+                                                                float* __restrict__ qs, const float* __restrict__ wm,
+                                                                int64_t head_rows) {
+  const int h = blockIdx.y;
+  const int lane = lane_id();
+  const int64_t wave0 = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave_id();
+  const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x / kWave);
+  float wcol[R];
+  score_index_load_wcol<R>(wm + (int64_t)h * (R * R + R), lane, wcol);
+  for (int64_t row = row0 + wave0; row < row1; row += nwaves) {
+    const float v = lane < R ? ld_f32<T>(a_k, (int64_t)h * head_stride + row * R + lane) : 0.0f;
+    float scale;
+    const uint8_t u = score_index_encode_row<R>(v, wcol, &scale);
+    if (lane < R) qa[((int64_t)h * head_rows + row) * R + lane] = u;
+    if (lane == 0) qs[(int64_t)h * head_rows + row] = scale;
+  }
+}
+
+template <typename T, int R>
+static void launch_build(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t from, int64_t upto,
+                         int64_t head_rows, hipStream_t st) {
+  float* wm = (float*)ctx->sidx_wm.p;
+  if (from == 0)  // first rows of this binding: they set W
+    hipLaunchKernelGGL((score_index_whiten_kernel<T, R>), dim3((unsigned)bh), dim3(256), 0, st, (const T*)a_k, head_stride,
+                       upto, wm);
+  const unsigned blocks = (unsigned)std::min<int64_t>(2048, (upto - from + 3) / 4);
+  hipLaunchKernelGGL((score_index_build_kernel<T, R>), dim3(blocks, (unsigned)bh), dim3(256), 0, st, (const T*)a_k,
+                     head_stride, from, upto, (uint8_t*)ctx->sidx_qa.p, (float*)ctx->sidx_qs.p, wm, head_rows);
+}
+
+int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t m, int r, int dtype,
+                        hipStream_t st, ScoreIndexView* view) {
+  if (!ctx->sidx_enabled) return 0;
+  if (!(r == 16 || r == 32 || r == 64) || head_stride % r != 0 || ((uintptr_t)a_k % 16 != 0)) return 0;
+  const int64_t head_rows = head_stride / r;
+  if (m > head_rows) return 0;
+  const bool bound = ctx->sidx_a_k == a_k && ctx->sidx_head_rows == head_rows && ctx->sidx_r == r &&
+                     ctx->sidx_dtype == dtype && ctx->sidx_bh == bh;
+  if (!bound) {
+    int rc;
+    if ((rc = ctx->sidx_qa.ensure((size_t)bh * head_rows * r))) return rc;
+    if ((rc = ctx->sidx_qs.ensure((size_t)bh * head_rows * sizeof(float)))) return rc;
+    if ((rc = ctx->sidx_wm.ensure((size_t)bh * (r * r + r) * sizeof(float)))) return rc;
+    ctx->sidx_a_k = a_k;
+    ctx->sidx_head_rows = head_rows;
+    ctx->sidx_r = r;
+    ctx->sidx_dtype = dtype;
+    ctx->sidx_bh = bh;
+    ctx->sidx_valid = 0;
+  }
+  if (ctx->sidx_valid < m) {
+    // index everything that is known to exist, so that the rows appended from now on stay contiguous
+    const int64_t upto = std::min(head_rows, std::max(m, ctx->sidx_rows_hint));
+    const int64_t from = ctx->sidx_valid;
+#define LRQK_SIDX_BUILD(TT)                                                                   \
+  (r == 16 ? launch_build<TT, 16>(ctx, a_k, head_stride, bh, from, upto, head_rows, st)       \
+   : r == 32 ? launch_build<TT, 32>(ctx, a_k, head_stride, bh, from, upto, head_rows, st)     \
+             : launch_build<TT, 64>(ctx, a_k, head_stride, bh, from, upto, head_rows, st))
+    if (dtype == LRQK_F32)
+      LRQK_SIDX_BUILD(float);
+    else
+      LRQK_SIDX_BUILD(bf16_t);
+#undef LRQK_SIDX_BUILD
+    LRQK_HIP_CHECK(hipGetLastError());
+    ctx->sidx_valid = upto;
+  }
+  view->qa = (const uint8_t*)ctx->sidx_qa.p;
+  view->qs = (const float*)ctx->sidx_qs.p;
+  view->wm = (const float*)ctx->sidx_wm.p;
+  view->head_rows = head_rows;
+  return 1;
+}
+
+}  // namespace lrqk
+
+using namespace lrqk;
+
+extern "C" int lrqk_ctx_score_index(lrqk_ctx* ctx, int enable) {
+  LRQK_REQUIRE(ctx != nullptr, LRQK_EINVAL, "ctx is null");
+  ctx->sidx_enabled = enable != 0;
+  ctx->sidx_a_k = nullptr;  // whatever was indexed is dropped; the next scan rebuilds what it needs
+  ctx->sidx_valid = 0;
+  return LRQK_OK;
+}

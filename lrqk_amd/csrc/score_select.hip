@@ -23,6 +23,7 @@
 #include "common.hpp"
 #include "ctx.hpp"
 #include "als_finish.hpp"
+#include "score_index.hpp"
 
 namespace lrqk {
 
@@ -191,6 +192,7 @@ constexpr int kFiltRPT = LRQK_FILT_RPT;  // rows per thread and tile
 #endif
 constexpr int kFiltTiles = LRQK_FILT_TILES;  // tiles per workgroup: one global list reservation for all of them
 constexpr int kFiltRows = kFiltThreads * kFiltRPT;
+constexpr int kPreCap = 2048;   // exact hits a prefilter workgroup can hold
 constexpr int kFiltMaxIt = 4;  // most iterations of the factor update whose pending iterate the filter can pick itself
 
 // Proxy query taken straight from the iterates of the factor update whose finish stage has not
@@ -308,6 +310,198 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
   if (n == 0) return;
   if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n);
   __syncthreads();
+  const int gb = g_base;
+  for (int j = tid; j < n; j += kFiltThreads) {
+    const int p = gb + j;
+    if (p < cand_cap) cand[(int64_t)h * cand_cap + p] = lc[j];
+  }
+}
+
+// --------------------------------------------------------------------------- score + filter through the score index
+// Same output as score_filter_kernel (the candidate list of all rows with key >= bound), read from
+// the 8-bit copy of A_K in whitened coordinates: 36 bytes per row instead of 64.  Every wave solves
+// W q' = q (back substitution, lane i holds row i of W; q' ends up in scalar registers); for every
+// row an upper bound of its (rounded) score follows from the copy:
+//   |score - s~| <= D = scale * |q'|_1 * kSidxDFactor,   s~ = scale * sum_j (u_j - 128) q'_j
+//   round_bf16(score) <= s~ + D + (|s~| + D) / 256       (half a bf16 ulp)
+// Rows whose bound reaches the threshold (or is not a number) are rescored exactly from A_K; only
+// those that really pass enter the list.  Two LDS lists: "maybe" row ids, then the (key, id) pairs.
+template <typename T, int R>
+__global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* __restrict__ a_k, int64_t head_stride,
+                                                                       const T* __restrict__ q_hat, int64_t m, int r,
+                                                                       int round_bf16, SelState st,
+                                                                       uint2* __restrict__ cand, int cand_cap,
+                                                                       FilterQ fq, ScoreIndexView six) {
+  static_assert(R == 16 || R == 32 || R == 64, "the score index covers ranks 16, 32, 64");
+  // `maybe` takes the rows whose bound passes (all rows of the workgroup at worst); `lc` collects
+  // the exact hits: if a workgroup had more than kPreCap of them it marks the head's list as
+  // overflowed, which makes the select kernel rescan that head exactly.
+  __shared__ uint2 lc[kPreCap];
+  __shared__ uint32_t maybe[kFiltTiles * kFiltRows];
+  __shared__ int l_count, m_count, g_base;
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x, lane = lane_id();
+  const T* A = a_k + (int64_t)h * head_stride;
+  const uint8_t* QA = six.qa + (int64_t)h * six.head_rows * R;
+  const float* QS = six.qs + (int64_t)h * six.head_rows;
+  RowScorer<T, R> rs;
+  if (tid == 0) {
+    l_count = 0;
+    m_count = 0;
+  }
+  __syncthreads();
+  const uint32_t t_prev = st.t_low[h];
+  const float qn_prev = st.q_norm[h];
+  const bool pending = fq.iter_out != nullptr;
+  float sacc[kFiltMaxIt], oit[kFiltMaxIt];
+  if (pending) {
+    als_delta_sums<kFiltMaxIt>(fq.deltas, fq.bh, fq.max_iter, sacc);
+#pragma unroll
+    for (int it = 0; it < kFiltMaxIt; ++it)
+      oit[it] = fq.iter_out[((int64_t)h * fq.max_iter + min(it, fq.max_iter - 1)) * 2 * r + min(lane, r - 1)];
+  } else {
+    rs.init(q_hat + (int64_t)h * r, r, round_bf16);
+  }
+  // row `lane` of W and 1 / W_ll (lanes >= R repeat the last row; their results are never read)
+  const float* Wm = six.wm + (int64_t)h * (R * R + R);
+  float wrow[R];
+  {
+    const float4* wp = reinterpret_cast<const float4*>(Wm + min(lane, R - 1) * R);
+#pragma unroll
+    for (int c = 0; c < R / 4; ++c) {
+      const float4 w4 = wp[c];
+      wrow[4 * c + 0] = w4.x;
+      wrow[4 * c + 1] = w4.y;
+      wrow[4 * c + 2] = w4.z;
+      wrow[4 * c + 3] = w4.w;
+    }
+  }
+  const float dinv = Wm[R * R + min(lane, R - 1)];
+  float q_lane = 0.0f;  // element `lane` of the proxy query as the exact score uses it
+  if (!pending) q_lane = ld_f32<T>(q_hat, (int64_t)h * r + min(lane, R - 1));
+  // the first rows of the copy are requested before the proxy query is resolved
+  constexpr int kPre = 2;
+  constexpr int QV = R / 16;  // 16-byte vectors per 8-bit row
+  const int64_t base0 = (int64_t)blockIdx.x * kFiltTiles * kFiltRows;
+  uint4 pre[kPre][QV];
+  float pre_s[kPre];
+#pragma unroll
+  for (int it = 0; it < kPre; ++it) {
+    const int64_t i = min(base0 + it * kFiltThreads + tid, m - 1);
+#pragma unroll
+    for (int c = 0; c < QV; ++c) pre[it][c] = reinterpret_cast<const uint4*>(QA + i * R)[c];
+    pre_s[it] = QS[i];
+  }
+  if (pending) {
+    const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
+    float qv = oit[0];
+#pragma unroll
+    for (int it = 1; it < kFiltMaxIt; ++it) qv = chosen == it ? oit[it] : qv;
+    if (blockIdx.x == 0 && tid < r) st_f32<T>((T*)fq.q_hat_out, (int64_t)h * r + tid, qv);
+    rs.init_from_lanes(qv, r, round_bf16);
+    q_lane = sizeof(T) == 2 ? round_to_bf16_f32(qv) : qv;
+  }
+  const float qn = rs.q_norm();
+  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn);
+  if (tid == 0 && blockIdx.x == 0) {
+    st.t_used[h] = tl;
+    st.q_cur[h] = qn;
+  }
+  // q' from W q' = q, last unknown first; lane i keeps the residual of equation i
+  float qc[R];
+  float qsum = 0.0f, ql1 = 0.0f;
+  {
+    float resid = q_lane;
+#pragma unroll
+    for (int j = R - 1; j >= 0; --j) {
+      const float x = sidx_readlane(resid * dinv, j);
+      qc[j] = x;
+      resid = __builtin_fmaf(-x, wrow[j], resid);
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      qsum += qc[j];
+      ql1 += fabsf(qc[j]);
+    }
+  }
+  const float dfac = ql1 * kSidxDFactor;
+  // float threshold; an unset bound (no key passes) keeps the list empty exactly like the plain filter
+  const bool any = tl != 0xffffffffu;
+  const float thr = key_score(tl);
+  const float thr_lo = thr - fabsf(thr) * 1e-6f;
+  auto bound_of = [&](const uint4 (&row)[QV], float scale) {
+    float t = 0.0f;
+#pragma unroll
+    for (int c = 0; c < QV; ++c) {
+      const uint32_t w[4] = {row[c].x, row[c].y, row[c].z, row[c].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        t = fmaf((float)((w[e] >> 0) & 0xffu), qc[c * 16 + e * 4 + 0], t);
+        t = fmaf((float)((w[e] >> 8) & 0xffu), qc[c * 16 + e * 4 + 1], t);
+        t = fmaf((float)((w[e] >> 16) & 0xffu), qc[c * 16 + e * 4 + 2], t);
+        t = fmaf((float)((w[e] >> 24) & 0xffu), qc[c * 16 + e * 4 + 3], t);
+      }
+    }
+    const float sa = scale * (t - 128.0f * qsum);
+    const float dd = scale * dfac;
+    return sa + dd + (fabsf(sa) + dd) * (1.0f / 256.0f);
+  };
+#pragma unroll 1
+  for (int tile = 0; tile < kFiltTiles; ++tile) {
+    const int64_t base = base0 + (int64_t)tile * kFiltRows;
+    if (base >= m) break;
+    uint32_t mask = 0;
+#pragma unroll
+    for (int it = 0; it < kFiltRPT; ++it) {
+      const int64_t i = base + it * kFiltThreads + tid;
+      float ub;
+      if (tile == 0 && it < kPre) {
+        ub = bound_of(pre[it < kPre ? it : 0], pre_s[it < kPre ? it : 0]);
+      } else {
+        const int64_t ic = min(i, m - 1);
+        uint4 row[QV];
+#pragma unroll
+        for (int c = 0; c < QV; ++c) row[c] = reinterpret_cast<const uint4*>(QA + ic * R)[c];
+        ub = bound_of(row, QS[ic]);
+      }
+      if (any && i < m && !(ub < thr_lo)) mask |= 1u << it;
+    }
+    const int cnt = __popc(mask);
+    const int incl = wave_inclusive_sum(cnt);
+    const int wtot = __shfl(incl, kWave - 1, kWave);
+    if (wtot) {
+      int wbase = 0;
+      if (lane == kWave - 1) wbase = atomicAdd(&m_count, wtot);
+      wbase = __shfl(wbase, kWave - 1, kWave);
+      int pos = wbase + incl - cnt;
+#pragma unroll
+      for (int it = 0; it < kFiltRPT; ++it)
+        if ((mask >> it) & 1u) maybe[pos++] = (uint32_t)(base + it * kFiltThreads + tid);
+    }
+  }
+  __syncthreads();
+  // exact scores of the rows that may pass
+  const int nm = m_count;
+  for (int j0 = 0; j0 < nm; j0 += kFiltThreads) {
+    const int j = j0 + tid;
+    const uint32_t i = maybe[min(j, nm - 1)];
+    const uint32_t key = score_key(rs.score(A, (int64_t)i));  // unconditional load (clamped), masked below
+    const bool hit = j < nm && key >= tl;
+    int wt;
+    const int rk = wave_rank(hit, wt);
+    if (wt) {
+      int wbase = 0;
+      if (lane == 0) wbase = atomicAdd(&l_count, wt);
+      wbase = __shfl(wbase, 0, kWave);
+      if (hit && wbase + rk < kPreCap) lc[wbase + rk] = make_uint2(key, i);
+    }
+  }
+  __syncthreads();
+  const int n = l_count;
+  if (n == 0) return;
+  if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n > kPreCap ? cand_cap + 1 : n);
+  __syncthreads();
+  if (n > kPreCap) return;
   const int gb = g_base;
   for (int j = tid; j < n; j += kFiltThreads) {
     const int p = gb + j;
@@ -921,8 +1115,20 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
     }
   }
   dim3 grid((unsigned)((m + (int64_t)kFiltRows * kFiltTiles - 1) / ((int64_t)kFiltRows * kFiltTiles)), (unsigned)bh);
-  hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), filt_smem, st, (const T*)a_k, head_stride,
-                     (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq);
+  bool via_index = false;
+  if constexpr (R == 16 || R == 32 || R == 64) {
+    ScoreIndexView six{};
+    const int ri = score_index_prepare(ctx, a_k, head_stride, bh, m, r, sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16, st, &six);
+    if (ri < 0) return ri;
+    if (ri == 1) {
+      hipLaunchKernelGGL((score_prefilter_kernel<T, R>), grid, dim3(kFiltThreads), 0, st, (const T*)a_k,
+                         head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six);
+      via_index = true;
+    }
+  }
+  if (!via_index)
+    hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), filt_smem, st, (const T*)a_k, head_stride,
+                       (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq);
   LRQK_HIP_CHECK(hipGetLastError());
   if (timed) {
     LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used + 1], st));

@@ -21,6 +21,7 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   const int n = topk + lite;
   int rc;
   ctx->fin_pending = ctx->qhat_pending = false;  // nothing survives a call that failed half-way
+  ctx->sidx_rows_hint = token;                   // rows [0, token) of A_K exist before this step
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
   // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | evict u8 [bh][topk]
   if ((rc = ctx->misc.ensure((size_t)bh * topk * 9 + (size_t)bh * 4 + 64))) return rc;

@@ -80,6 +80,8 @@ class LightAttentionIndicesFactory:
         self._fetch_mode = "direct"
         # rows per head of the device-side victim cache of evicted K/V rows (0 = off); None = attn_topk
         self.victim_rows: Optional[int] = None
+        # 8-bit copy of the A_K rows read by the scan (bounds + exact rescoring of the rows that may pass)
+        self.use_score_index = True
 
     # ------------------------------------------------------------------ small accessors
     @property
@@ -153,6 +155,8 @@ class LightAttentionIndicesFactory:
         self.B_Q = B_Q
         self._A_K.append(A_K)
         self.B_K = B_K
+        # rows of A_K were written behind the library's back: whatever the scan had indexed is dropped
+        self.ws.score_index(self.use_score_index)
         return self
 
     def _is_overridden(self, name: str) -> bool:

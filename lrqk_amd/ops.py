@@ -52,6 +52,10 @@ class Workspace:
         hipMemcpyAsync on a side stream, as the reference stages its misses."""
         check(_lib.load().lrqk_ctx_set_fetch_mode(self.handle, {"direct": 0, "staged": 1}[mode], int(host_threads)))
 
+    def score_index(self, enable: bool):
+        """Switch the 8-bit score index of the scan on or off; either way what was indexed is dropped."""
+        check(_lib.load().lrqk_ctx_score_index(self.handle, 1 if enable else 0))
+
     def victim_cache(self, rows_per_head: int):
         """Size (and empty) the victim cache of the fused decode step; 0 switches it off."""
         check(_lib.load().lrqk_ctx_victim_cache(self.handle, int(rows_per_head)))
