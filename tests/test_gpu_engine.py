@@ -207,6 +207,40 @@ def test_victim_cache_is_invisible(lrqk):
     assert missed > 0 and 0 < host < 0.9 * missed
 
 
+def test_score_index_is_invisible(lrqk):
+    """The 8-bit score index only prefilters the scan: engines with and without it, on the same
+    stream, must select the same tokens and produce the same bits after every step, also once
+    rows appended during decoding (indexed by the finish stage) are among the selected ones."""
+    _say("score index on/off")
+    from lrqk_amd import synth
+    wl = synth.Workload("s", 8, 2, 64, 1, torch.bfloat16, 3000, 32, 256, 8, (2, 2), (1e-2, 1e-2), 96, rho=16)
+    dev = torch.device(DEV)
+    Q, K, V, bases, gen = synth.prompt_qkv(wl, 7, 3000, device=dev)
+    A0 = synth.init_factors(wl, 3000, 8, device=dev)
+    engs = []
+    for on in (False, True):
+        e = lrqk.LightAttentionIndicesFactory(num_lite_tokens=8, attn_topk=256, num_key_value_groups=4, r=32,
+                                              max_iter=(2, 2), tol=(1e-2, 1e-2), capacity=1024)
+        e.use_score_index = on
+        e.init_factors = (A0[0].clone(), A0[1].clone())
+        e.attn_in_step = True
+        e.prefill(Q, K, V)
+        engs.append(e)
+    stream = synth.DecodeStream(wl, Q[:, :, -1:], bases, gen)
+    late = 0
+    for step in range(96):
+        q, k, v = [t.contiguous() for t in stream.next()]
+        for e in engs:
+            e.decode(q, k, v)
+        a, b = engs
+        assert torch.equal(a._active_idx, b._active_idx), step
+        assert torch.equal(a.last_evict, b.last_evict) and torch.equal(a.last_miss_count, b.last_miss_count), step
+        assert torch.equal(a.Kgpu, b.Kgpu) and torch.equal(a.Vgpu, b.Vgpu), step
+        assert torch.equal(a.last_attn, b.last_attn) and torch.equal(a.A_K, b.A_K), step
+        late += int((b._active_idx[:, :, :256] >= 3000).sum())
+    assert late > 0      # tokens appended during decoding were selected
+
+
 def test_no_hit_miss_variant(lrqk, oracle):
     _say("no hit/miss trace")
     _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=16, l=40, r=4, k=8, L=4, steps=12, dtype=torch.float32,

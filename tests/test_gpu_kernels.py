@@ -156,6 +156,59 @@ def test_score_select_filtered_path_ties(ops, oracle):
     assert torch.equal(got, torch.arange(k, dtype=torch.int32).expand(b, H, k))
 
 
+@pytest.mark.parametrize("dtype,r", [(torch.bfloat16, 32), (torch.float32, 32), (torch.bfloat16, 16),
+                                     (torch.bfloat16, 64), (torch.float32, 64)])
+def test_score_select_with_score_index(ops, oracle, dtype, r):
+    """The 8-bit score index only prefilters: with it the selection must equal the oracle's
+    full sort bit for bit, also on rows chosen to stress its bound -- heads whose rows are
+    almost rank one with the query across the dominant direction, columns of very different
+    size, zero rows, a head of all zeros, duplicated columns, a dynamic range of 2^40, scores
+    tied at the threshold -- while the query drifts, jumps and the number of rows grows."""
+    _say("score_select with score index", dtype, r)
+    from lrqk_amd import synth
+    ws = ops.Workspace()
+    ws.score_index(True)
+    g = torch.Generator().manual_seed(21 + r)
+    b, H, m, cap, k = 1, 8, 24000, 24064, 1024
+    A = torch.randn((b, H, cap, r), generator=g)
+    u = torch.randn((r,), generator=g)
+    u /= u.norm()
+    A[0, 1] = torch.randn((cap, 1), generator=g) * 30.0 * u + 0.05 * torch.randn((cap, r), generator=g)  # rank one + noise
+    A[0, 2] *= torch.logspace(-3, 3, r)                                   # columns of very different size
+    A[0, 3, ::3] = 0.0                                                    # zero rows
+    A[0, 4] = 0.0                                                         # nothing at all
+    A[0, 5, :, 1] = A[0, 5, :, 0]                                         # duplicated column
+    A[0, 6] *= torch.exp2(torch.randint(-20, 21, (cap, 1), generator=g).float())   # row sizes over 2^40
+    A[0, 7] = (A[0, 7] * 2).round() / 2                                   # few distinct values: ties
+    A = A.to(dtype)
+    q = torch.randn((b, H, 1, r), generator=g)
+    q[0, 1, 0] -= (q[0, 1, 0] @ u) * u * 0.999                            # across the dominant direction
+    q[0, 7, 0] = 0.0
+    q[0, 7, 0, :2] = 1.0
+    Ad = A.to(DEV)
+    rnd = dtype == torch.bfloat16
+    for step in range(5):
+        qd = q.to(dtype)
+        exp = oracle.compute_hit_indices(qd, A[:, :, :m + 7 * step].contiguous(), k, rnd)[..., 0].to(torch.int32)
+        got = ops.score_select(ws, Ad, qd.to(DEV), m + 7 * step, k, rnd).cpu()
+        assert torch.equal(got, exp), step
+        q = synth.rotate_query(g, q, 0.05)
+    fast, full = ws.select_stats()
+    assert fast >= 12, (fast, full)         # later calls are served from the prefiltered list (heads 4 and 7 tie too much)
+    for scale in (50.0, 0.02, -1.0):
+        qd = (q * scale).to(dtype)
+        exp = oracle.compute_hit_indices(qd, A[:, :, :m].contiguous(), k, rnd)[..., 0].to(torch.int32)
+        got = ops.score_select(ws, Ad, qd.to(DEV), m, k, rnd).cpu()
+        assert torch.equal(got, exp), scale
+    # switching the index off and on again drops and rebuilds it
+    ws.score_index(False)
+    qd = q.to(dtype)
+    exp = oracle.compute_hit_indices(qd, A[:, :, :m].contiguous(), k, rnd)[..., 0].to(torch.int32)
+    assert torch.equal(ops.score_select(ws, Ad, qd.to(DEV), m, k, rnd).cpu(), exp)
+    ws.score_index(True)
+    assert torch.equal(ops.score_select(ws, Ad, qd.to(DEV), m, k, rnd).cpu(), exp)
+
+
 # ---------------------------------------------------------------- diff
 
 def _check_diff(ops, oracle, now, new):
