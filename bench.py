@@ -30,7 +30,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the proxy-score kernel read from hardware counters (rocprofv3 --pmc FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB device copy: x2.000 and x1.000), per
 # workload at its default context.  The summary of those runs is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"llama8b_128k_bf16": (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
+# Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
+# 8-bit copy (36 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
+MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (84807.1 * 2.000 + 1058.7 * 1.000) * 1024,
+                          ("llama8b_128k_bf16", False): (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
 
 
 def parse():
@@ -279,6 +282,9 @@ def main():
                   + bh * n_act * w.r * e + 4 * bh * w.r * w.head_dim * e + 3 * bh * w.num_active_tokens * 4
                   + n_miss / a.steps * row_bytes)
 
+    sidx_on = (not a.no_score_index) and w.r in (16, 32, 64)
+    traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) if a.context is None and a.variant == "default" else None
+
     if a.calib_copy_mb > 0:
         src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -314,7 +320,7 @@ def main():
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
                    "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
-                   "variant": a.variant, "fetch": a.fetch, "score_index": not a.no_score_index, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
+                   "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
@@ -324,10 +330,14 @@ def main():
                          "served": round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0},
         "step_algorithmic_bytes": round(step_bytes),
         "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": {"bound": "hbm", "kernel": "score_filter_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+        # achieved = algorithmic bytes of the scan (r values of the storage type per cached token and head) over
+        # the kernel's duration; with the score index the kernel moves fewer bytes than that (see traffic), so
+        # the algorithmic rate can exceed what the memory system actually delivered (traffic_gbs).
+        "roofline": {"bound": "hbm", "kernel": "score_prefilter_kernel" if sidx_on else "score_filter_kernel",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (round(MEASURED_TRAFFIC_BYTES[w.name]) if w.name in MEASURED_TRAFFIC_BYTES
-                                 and a.context is None and a.variant == "default" else None),
+                     "traffic": round(traffic) if traffic else None,
+                     "traffic_gbs": round(traffic / (kern_us * 1e-6) / 1e9, 1) if traffic and launches else None,
                      "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
         "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full, "list_short": sel_short,
                            "list_overflow": sel_over},
