@@ -56,6 +56,7 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->sidx_qa.release();
   ctx->sidx_qs.release();
   ctx->sidx_wm.release();
+  ctx->sidx_part.release();
   ctx->vic_meta.release();
   if (ctx->stage_host) (void)hipHostFree(ctx->stage_host);
   if (ctx->stage_ev) (void)hipEventDestroy(ctx->stage_ev);

@@ -60,7 +60,7 @@ struct lrqk_ctx {
   bool fin_pending = false;   // B update / outputs / A_K row not done yet
   bool qhat_pending = false;  // q_hat not written yet
   // score index: 8-bit copy of the A_K rows for the scan (off unless lrqk_ctx_score_index enabled it)
-  lrqk::DevBuf sidx_qa, sidx_qs, sidx_wm;
+  lrqk::DevBuf sidx_qa, sidx_qs, sidx_wm, sidx_part;
   bool sidx_enabled = false;
   const void* sidx_a_k = nullptr;   // A_K buffer the index was built from
   int64_t sidx_head_rows = 0, sidx_valid = 0;  // rows per head; rows [0, valid) are indexed

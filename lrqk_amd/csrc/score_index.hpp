@@ -32,6 +32,21 @@ struct ScoreIndexView {
   int64_t head_rows;  // rows per head of qa and qs (= rows per head of A_K)
 };
 
+// Scale of a row from max_j |a'_j| and max_j g_j.  The floor keeps the bound above anything a
+// flush of subnormal products could lose (r * 1.2e-38 per element); a row with a NaN or an
+// infinity gets a NaN scale, which makes the scan rescore it exactly every time.
+__device__ __forceinline__ float score_index_scale(float row_max, float g_max, int r) {
+  const float coef = 3.0f * (float)(r + 2) * 5.9604645e-8f * (1.000001f / kSidxBeta);
+  float scale = fmaxf(fmaxf(row_max * (1.0f / 127.0f), g_max * coef), 1e-30f);
+  if (!(g_max < INFINITY)) scale = NAN;
+  return scale;
+}
+__device__ __forceinline__ uint8_t score_index_code(float a, float inv_scale) {
+  float qv = rintf(a * inv_scale);
+  qv = fminf(fmaxf(qv, -127.0f), 127.0f);  // (also turns a NaN into a number: the NaN scale keeps the row)
+  return (uint8_t)((int)qv + 128);
+}
+
 __device__ __forceinline__ float sidx_readlane(float v, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
@@ -56,14 +71,10 @@ __device__ __forceinline__ uint8_t score_index_encode_row(float a_lane, const fl
   }
   const float row_max = wave_max(fabsf(acc));
   const float g_max = wave_max(g);
-  const float coef = 3.0f * (float)(R + 2) * 5.9604645e-8f * (1.000001f / kSidxBeta);
-  float scale = fmaxf(row_max * (1.0f / 127.0f), g_max * coef);
-  if (!(g_max < INFINITY)) scale = NAN;  // a row with a NaN or an infinity is always rescored exactly
-  const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-  float qv = rintf(acc * inv);
-  qv = fminf(fmaxf(qv, -127.0f), 127.0f);  // (also turns a NaN into a number: the NaN scale keeps the row)
+  const float scale = score_index_scale(row_max, g_max, R);
+  const float inv = 1.0f / scale;
   *scale_out = scale;
-  return (uint8_t)((int)qv + 128);
+  return score_index_code(acc, inv);
 }
 
 }  // namespace lrqk
