@@ -262,7 +262,7 @@ def main():
     sel_fast, sel_full = eng.ws.select_stats()
     sel_short, sel_over = eng.ws.select_stats_detail()
     host_rows = eng.ws.victim_stats()
-    vic_on = (eng.victim_rows if eng.victim_rows is not None else w.num_active_tokens) > 0 and a.fetch == "direct" \
+    vic_on = eng.victim_rows_effective > 0 and a.fetch == "direct" \
         and not a.no_attn and a.variant == "default"
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
@@ -325,7 +325,7 @@ def main():
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
         "missed_bytes_per_step": round(n_miss / a.steps * row_bytes),
-        "victim_cache": {"rows_per_head": (eng.victim_rows if eng.victim_rows is not None else w.num_active_tokens)
+        "victim_cache": {"rows_per_head": eng.victim_rows_effective
                          if vic_on else 0,
                          "served": round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0},
         "step_algorithmic_bytes": round(step_bytes),

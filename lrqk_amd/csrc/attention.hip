@@ -202,7 +202,8 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
                                                      const int32_t* __restrict__ miss_count, int hq, int hkv, int cpr,
                                                      int k, int h, int blk, int nblk, const T* __restrict__ q, int d,
                                                      float scale_log2e, float* __restrict__ pout,
-                                                     const int32_t* __restrict__ miss_old, const VictimView& vic) {
+                                                     const int32_t* __restrict__ miss_old, const VictimView& vic,
+                                                     const int32_t* __restrict__ miss_new) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float accs[8][256 + 2];               // [row group][m, l, acc[d]] (at most 8 groups are merged at a time)
   const int tid = threadIdx.x, lane = lane_id();
@@ -223,61 +224,70 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
   }
   AttnAcc<VEC> st;  // meaningful in the V lanes
   st.init();
-  const int trips = (cnt + nblk * rpb - 1) / (nblk * rpb);  // uniform over the workgroup
-  for (int it = 0; it < trips; ++it) {
+  const int nv = vic.nv;  // uniform
+  const int vbase = nv > 0 ? vic.base[h] : 0;
+  // Every load is unconditional (clamped index, valid address) so that the loads of one stage go out
+  // together: j -> (slot, token, previous token) -> FIFO positions -> row (+ FIFO tags) -> stores.
+  for (int it = 0;; ++it) {
     const int j = blk * rpb + jl + it * nblk * rpb;
-    bool ok = j < cnt;
-    int slot = 0;
-    int32_t tok = 0;
-    if (ok) {
-      slot = miss_slots[(int64_t)h * k + j];
-      ok = slot >= 0 && slot < k;
-      if (ok) {
-        tok = hit[(int64_t)h * hit_stride + slot];
-        ok = tok >= 0 && tok < cap;
+    const int jc = min(j, k - 1);
+    int slot = miss_slots[(int64_t)h * k + jc];
+    int32_t tok = miss_new ? miss_new[(int64_t)h * k + jc] : 0;
+    int32_t old = nv > 0 ? miss_old[(int64_t)h * k + jc] : -1;
+    const int trips = (cnt + nblk * rpb - 1) / (nblk * rpb);  // uniform over the workgroup (first use of cnt)
+    if (it >= trips) break;
+    bool ok = j < cnt && slot >= 0 && slot < k;
+    slot = ok ? slot : 0;
+    if (!miss_new) tok = hit[(int64_t)h * hit_stride + slot];
+    ok = ok && tok >= 0 && tok < cap;
+    tok = ok ? tok : 0;
+    const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
+    const uint4* host_src = store + (((int64_t)b * hkv + kvh) * cap + tok) * chunks + c;
+    // a lane without a row reads a device address (its own slot), never the host store
+    const uint4* own = is_k ? k_act + dst + c : v_act + dst + (c - cpr);
+    uint4 val;
+    if (nv > 0) {
+      // Victim cache.  The row that leaves the slot goes to FIFO position base + j (unless the
+      // cache still holds it); the row that enters is taken from the FIFO if it is there and
+      // not being replaced in this very step.  All reads of the metadata come before the writes,
+      // and a row's lanes share one wave, so they decide alike.
+      const int n_ins = min(cnt, nv);
+      const int p_ins = (vbase + jc) % nv;
+      bool do_ins = ok && j < nv && old >= 0 && old < vic.cap;
+      const int q_old = vic.pos[(int64_t)h * vic.cap + (do_ins ? old : 0)];
+      const int p_new = vic.pos[(int64_t)h * vic.cap + (tok < vic.cap ? tok : 0)];
+      const bool old_cached = do_ins && q_old >= 0 && q_old < nv && !victim_slot_in_flight(q_old, vbase, n_ins, nv);
+      bool from_fifo = ok && tok < vic.cap && p_new >= 0 && p_new < nv && !victim_slot_in_flight(p_new, vbase, n_ins, nv);
+      // the row is requested from where the position table points; the tags confirm it afterwards
+      const uint4* src = from_fifo ? vic.rows + ((int64_t)h * nv + p_new) * chunks + c : (ok ? host_src : own);
+      val = *src;
+      const uint4 old_val = *own;
+      const int32_t tag_new = vic.tok[(int64_t)h * nv + (from_fifo ? p_new : 0)];
+      const int32_t tag_old = vic.tok[(int64_t)h * nv + (old_cached ? q_old : 0)];
+      const int32_t prev = vic.tok[(int64_t)h * nv + p_ins];
+      if (old_cached && tag_old == old) do_ins = false;
+      if (from_fifo && tag_new != tok) {  // (the table and the tags disagree: take the row from the store)
+        from_fifo = false;
+        val = *host_src;
       }
-    }
-    uint4 val = make_uint4(0, 0, 0, 0);
-    if (ok) {
-      const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
-      const uint4* src = store + (((int64_t)b * hkv + kvh) * cap + tok) * chunks + c;
-      if (vic.nv > 0) {
-        // Victim cache.  The row that leaves the slot goes to FIFO position base + j (unless the
-        // cache still holds it); the row that enters is taken from the FIFO if it is there and
-        // not being replaced in this very step.  All reads of the metadata come before the writes,
-        // and a row's lanes share one wave, so they decide alike.
-        const int nv = vic.nv;
-        const int base = vic.base[h];
-        const int n_ins = min(cnt, nv);
-        const int32_t old = miss_old[(int64_t)h * k + j];
-        const int p_ins = (base + j) % nv;
-        bool do_ins = j < nv && old >= 0 && old < vic.cap;
-        int q_old = -1;
-        if (do_ins) q_old = vic.pos[(int64_t)h * vic.cap + old];
-        int p_new = tok < vic.cap ? (int)vic.pos[(int64_t)h * vic.cap + tok] : -1;
-        if (q_old >= 0 && !victim_slot_in_flight(q_old, base, n_ins, nv) && vic.tok[(int64_t)h * nv + q_old] == old)
-          do_ins = false;
-        bool from_fifo = p_new >= 0 && !victim_slot_in_flight(p_new, base, n_ins, nv);
-        if (from_fifo) from_fifo = vic.tok[(int64_t)h * nv + p_new] == tok;
-        const int32_t prev = do_ins ? vic.tok[(int64_t)h * nv + p_ins] : -1;
-        int prev_pos = -1;
-        if (prev >= 0 && prev < vic.cap) prev_pos = vic.pos[(int64_t)h * vic.cap + prev];
-        if (from_fifo) src = vic.rows + ((int64_t)h * nv + p_new) * chunks + c;
-        const uint4 old_val = is_k ? k_act[dst + c] : v_act[dst + (c - cpr)];
-        val = *src;
-        if (do_ins) {
-          vic.rows[((int64_t)h * nv + p_ins) * chunks + c] = old_val;
-          if (c == 0) {
-            if (prev_pos == p_ins) vic.pos[(int64_t)h * vic.cap + prev] = -1;
-            vic.tok[(int64_t)h * nv + p_ins] = old;
-            vic.pos[(int64_t)h * vic.cap + old] = (int16_t)p_ins;
-          }
+      int prev_pos = -1;
+      if (do_ins && prev >= 0 && prev < vic.cap) prev_pos = vic.pos[(int64_t)h * vic.cap + prev];
+      if (do_ins) {
+        vic.rows[((int64_t)h * nv + p_ins) * chunks + c] = old_val;
+        if (c == 0) {
+          if (prev_pos == p_ins) vic.pos[(int64_t)h * vic.cap + prev] = -1;
+          vic.tok[(int64_t)h * nv + p_ins] = old;
+          vic.pos[(int64_t)h * vic.cap + old] = (int16_t)p_ins;
         }
-        if (c == 0 && !from_fifo) atomicAdd(&vic.host_rows[h], 1);
-      } else {
-        val = *src;
       }
+      if (ok && c == 0 && !from_fifo) atomicAdd(&vic.host_rows[h], 1);
+    } else {
+      val = *(ok ? host_src : own);
+    }
+    if (ok) {
       if (is_k) k_act[dst + c] = val; else v_act[dst + (c - cpr)] = val;
+    } else {
+      val = make_uint4(0, 0, 0, 0);
     }
     Vec16<T> vv;
     vv.raw = *reinterpret_cast<decltype(vv.raw)*>(&val);
@@ -343,7 +353,7 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
     int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
     int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
-    FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic) {
+    FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic, const int32_t* __restrict__ miss_new) {
   const int h = blockIdx.y;
   if (with_finish && (int)blockIdx.x >= n_fetch + S) {
     if ((int)blockIdx.x == n_fetch + S)
@@ -355,7 +365,7 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
   if ((int)blockIdx.x < n_fetch) {
     fetch_rows_attn_body<T>(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv,
                             cpr, k, h, blockIdx.x, n_fetch, q, d, scale_log2e,
-                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic);
+                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic, miss_new);
     return;
   }
   attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
@@ -465,7 +475,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
                                 int n_slots, int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
                                 const int32_t* miss_count, const uint8_t* evict, int b, int hq, int hkv, int d, int k,
                                 const void* q, void* out, hipStream_t st, const int32_t* miss_old,
-                                const VictimView* vicp) {
+                                const VictimView* vicp, const int32_t* miss_new) {
   const int bh = b * hq;
   VictimView vic{};
   if (vicp && miss_old && vicp->nv > 0) vic = *vicp;
@@ -474,7 +484,9 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   if (rc) return rc;
   const int cpr = d * (int)sizeof(T) / 16;
   LRQK_REQUIRE(2 * cpr <= kWave, LRQK_ELIMIT, "row of %d bytes does not fit one wave", 2 * cpr * 16);
-  int S = (n_slots + 63) / 64;
+  // 128 slots per attention workgroup: with 64 the launch has twice the workgroups the GPU holds at a time, and
+  // the second half starts only when the first has finished
+  int S = (n_slots + 127) / 128;
   if (S > 64) S = 64;
   const int rpb = kAttnThreads / (2 * cpr);
   const int n_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));  // sized for a miss rate of 1/8
@@ -494,7 +506,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish + index_role), (unsigned)bh),
                      dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
-                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic);
+                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new);
   LRQK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
                      (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);
@@ -507,7 +519,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
-                    hipStream_t st, const int32_t* miss_old, const VictimView* vic) {
+                    hipStream_t st, const int32_t* miss_old, const VictimView* vic, const int32_t* miss_new) {
   const void* dev_store = nullptr;
   int rc = resolve_store(kv_store, &dev_store);
   if (rc) return rc;
@@ -516,9 +528,9 @@ int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_ac
                LRQK_EINVAL, "pointers must be 16-byte aligned");
   if (dtype == LRQK_F32)
     return fetch_attention_impl<float>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                       miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic);
+                                       miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new);
   return fetch_attention_impl<bf16_t>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                      miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic);
+                                      miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new);
 }
 
 }  // namespace lrqk

@@ -96,7 +96,7 @@ namespace lrqk {
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
-                      int32_t* miss_old = nullptr, const VictimView* vic = nullptr);
+                      int32_t* miss_old = nullptr, const VictimView* vic = nullptr, int32_t* miss_new = nullptr);
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
 // into its first kernel.
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
@@ -111,7 +111,8 @@ int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st);
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
-                    hipStream_t st, const int32_t* miss_old = nullptr, const VictimView* vic = nullptr);
+                    hipStream_t st, const int32_t* miss_old = nullptr, const VictimView* vic = nullptr,
+                    const int32_t* miss_new = nullptr);
 // Makes the score index cover rows [0, m) of a_k (building or extending it as needed).  Returns 1 and
 // fills `view` if the scan may use it, 0 if the index is off or does not apply, negative on error.
 int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t m, int r, int dtype,

@@ -626,6 +626,7 @@ struct DiffArgs {
   int32_t* miss_count; // [bh] or nullptr
   int replace_all;     // ablation: hit <- new, everything refetched
   int32_t* miss_old;   // [bh][k] or nullptr: token that the j-th refetched slot held before
+  int32_t* miss_new;   // [bh][k] or nullptr: token that the j-th refetched slot holds now
   int32_t* vic_ptr;    // victim FIFO bookkeeping (nullptr = no victim cache): next insert position per head,
   int32_t* vic_base;   //   and where this step's victims start
   int vic_nv;
@@ -1003,6 +1004,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   for (int j = tid; j < n_pair; j += kSelThreads) {
     const int s = ev_list[j];
     if (df.miss_old) df.miss_old[(int64_t)h * k + j] = hit[s];
+    if (df.miss_new) df.miss_new[(int64_t)h * k + j] = miss_s[j];
     hit[s] = miss_s[j];
     if (df.miss_slots) df.miss_slots[(int64_t)h * k + j] = s;
   }
@@ -1182,7 +1184,7 @@ static int arange_result(int bh, int64_t m, int32_t* out_idx, int64_t out_stride
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
-                      int32_t* miss_old, const VictimView* vic) {
+                      int32_t* miss_old, const VictimView* vic, int32_t* miss_new) {
   int rc = check_select_args(ctx, bh, m, topk, new_idx, topk);
   if (rc) return rc;
   if (m <= topk || topk > kFusedDiffMaxK) {
@@ -1191,7 +1193,7 @@ int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
   }
   SelectBufs sb;
   if ((rc = prepare_select(ctx, bh, m, topk, st, &sb))) return rc;
-  DiffArgs df{hit, hit_stride, evict, miss_slots, miss_count, replace_all, miss_old,
+  DiffArgs df{hit, hit_stride, evict, miss_slots, miss_count, replace_all, miss_old, miss_new,
               vic && vic->nv > 0 ? vic->ptr : nullptr, vic && vic->nv > 0 ? vic->base : nullptr, vic ? vic->nv : 0};
   if (dtype == LRQK_F32)
     rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, new_idx, topk, df, st);
@@ -1232,7 +1234,7 @@ extern "C" int lrqk_score_select(lrqk_ctx* ctx, const void* a_k, int64_t head_st
   if (m <= topk) return arange_result(bh, m, out_idx, out_stride, st);
   SelectBufs sb;
   if ((rc = prepare_select(ctx, bh, m, topk, st, &sb))) return rc;
-  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0};
+  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0};
   if (dtype == LRQK_F32)
     rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, out_idx, out_stride, df, st);
   else
@@ -1279,7 +1281,7 @@ extern "C" int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int b
                                        (int)smem));
     attr_done = true;
   }
-  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0};
+  DiffArgs df{nullptr, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0};
   hipLaunchKernelGGL((select_kernel<float, 0>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, 1, sb.cand, sb.cand_cap,
                      sb.st, sb.keys, sb.key_stride, (const float*)nullptr, (int64_t)0, (const float*)nullptr, m, 1, 0,
                      topk, out_idx, out_stride, df);

@@ -23,13 +23,15 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   ctx->fin_pending = ctx->qhat_pending = false;  // nothing survives a call that failed half-way
   ctx->sidx_rows_hint = token;                   // rows [0, token) of A_K exist before this step
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
-  // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | evict u8 [bh][topk]
-  if ((rc = ctx->misc.ensure((size_t)bh * topk * 9 + (size_t)bh * 4 + 64))) return rc;
+  // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | miss_old i32 [bh][topk] | miss_new i32 [bh][topk] |
+  // evict u8 [bh][topk]
+  if ((rc = ctx->misc.ensure((size_t)bh * topk * 13 + (size_t)bh * 4 + 64))) return rc;
   int32_t* new_idx = (int32_t*)ctx->new_idx.p;
   int32_t* miss_slots = (int32_t*)ctx->misc.p;
   int32_t* mcount = miss_count ? miss_count : miss_slots + (size_t)bh * topk;
   int32_t* miss_old = miss_slots + (size_t)bh * topk + bh;
-  uint8_t* ev = evict ? evict : (uint8_t*)(miss_old + (size_t)bh * topk);
+  int32_t* miss_new = miss_old + (size_t)bh * topk;
+  uint8_t* ev = evict ? evict : (uint8_t*)(miss_new + (size_t)bh * topk);
 
   // The finish stage of the factor update (B update, outputs, A_K row) is off the critical path: when
   // the step ends with the fetch + attention launch it rides there, and the scan takes the proxy
@@ -55,8 +57,9 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   }
   const VictimView* vic = fused_tail && ctx->vic.nv > 0 && !ctx->vic_dirty ? &ctx->vic : nullptr;
   rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, active_idx, n, ev,
-                         miss_slots, mcount, no_hit_miss, (hipStream_t)stream, miss_old, vic);
-  const bool vic_active = vic != nullptr && rc == 1;
+                         miss_slots, mcount, no_hit_miss, (hipStream_t)stream, miss_old, vic, miss_new);
+  const bool fused_diff = rc == 1;  // the select kernel also wrote miss_old / miss_new
+  const bool vic_active = vic != nullptr && fused_diff;
   if (rc < 0) return rc;
   if (ctx->qhat_pending) {  // no scan took the iterate over (cannot happen on the paths above; kept as a guard)
     int rcf = flush_pending_finish(ctx, (hipStream_t)stream);
@@ -83,7 +86,8 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   if (fused_tail) {
     // the fetch is bound by the host link: the attention over the resident slots runs beside it
     return fetch_attention(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, ev, b, hq, hkv, d,
-                           topk, q, attn_out, dtype, (hipStream_t)stream, miss_old, vic_active ? vic : nullptr);
+                           topk, q, attn_out, dtype, (hipStream_t)stream, miss_old, vic_active ? vic : nullptr,
+                           fused_diff ? miss_new : nullptr);
   }
   if ((rc = lrqk_fetch_rows(kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv, d, topk, dtype,
                             stream)))

@@ -78,12 +78,17 @@ class LightAttentionIndicesFactory:
         self.last_attn = None
         self.attn_in_step = False     # compute attention inside the fused step (uses the step's q)
         self._fetch_mode = "direct"
-        # rows per head of the device-side victim cache of evicted K/V rows (0 = off); None = attn_topk
+        # rows per head of the device-side victim cache of evicted K/V rows (0 = off); None = 4 * attn_topk
         self.victim_rows: Optional[int] = None
         # 8-bit copy of the A_K rows read by the scan (bounds + exact rescoring of the rows that may pass)
         self.use_score_index = True
 
     # ------------------------------------------------------------------ small accessors
+    @property
+    def victim_rows_effective(self) -> int:
+        """Rows per head the victim cache is created with (the library's limit is 32767)."""
+        return min(4 * self.attn_topk, 32767) if self.victim_rows is None else self.victim_rows
+
     @property
     def fetch_mode(self) -> str:
         """'direct' (the fetch kernel reads the pinned store) or 'staged' (host gather into pinned staging +
@@ -211,7 +216,7 @@ class LightAttentionIndicesFactory:
         self.prefill_length = seq_len
         self.current_len = seq_len
         # a new sequence: whatever the victim cache holds belongs to the previous one
-        self.ws.victim_cache(self.attn_topk if self.victim_rows is None else self.victim_rows)
+        self.ws.victim_cache(self.victim_rows_effective)
 
         from .factor import cast_lrqk_prefill
         A_Q, B_Q, A_K, B_K = cast_lrqk_prefill(query_states, key_states, r=self.r, lambda_Q=self.weights[0],
