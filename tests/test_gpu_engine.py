@@ -148,6 +148,17 @@ def test_buffer_growth_during_decode(lrqk, oracle):
     assert eng._A_K.capacity > 30
 
 
+def test_growth_with_score_index_and_victim_cache(lrqk, oracle):
+    """r 16 with a small capacity: the factor buffer is reallocated twice while decoding, so the
+    8-bit score index is rebuilt from the new buffer and the victim cache's position table is
+    re-sized; the trace must stay in lock step with the oracle throughout."""
+    _say("growth trace, score index on")
+    eng, orc, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=32, l=300, r=16, k=64, L=8, steps=400,
+                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=24, capacity=64, fp_tol=3e-2,
+                            compare_factors=False)
+    assert n > 0 and eng._A_K.capacity == orc._A_K.capacity and eng._A_K.capacity >= 675   # 450 -> 675 (-> 1012)
+
+
 def test_edge_branch_then_main(lrqk, oracle):
     """k <= l <= k+L at prefill: the growing-prefix branch, then the switch to selection."""
     _say("edge trace")
