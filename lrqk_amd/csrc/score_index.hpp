@@ -9,7 +9,8 @@
 //   a'_j = (u_j - 128) * scale + d_j,  |d_j| <= 0.50002 * scale.
 // The scan solves W q' = q by back substitution and uses  a . q = a' . q'.  Any nonsingular W keeps
 // the bound valid (a stale or poor W only loosens it), because every rounding error is charged to
-// the row: with g_j = sum_i |a_i| |W_ij| and c = 3 (r + 2) 2^-24, the errors of forming a' in fp32,
+// the row: with g_j = sum_i |a_i| |W_ij| and c = 5 (r + 2) 2^-24, the errors of forming a' in fp32
+// (3 r 2^-24 would do for round-to-nearest chains; the margin covers a matrix pipe that truncates),
 // of the back substitution (backward error in W) and of the exact fp32 score chain are together at
 // most c * sum_j g_j |q'_j|, and the scale of a row is raised until c * max_j g_j <= kSidxBeta * scale:
 //   |score - scale * sum_j (u_j - 128) q'_j| <= scale * |q'|_1 * (0.50002 + kSidxBeta + fp32 slack of the sum)
@@ -36,7 +37,7 @@ struct ScoreIndexView {
 // flush of subnormal products could lose (r * 1.2e-38 per element); a row with a NaN or an
 // infinity gets a NaN scale, which makes the scan rescore it exactly every time.
 __device__ __forceinline__ float score_index_scale(float row_max, float g_max, int r) {
-  const float coef = 3.0f * (float)(r + 2) * 5.9604645e-8f * (1.000001f / kSidxBeta);
+  const float coef = 5.0f * (float)(r + 2) * 5.9604645e-8f * (1.000001f / kSidxBeta);
   float scale = fmaxf(fmaxf(row_max * (1.0f / 127.0f), g_max * coef), 1e-30f);
   if (!(g_max < INFINITY)) scale = NAN;
   return scale;
