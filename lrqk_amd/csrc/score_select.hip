@@ -174,11 +174,17 @@ __global__ void init_select_state_kernel(SelState st, int bh) {
 
 // The proxy scores scale with |q_hat|, so the bound carried over from the previous call is
 // rescaled by the ratio of the norms (positive bounds only) and relaxed by 2 %.
-__device__ __forceinline__ uint32_t rescaled_bound(uint32_t t_low, float q_norm_prev, float q_norm_now) {
+// With scores rounded to bf16 every key ends in 0x0000 (score >= 0) or 0xffff (score < 0); the bound is
+// lowered to the next key of that form, so that (key - bound) keeps its 16 trailing zero bits and
+// the radix select of the candidates needs one pass instead of two or three.
+__device__ __forceinline__ uint32_t rescaled_bound(uint32_t t_low, float q_norm_prev, float q_norm_now,
+                                                   int round_bf16) {
   if (t_low == 0xffffffffu || !(q_norm_prev > 0.0f) || !(q_norm_now > 0.0f)) return t_low;
   const float s = key_score(t_low);
   if (!(s > 0.0f)) return t_low;
-  return score_key(s * (q_norm_now / q_norm_prev) * 0.98f);
+  uint32_t key = score_key(s * (q_norm_now / q_norm_prev) * 0.98f);
+  if (round_bf16) key &= 0xffff0000u;  // (s > 0: the key is in the upper half, where rounding down clears the low bits)
+  return key;
 }
 
 // --------------------------------------------------------------------------- score + filter
@@ -278,7 +284,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
     }
     if (tile == 0) {
       const float qn = rs.q_norm();
-      tl = rescaled_bound(t_prev, qn_prev, qn);
+      tl = rescaled_bound(t_prev, qn_prev, qn, round_bf16);
       if (tid == 0 && blockIdx.x == 0) {
         st.t_used[h] = tl;
         st.q_cur[h] = qn;
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     q_lane = sizeof(T) == 2 ? round_to_bf16_f32(qv) : qv;
   }
   const float qn = rs.q_norm();
-  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn);
+  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn, round_bf16);
   if (tid == 0 && blockIdx.x == 0) {
     st.t_used[h] = tl;
     st.q_cur[h] = qn;
