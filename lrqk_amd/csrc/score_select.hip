@@ -337,7 +337,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
                                                                        const T* __restrict__ q_hat, int64_t m, int r,
                                                                        int round_bf16, SelState st,
                                                                        uint2* __restrict__ cand, int cand_cap,
-                                                                       FilterQ fq, ScoreIndexView six) {
+                                                                       FilterQ fq, ScoreIndexView six, int tiles_per_wg) {
   static_assert(R == 16 || R == 32 || R == 64, "the score index covers ranks 16, 32, 64");
   // `maybe` takes the rows whose bound passes (all rows of the workgroup at worst); `lc` collects
   // the exact hits: if a workgroup had more than kPreCap of them it marks the head's list as
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
   // the first rows of the copy are requested before the proxy query is resolved
   constexpr int kPre = 2;
   constexpr int QV = R / 16;  // 16-byte vectors per 8-bit row
-  const int64_t base0 = (int64_t)blockIdx.x * kFiltTiles * kFiltRows;
+  const int64_t base0 = (int64_t)blockIdx.x * tiles_per_wg * kFiltRows;
   uint4 pre[kPre][QV];
   float pre_s[kPre];
 #pragma unroll
@@ -452,10 +452,39 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     const float dd = scale * dfac;
     return sa + dd + (fabsf(sa) + dd) * (1.0f / 256.0f);
   };
+  // exact scores of the collected rows; the ones that really pass go to lc
+  auto rescore = [&]() {
+    const int nm = m_count;
+    for (int j0 = 0; j0 < nm; j0 += kFiltThreads) {
+      const int j = j0 + tid;
+      const uint32_t i = maybe[min(j, nm - 1)];
+      const uint32_t key = score_key(rs.score(A, (int64_t)i));  // unconditional load (clamped), masked below
+      const bool hit = j < nm && key >= tl;
+      int wt;
+      const int rk = wave_rank(hit, wt);
+      if (wt) {
+        int wbase = 0;
+        if (lane == 0) wbase = atomicAdd(&l_count, wt);
+        wbase = __shfl(wbase, 0, kWave);
+        if (hit && wbase + rk < kPreCap) lc[wbase + rk] = make_uint2(key, i);
+      }
+    }
+    __syncthreads();
+  };
+  // A workgroup takes tiles_per_wg consecutive tiles (2 unless the context is so long that the launch
+  // would otherwise hold more workgroups than the GPU does at a time).
 #pragma unroll 1
-  for (int tile = 0; tile < kFiltTiles; ++tile) {
+  for (int tile = 0; tile < tiles_per_wg; ++tile) {
     const int64_t base = base0 + (int64_t)tile * kFiltRows;
     if (base >= m) break;
+    if (tile >= kFiltTiles) {  // (uniform) long contexts only: make room in the list if the next tile might not fit
+      __syncthreads();
+      if (m_count > kFiltTiles * kFiltRows - kFiltRows) {
+        rescore();
+        if (tid == 0) m_count = 0;
+        __syncthreads();
+      }
+    }
     uint32_t mask = 0;
 #pragma unroll
     for (int it = 0; it < kFiltRPT; ++it) {
@@ -486,23 +515,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     }
   }
   __syncthreads();
-  // exact scores of the rows that may pass
-  const int nm = m_count;
-  for (int j0 = 0; j0 < nm; j0 += kFiltThreads) {
-    const int j = j0 + tid;
-    const uint32_t i = maybe[min(j, nm - 1)];
-    const uint32_t key = score_key(rs.score(A, (int64_t)i));  // unconditional load (clamped), masked below
-    const bool hit = j < nm && key >= tl;
-    int wt;
-    const int rk = wave_rank(hit, wt);
-    if (wt) {
-      int wbase = 0;
-      if (lane == 0) wbase = atomicAdd(&l_count, wt);
-      wbase = __shfl(wbase, 0, kWave);
-      if (hit && wbase + rk < kPreCap) lc[wbase + rk] = make_uint2(key, i);
-    }
-  }
-  __syncthreads();
+  rescore();
   const int n = l_count;
   if (n == 0) return;
   if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n > kPreCap ? cand_cap + 1 : n);
@@ -1129,8 +1142,22 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
     const int ri = score_index_prepare(ctx, a_k, head_stride, bh, m, r, sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16, st, &six);
     if (ri < 0) return ri;
     if (ri == 1) {
-      hipLaunchKernelGGL((score_prefilter_kernel<T, R>), grid, dim3(kFiltThreads), 0, st, (const T*)a_k,
-                         head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six);
+      // no more workgroups than the GPU holds at a time: beyond that a workgroup takes more tiles
+      static int slots = 0;
+      if (slots == 0) {
+        int per_cu = 0, dev = 0, n_cu = 0;
+        LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, score_prefilter_kernel<T, R>, kFiltThreads, 0));
+        LRQK_HIP_CHECK(hipGetDevice(&dev));
+        LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        slots = std::max(1, per_cu * n_cu);
+      }
+      const int64_t tiles = (m + kFiltRows - 1) / kFiltRows;
+      const int64_t wgs = std::max<int64_t>(1, std::min<int64_t>((tiles + kFiltTiles - 1) / kFiltTiles, slots / bh));
+      const int tiles_per_wg = (int)std::max<int64_t>(kFiltTiles, (tiles + wgs - 1) / wgs);
+      dim3 grid_ix((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)bh);
+      hipLaunchKernelGGL((score_prefilter_kernel<T, R>), grid_ix, dim3(kFiltThreads), 0, st, (const T*)a_k,
+                         head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six,
+                         tiles_per_wg);
       via_index = true;
     }
   }
