@@ -7,7 +7,7 @@
 //
 // Decode-time structure (two launches, scores never reach HBM):
 //   score_filter : streams A_K once; a row becomes a CANDIDATE if its key is >= the head's
-//                  running lower bound t_low (the key that had rank ~2k at the previous
+//                  running lower bound t_low (the key that had rank ~1.5k at the previous
 //                  call).  Candidates (key, index) are packed per workgroup in LDS and
 //                  appended to a small per-head list.
 //   select       : one workgroup per head.  If the list holds at least k (and not too many)
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void arange_kernel(int32_t* out, int64_t out_s
     out[(int64_t)h * out_stride + i] = i;
 }
 
-// Per-head selector state: t_low (key that had rank ~2k at the previous call), q_norm (|q_hat|
+// Per-head selector state: t_low (key that had rank ~1.5k at the previous call), q_norm (|q_hat|
 // of that call), t_used / q_cur (bound and norm the filter of the current call used).
 struct SelState {
   uint32_t* t_low;
@@ -530,6 +530,10 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
 
 // --------------------------------------------------------------------------- select (+ diff)
 constexpr int kSelThreads = 1024;
+// The bound carried to the next call is the key of rank 1.5 k: the list then holds ~1.5 k candidates per
+// head and stays usable as long as the number of rows above the (rescaled) bound does not drop by a third
+// from one call to the next.  (2 k: 1.3 us slower per 128K step; 1.25 k: 3 rescans in 16384 head-steps.)
+constexpr int kBoundRankNum = 3, kBoundRankDen = 2;
 constexpr int kSelWaves = kSelThreads / kWave;
 constexpr int kChunkBits = 262144;            // token ids covered by one bitmap pass
 constexpr int kChunkWords = kChunkBits / 32;  // 8192 words = 32 KB per bitmap
@@ -791,7 +795,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   const int nbits = range ? (32 - __clz((int)(range >> tz))) : 0;  // significant bits of (key - lo) >> tz
   const int s1 = max(nbits - 12, 0), s2 = max(s1 - 12, 0);
 
-  const int k2 = (int)min((int64_t)2 * k, N);  // rank that defines the next t_low
+  const int k2 = (int)min(((int64_t)kBoundRankNum * k) / kBoundRankDen, N);  // rank that defines the next t_low
   // ---- pass 1 (both ranks share it)
   for_each([&](uint32_t key, int64_t) { atomicAdd(&hist[((key - lo) >> tz) >> s1], 1u); });
   __syncthreads();
@@ -838,7 +842,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   }
   const uint32_t Tk = lo + (offT << tz);
   if (tid == 0) {
-    st.t_low[h] = lo + (offE << tz);  // rank >= 2k (rounded down to the resolved bits)
+    st.t_low[h] = lo + (offE << tz);  // rank >= 1.5k (rounded down to the resolved bits)
     st.q_norm[h] = mode == 0 ? st.q_cur[h] : 0.0f;
   }
 
