@@ -21,7 +21,6 @@ namespace lrqk {
 constexpr int kAttnThreads = 256;          // partial pass
 constexpr int kAttnWaves = kAttnThreads / kWave;
 constexpr int kCombThreads = 1024;         // combine: wide enough to take a head's refetched rows in one pass
-constexpr int kCombWaves = kCombThreads / kWave;
 
 // Online-softmax state of one lane group: running max, sum and the accumulator slice.
 template <int VEC>
