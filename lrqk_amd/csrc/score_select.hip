@@ -339,9 +339,8 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
                                                                        uint2* __restrict__ cand, int cand_cap,
                                                                        FilterQ fq, ScoreIndexView six, int tiles_per_wg) {
   static_assert(R == 16 || R == 32 || R == 64, "the score index covers ranks 16, 32, 64");
-  // `maybe` takes the rows whose bound passes (all rows of the workgroup at worst); `lc` collects
-  // the exact hits: if a workgroup had more than kPreCap of them it marks the head's list as
-  // overflowed, which makes the select kernel rescan that head exactly.
+  // `maybe` takes the rows whose bound passes, `lc` the exact hits among them; both are emptied in
+  // between if a workgroup collects more than they hold.
   __shared__ uint2 lc[kPreCap];
   __shared__ uint32_t maybe[kFiltTiles * kFiltRows];
   __shared__ int l_count, m_count, g_base;
@@ -452,10 +451,32 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     const float dd = scale * dfac;
     return sa + dd + (fabsf(sa) + dd) * (1.0f / 256.0f);
   };
-  // exact scores of the collected rows; the ones that really pass go to lc
+  // the exact hits collected in lc go to the head's list (one reservation per call)
+  auto flush_hits = [&](bool last) {
+    const int n = l_count;  // (uniform: a barrier precedes every call)
+    if (n == 0) return;
+    if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n);
+    __syncthreads();
+    const int gb = g_base;
+    for (int j = tid; j < n; j += kFiltThreads) {
+      const int p = gb + j;
+      if (p < cand_cap) cand[(int64_t)h * cand_cap + p] = lc[j];  // (beyond the capacity the count alone tells the select kernel)
+    }
+    if (!last) {
+      __syncthreads();
+      if (tid == 0) l_count = 0;
+      __syncthreads();
+    }
+  };
+  // exact scores of the collected rows; the ones that really pass go to lc, which is emptied
+  // whenever kPreCap rows have been looked at (so it cannot overflow)
   auto rescore = [&]() {
     const int nm = m_count;
     for (int j0 = 0; j0 < nm; j0 += kFiltThreads) {
+      if (j0 > 0 && j0 % kPreCap == 0) {  // (uniform)
+        __syncthreads();
+        flush_hits(false);
+      }
       const int j = j0 + tid;
       const uint32_t i = maybe[min(j, nm - 1)];
       const uint32_t key = score_key(rs.score(A, (int64_t)i));  // unconditional load (clamped), masked below
@@ -466,7 +487,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
         int wbase = 0;
         if (lane == 0) wbase = atomicAdd(&l_count, wt);
         wbase = __shfl(wbase, 0, kWave);
-        if (hit && wbase + rk < kPreCap) lc[wbase + rk] = make_uint2(key, i);
+        if (hit) lc[wbase + rk] = make_uint2(key, i);
       }
     }
     __syncthreads();
@@ -481,6 +502,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
       __syncthreads();
       if (m_count > kFiltTiles * kFiltRows - kFiltRows) {
         rescore();
+        flush_hits(false);
         if (tid == 0) m_count = 0;
         __syncthreads();
       }
@@ -516,16 +538,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
   }
   __syncthreads();
   rescore();
-  const int n = l_count;
-  if (n == 0) return;
-  if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n > kPreCap ? cand_cap + 1 : n);
-  __syncthreads();
-  if (n > kPreCap) return;
-  const int gb = g_base;
-  for (int j = tid; j < n; j += kFiltThreads) {
-    const int p = gb + j;
-    if (p < cand_cap) cand[(int64_t)h * cand_cap + p] = lc[j];
-  }
+  flush_hits(true);
 }
 
 // --------------------------------------------------------------------------- select (+ diff)

@@ -209,6 +209,30 @@ def test_score_select_with_score_index(ops, oracle, dtype, r):
     assert torch.equal(ops.score_select(ws, Ad, qd.to(DEV), m, k, rnd).cpu(), exp)
 
 
+def test_score_select_index_many_tiles_per_workgroup(ops, oracle):
+    """Many heads and a long range: the scan launches only as many workgroups as the GPU holds, so each one
+    walks ten tiles, and with k = 4096 it collects more rows than its list holds and rescores them in
+    between.  Bit-exact against the oracle on the first call (rescan) and on the filtered calls."""
+    _say("score_select with score index, many tiles per workgroup")
+    from lrqk_amd import synth
+    ws = ops.Workspace()
+    ws.score_index(True)
+    g = torch.Generator().manual_seed(77)
+    b, H, m, r, k = 1, 512, 40000, 16, 4096
+    A = (torch.randn((b, H, m, r), generator=g) * 0.5).bfloat16()
+    q = torch.randn((b, H, 1, r), generator=g)
+    Ad = A.to(DEV)
+    ws.select_stats()
+    for step in range(3):
+        qb = q.bfloat16()
+        exp = oracle.compute_hit_indices(qb, A, k, True)[..., 0].to(torch.int32)
+        got = ops.score_select(ws, Ad, qb.to(DEV), m, k, True).cpu()
+        assert torch.equal(got, exp), step
+        q = synth.rotate_query(g, q, 0.03)
+    fast, full = ws.select_stats()
+    assert fast >= H, (fast, full)      # the later calls went through the filtered list
+
+
 # ---------------------------------------------------------------- diff
 
 def _check_diff(ops, oracle, now, new):
