@@ -483,12 +483,24 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   if (rc) return rc;
   const int cpr = d * (int)sizeof(T) / 16;
   LRQK_REQUIRE(2 * cpr <= kWave, LRQK_ELIMIT, "row of %d bytes does not fit one wave", 2 * cpr * 16);
-  // 128 slots per attention workgroup: with 64 the launch has twice the workgroups the GPU holds at a time, and
-  // the second half starts only when the first has finished
-  int S = (n_slots + 127) / 128;
-  if (S > 64) S = 64;
+  // The launch should not hold more workgroups than the GPU does at a time (a second batch would only start when
+  // the first has finished): 128 slots per attention workgroup if everything fits, else 256, and as many fetch
+  // workgroups as still fit, between 8 and the number that a miss rate of 1/8 keeps busy.
+  static int slots = 0;
+  if (slots == 0) {
+    int per_cu = 0, dev = 0, n_cu = 0;
+    LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fetch_attn_partial_kernel<T>, kAttnThreads, 0));
+    LRQK_HIP_CHECK(hipGetDevice(&dev));
+    LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    slots = std::max(1, per_cu * n_cu);
+  }
   const int rpb = kAttnThreads / (2 * cpr);
-  const int n_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));  // sized for a miss rate of 1/8
+  const int want_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));
+  int S = (n_slots + 127) / 128;  // small launches: finer attention splits
+  if ((int64_t)(S + want_fetch + 2) * bh > slots) S = (n_slots + 255) / 256;
+  if (S > 64) S = 64;
+  const int room = slots / bh - S - 2;
+  const int n_fetch = std::min(want_fetch, std::max(room, 8));
   if ((rc = ctx->attn_part.ensure((size_t)bh * (S + n_fetch) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   static_assert(kAttnThreads == kFinThreads, "the finish stage rides in an attention-sized workgroup");
