@@ -38,9 +38,9 @@ struct AttnAcc {
 // Items begin..end-1 of a sequence; row_of(i, valid) gives the slot row of item i (always a
 // readable row; `valid` says whether it counts).  Each K/V row of d elements is read as
 // d*sizeof(T)/16 chunks by `lpr` adjacent lanes, so a wave covers 64/lpr rows per load
-// instruction with fully coalesced 16-byte accesses; four row groups per pass have their loads
+// instruction with fully coalesced 16-byte accesses; U row groups per pass have their loads
 // issued together (one memory latency), unconditionally, and are masked afterwards.
-template <typename T, int NW, typename RowOf>
+template <typename T, int NW, int U, typename RowOf>
 __device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__ Kh, const T* __restrict__ Vh, int d,
                                           int lpr_log2, int begin, int end, RowOf row_of,
                                           AttnAcc<Vec16<T>::N>& st) {
@@ -51,11 +51,11 @@ __device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__
   const int grp = lane >> lpr_log2;
   const int gpw = kWave >> lpr_log2;  // row groups per wave
   const int rows_per_iter = gpw * NW;
-  for (int base = begin; base < end; base += 4 * rows_per_iter) {
-    Vec16<T> kv[4], vv[4];
-    bool ok[4];
+  for (int base = begin; base < end; base += U * rows_per_iter) {
+    Vec16<T> kv[U], vv[U];
+    bool ok[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int i = base + u * rows_per_iter + wave * gpw + grp;
       bool valid;
       const int rr = row_of(min(i, end - 1), valid);
@@ -64,7 +64,7 @@ __device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__
       vv[u].load(Vh + (int64_t)rr * d + sub * VEC);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       float kf[VEC], vf[VEC];
       kv[u].unpack(kf);
       vv[u].unpack(vf);
@@ -147,7 +147,7 @@ __device__ __forceinline__ void load_query(const T* q, int h, int d, int lpr_log
 
 // Partial layout per (head, split): [m, l, acc[d]] fp32; `stride_s` triples per head.
 // skip (optional): u8 [bh][k_skip], slots s < k_skip with skip != 0 are left out.
-template <typename T>
+template <typename T, int U = 4>
 __device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const T* __restrict__ K,
                                                   const T* __restrict__ V, int n_slots, int n_valid, int d,
                                                   int lpr_log2, float scale_log2e, float* __restrict__ part, int S,
@@ -166,12 +166,12 @@ __device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const
   st.init();
   if (skip) {
     const uint8_t* sk = skip + (int64_t)h * k_skip;
-    attn_scan<T, kAttnWaves>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
+    attn_scan<T, kAttnWaves, U>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
       valid = sk[min(i, k_skip - 1)] == 0 || i >= k_skip;
       return i;
     }, st);
   } else {
-    attn_scan<T, kAttnWaves>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
+    attn_scan<T, kAttnWaves, U>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
       valid = true;
       return i;
     }, st);
@@ -227,87 +227,130 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
   const int vbase = nv > 0 ? vic.base[h] : 0;
   // Every load is unconditional (clamped index, valid address) so that the loads of one stage go out
   // together: j -> (slot, token, previous token) -> FIFO positions -> row (+ FIFO tags) -> stores.
+  // A lane group handles kFR rows per trip, stage by stage, so that one trip covers the usual number of misses.
+  constexpr int kFR = 2;
+  const int per_trip = kFR * nblk * rpb;
   for (int it = 0;; ++it) {
-    const int j = blk * rpb + jl + it * nblk * rpb;
-    const int jc = min(j, k - 1);
-    int slot = miss_slots[(int64_t)h * k + jc];
-    int32_t tok = miss_new ? miss_new[(int64_t)h * k + jc] : 0;
-    int32_t old = nv > 0 ? miss_old[(int64_t)h * k + jc] : -1;
-    const int trips = (cnt + nblk * rpb - 1) / (nblk * rpb);  // uniform over the workgroup (first use of cnt)
+    int j[kFR], slot[kFR];
+    int32_t tok[kFR], old[kFR];
+#pragma unroll
+    for (int u = 0; u < kFR; ++u) {
+      j[u] = blk * rpb + jl + (it * kFR + u) * nblk * rpb;
+      const int jc = min(j[u], k - 1);
+      slot[u] = miss_slots[(int64_t)h * k + jc];
+      tok[u] = miss_new ? miss_new[(int64_t)h * k + jc] : 0;
+      old[u] = nv > 0 ? miss_old[(int64_t)h * k + jc] : -1;
+    }
+    const int trips = (cnt + per_trip - 1) / per_trip;  // uniform over the workgroup (first use of cnt)
     if (it >= trips) break;
-    bool ok = j < cnt && slot >= 0 && slot < k;
-    slot = ok ? slot : 0;
-    if (!miss_new) tok = hit[(int64_t)h * hit_stride + slot];
-    ok = ok && tok >= 0 && tok < cap;
-    tok = ok ? tok : 0;
-    const int64_t dst = ((int64_t)h * n_slots + slot) * cpr;
-    const uint4* host_src = store + (((int64_t)b * hkv + kvh) * cap + tok) * chunks + c;
-    // a lane without a row reads a device address (its own slot), never the host store
-    const uint4* own = is_k ? k_act + dst + c : v_act + dst + (c - cpr);
-    uint4 val;
+    bool ok[kFR];
+    int64_t dst[kFR];
+    const uint4* host_src[kFR];
+    const uint4* own[kFR];
+#pragma unroll
+    for (int u = 0; u < kFR; ++u) {
+      ok[u] = j[u] < cnt && slot[u] >= 0 && slot[u] < k;
+      slot[u] = ok[u] ? slot[u] : 0;
+    }
+    if (!miss_new) {
+#pragma unroll
+      for (int u = 0; u < kFR; ++u) tok[u] = hit[(int64_t)h * hit_stride + slot[u]];
+    }
+#pragma unroll
+    for (int u = 0; u < kFR; ++u) {
+      ok[u] = ok[u] && tok[u] >= 0 && tok[u] < cap;
+      tok[u] = ok[u] ? tok[u] : 0;
+      dst[u] = ((int64_t)h * n_slots + slot[u]) * cpr;
+      host_src[u] = store + (((int64_t)b * hkv + kvh) * cap + tok[u]) * chunks + c;
+      // a lane without a row reads a device address (its own slot), never the host store
+      own[u] = is_k ? k_act + dst[u] + c : v_act + dst[u] + (c - cpr);
+    }
+    uint4 val[kFR];
     if (nv > 0) {
       // Victim cache.  The row that leaves the slot goes to FIFO position base + j (unless the
       // cache still holds it); the row that enters is taken from the FIFO if it is there and
       // not being replaced in this very step.  All reads of the metadata come before the writes,
       // and a row's lanes share one wave, so they decide alike.
       const int n_ins = min(cnt, nv);
-      const int p_ins = (vbase + jc) % nv;
-      bool do_ins = ok && j < nv && old >= 0 && old < vic.cap;
-      const int q_old = vic.pos[(int64_t)h * vic.cap + (do_ins ? old : 0)];
-      const int p_new = vic.pos[(int64_t)h * vic.cap + (tok < vic.cap ? tok : 0)];
-      const bool old_cached = do_ins && q_old >= 0 && q_old < nv && !victim_slot_in_flight(q_old, vbase, n_ins, nv);
-      bool from_fifo = ok && tok < vic.cap && p_new >= 0 && p_new < nv && !victim_slot_in_flight(p_new, vbase, n_ins, nv);
-      // the row is requested from where the position table points; the tags confirm it afterwards
-      const uint4* src = from_fifo ? vic.rows + ((int64_t)h * nv + p_new) * chunks + c : (ok ? host_src : own);
-      val = *src;
-      const uint4 old_val = *own;
-      const int32_t tag_new = vic.tok[(int64_t)h * nv + (from_fifo ? p_new : 0)];
-      const int32_t tag_old = vic.tok[(int64_t)h * nv + (old_cached ? q_old : 0)];
-      const int32_t prev = vic.tok[(int64_t)h * nv + p_ins];
-      if (old_cached && tag_old == old) do_ins = false;
-      if (from_fifo && tag_new != tok) {  // (the table and the tags disagree: take the row from the store)
-        from_fifo = false;
-        val = *host_src;
+      int p_ins[kFR], q_old[kFR], p_new[kFR];
+      bool do_ins[kFR], old_cached[kFR], from_fifo[kFR];
+#pragma unroll
+      for (int u = 0; u < kFR; ++u) {
+        p_ins[u] = (vbase + min(j[u], k - 1)) % nv;
+        do_ins[u] = ok[u] && j[u] < nv && old[u] >= 0 && old[u] < vic.cap;
+        q_old[u] = vic.pos[(int64_t)h * vic.cap + (do_ins[u] ? old[u] : 0)];
+        p_new[u] = vic.pos[(int64_t)h * vic.cap + (tok[u] < vic.cap ? tok[u] : 0)];
       }
-      int prev_pos = -1;
-      if (do_ins && prev >= 0 && prev < vic.cap) prev_pos = vic.pos[(int64_t)h * vic.cap + prev];
-      if (do_ins) {
-        vic.rows[((int64_t)h * nv + p_ins) * chunks + c] = old_val;
-        if (c == 0) {
-          if (prev_pos == p_ins) vic.pos[(int64_t)h * vic.cap + prev] = -1;
-          vic.tok[(int64_t)h * nv + p_ins] = old;
-          vic.pos[(int64_t)h * vic.cap + old] = (int16_t)p_ins;
+      uint4 old_val[kFR];
+      int32_t tag_new[kFR], tag_old[kFR], prev[kFR];
+#pragma unroll
+      for (int u = 0; u < kFR; ++u) {
+        old_cached[u] = do_ins[u] && q_old[u] >= 0 && q_old[u] < nv && !victim_slot_in_flight(q_old[u], vbase, n_ins, nv);
+        from_fifo[u] = ok[u] && tok[u] < vic.cap && p_new[u] >= 0 && p_new[u] < nv &&
+                       !victim_slot_in_flight(p_new[u], vbase, n_ins, nv);
+        // the row is requested from where the position table points; the tags confirm it afterwards
+        const uint4* src = from_fifo[u] ? vic.rows + ((int64_t)h * nv + p_new[u]) * chunks + c : (ok[u] ? host_src[u] : own[u]);
+        val[u] = *src;
+        old_val[u] = *own[u];
+        tag_new[u] = vic.tok[(int64_t)h * nv + (from_fifo[u] ? p_new[u] : 0)];
+        tag_old[u] = vic.tok[(int64_t)h * nv + (old_cached[u] ? q_old[u] : 0)];
+        prev[u] = vic.tok[(int64_t)h * nv + p_ins[u]];
+      }
+      int prev_pos[kFR];
+#pragma unroll
+      for (int u = 0; u < kFR; ++u) {
+        if (old_cached[u] && tag_old[u] == old[u]) do_ins[u] = false;
+        if (from_fifo[u] && tag_new[u] != tok[u]) {  // (the table and the tags disagree: take the row from the store)
+          from_fifo[u] = false;
+          val[u] = *host_src[u];
         }
+        prev_pos[u] = -1;
+        if (do_ins[u] && prev[u] >= 0 && prev[u] < vic.cap) prev_pos[u] = vic.pos[(int64_t)h * vic.cap + prev[u]];
       }
-      if (ok && c == 0 && !from_fifo) atomicAdd(&vic.host_rows[h], 1);
-    } else {
-      val = *(ok ? host_src : own);
-    }
-    if (ok) {
-      if (is_k) k_act[dst + c] = val; else v_act[dst + (c - cpr)] = val;
-    } else {
-      val = make_uint4(0, 0, 0, 0);
-    }
-    Vec16<T> vv;
-    vv.raw = *reinterpret_cast<decltype(vv.raw)*>(&val);
-    float f[VEC];
-    vv.unpack(f);
-    float sc = 0.0f;
-    if (is_k) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) sc = fmaf(f[e], qf[e], sc);
-    }
-    sc = group_sum(sc, cpr);  // K lanes: the row's score
-    const float s_row = __shfl(sc, (lane & ~(chunks - 1)) | 0, kWave);           // first K lane of this row
-    if (!is_k) {
-      const float s_use = ok ? s_row : -INFINITY;
-      const float m_new = fmaxf(st.m, s_use);
-      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
-      const float p = (m_new == -INFINITY) ? 0.0f : exp2f(s_use - m_new);
-      st.l = st.l * alpha + p;
+      for (int u = 0; u < kFR; ++u) {
+        if (do_ins[u]) {
+          vic.rows[((int64_t)h * nv + p_ins[u]) * chunks + c] = old_val[u];
+          if (c == 0) {
+            if (prev_pos[u] == p_ins[u]) vic.pos[(int64_t)h * vic.cap + prev[u]] = -1;
+            vic.tok[(int64_t)h * nv + p_ins[u]] = old[u];
+            vic.pos[(int64_t)h * vic.cap + old[u]] = (int16_t)p_ins[u];
+          }
+        }
+        if (ok[u] && c == 0 && !from_fifo[u]) atomicAdd(&vic.host_rows[h], 1);
+      }
+    } else {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) st.acc[e] = st.acc[e] * alpha + p * f[e];
-      st.m = m_new;
+      for (int u = 0; u < kFR; ++u) val[u] = *(ok[u] ? host_src[u] : own[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kFR; ++u) {
+      if (ok[u]) {
+        if (is_k) k_act[dst[u] + c] = val[u]; else v_act[dst[u] + (c - cpr)] = val[u];
+      } else {
+        val[u] = make_uint4(0, 0, 0, 0);
+      }
+      Vec16<T> vv;
+      vv.raw = *reinterpret_cast<decltype(vv.raw)*>(&val[u]);
+      float f[VEC];
+      vv.unpack(f);
+      float sc = 0.0f;
+      if (is_k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sc = fmaf(f[e], qf[e], sc);
+      }
+      sc = group_sum(sc, cpr);  // K lanes: the row's score
+      const float s_row = __shfl(sc, (lane & ~(chunks - 1)) | 0, kWave);           // first K lane of this row
+      if (!is_k) {
+        const float s_use = ok[u] ? s_row : -INFINITY;
+        const float m_new = fmaxf(st.m, s_use);
+        const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
+        const float p = (m_new == -INFINITY) ? 0.0f : exp2f(s_use - m_new);
+        st.l = st.l * alpha + p;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) st.acc[e] = st.acc[e] * alpha + p * f[e];
+        st.m = m_new;
+      }
     }
   }
   // merge the row groups: V lane (jl, cv) owns columns cv*VEC .. of group jl
@@ -367,8 +410,9 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
                             part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic, miss_new);
     return;
   }
-  attn_partial_body<T>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
-                       (int)blockIdx.x - n_fetch);
+  // (eight row groups in flight per wave: the launch has few attention workgroups)
+  attn_partial_body<T, 8>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
+                          (int)blockIdx.x - n_fetch);
 }
 
 // One workgroup per head merges its S partial (max, sum, acc) triples (S <= kCombMaxS).
