@@ -48,6 +48,101 @@ struct GramAppend {
   int hq, hkv;
 };
 
+// Everything the solve needs from B_Q, B_K, q and the new k -- B_Q B_Q^T and B_K B_K^T (four 32 x 32
+// MFMA tiles: matrix x half of the d axis), q B_Q^T, k B_K^T and q . k -- does not depend on the Gram
+// pass over the active rows, so one more workgroup per head of that launch forms it beside them.
+// out (kPreNe floats per head): tiles [4][1024] | q B_Q^T [32] | k B_K^T [32] | q . k.
+constexpr int kPreNe = 4 * 1024 + 32 + 32 + 1;
+template <typename T>
+__device__ __forceinline__ void als_bgram_body(const T* __restrict__ b_q, const T* __restrict__ b_k,
+                                               const T* __restrict__ q, const T* __restrict__ k_new, int h, int hq,
+                                               int hkv, int r, int d, int vshift, float* __restrict__ out,
+                                               float* __restrict__ sm) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int kMaxVec = 8;  // 16-byte vectors per thread per matrix: r * d / VEC <= 2048
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int b = h / hq, head = h % hq;
+  const int kvh = head / (hq / hkv);
+  const int ld = d + 1;
+  float* BQ = sm;            // [32][d+1]  (rows >= r are zero)
+  float* BK = BQ + 32 * ld;  // [32][d+1]
+  float* qv = BK + 32 * ld;  // [d]
+  float* kv = qv + d;        // [d]
+  const int vpr = 1 << vshift;
+  const int nvec = r << vshift;
+  Vec16<T> vq[kMaxVec], vk[kMaxVec];
+#pragma unroll
+  for (int u = 0; u < kMaxVec; ++u) {
+    const int vi = min(tid + u * kGramThreads, nvec - 1);
+    vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
+    vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
+  }
+  {
+    const int c = min(tid, d - 1);
+    const float qx = ld_f32<T>(q, (int64_t)h * d + c);
+    const float kx = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
+    if (tid < d) {
+      qv[tid] = qx;
+      kv[tid] = kx;
+    }
+  }
+  // zero the padded rows of BQ/BK, then scatter the vectors
+  for (int e = tid; e < (32 - r) * ld; e += kGramThreads) {
+    BQ[r * ld + e] = 0.0f;
+    BK[r * ld + e] = 0.0f;
+  }
+#pragma unroll
+  for (int u = 0; u < kMaxVec; ++u) {
+    const int vi = tid + u * kGramThreads;
+    if (vi < nvec) {
+      const int row = vi >> vshift, c0 = (vi & (vpr - 1)) * VEC;
+      float fq[VEC], fk[VEC];
+      vq[u].unpack(fq);
+      vk[u].unpack(fk);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        BQ[row * ld + c0 + e] = fq[e];
+        BK[row * ld + c0 + e] = fk[e];
+      }
+    }
+  }
+  __syncthreads();
+  // B_Q B_Q^T and B_K B_K^T on the matrix cores: wave -> (matrix, half of the d axis)
+  {
+    const int col = lane & 31, khalf = lane >> 5;
+    const int which = wave & 1, half = wave >> 1;
+    const float* B = (which ? BK : BQ) + col * ld + khalf;
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    const int k1 = (half + 1) * (d / 2);
+#pragma unroll 8
+    for (int kk = half * (d / 2); kk < k1; kk += 2)  // d >= 8 is a power of two
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(B[kk], B[kk], acc, 0, 0, 0);
+    float* mine = out + (which * 2 + half) * 1024;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mine[mfma_row(lane, v) * 32 + col] = acc[v];
+  }
+  // q B_Q^T and k B_K^T : thread -> (output i = tid >> 2, quarter of d)
+  {
+    const int i = tid >> 2, qtr = tid & 3;
+    const int which = i >> 5, row = i & 31;
+    const float* B = (which ? BK : BQ) + row * ld;
+    const float* vec = which ? kv : qv;
+    float v = 0.0f;
+#pragma unroll 8
+    for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], B[c], v);
+    v = group_sum(v, 4);
+    if (qtr == 0) out[4 * 1024 + which * 32 + row] = v;
+  }
+  if (wave == 0) {
+    float v = 0.0f;
+    for (int c = lane; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
+    v = wave_sum(v);
+    if (lane == 0) out[4 * 1024 + 64] = v;
+  }
+}
+
 // Partial layout per (head, split): 32*32 floats of A^T A (row stride 32) then 32 floats of
 // A^T w.  Rows/columns >= r are zero.
 template <typename T>
@@ -56,12 +151,19 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
                                                                 int64_t idx_stride, T* k_prev,
                                                                 int kprev_slots, int n, const T* __restrict__ q, int r,
                                                                 int d, int lpr_log2, float* __restrict__ part, int S,
-                                                                GramAppend ap) {
+                                                                GramAppend ap, const T* __restrict__ b_q,
+                                                                const T* __restrict__ b_k, const T* __restrict__ k_new,
+                                                                int hq, int hkv, float* __restrict__ pre) {
   constexpr int VEC = Vec16<T>::N;
+  extern __shared__ __align__(16) float gram_dyn[];  // used by the extra workgroup only
   __shared__ float w_all[kGramWaves][kGramChunk];
   __shared__ float red[kGramWaves][kGramNe];
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.y, s = blockIdx.x;
+  if (s == S) {  // one workgroup per head beside the S splits
+    als_bgram_body<T>(b_q, b_k, q, k_new, h, hq, hkv, r, d, lpr_log2, pre + (int64_t)h * kPreNe, gram_dyn);
+    return;
+  }
   float* w_s = w_all[wave];
 
   const int lpr = 1 << lpr_log2;
@@ -234,27 +336,16 @@ __device__ __forceinline__ float sum_lanes_0_31(float x) {
 // iter_out per head: [max_iter][2r] (q_hat then k_hat of each iteration);
 // deltas: [bh][max_iter] sum over r of (k_hat - k_hat')^2.
 template <typename T>
-__global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __restrict__ b_q, const T* __restrict__ b_k,
-                                                                  const float* __restrict__ part, int S,
-                                                                  const T* __restrict__ q, const T* __restrict__ k_new,
-                                                                  int hq, int hkv, int r, int d, int vshift,
+__global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* __restrict__ pre,
+                                                                  const float* __restrict__ part, int S, int r,
                                                                   int max_iter, float* __restrict__ iter_out,
                                                                   float* __restrict__ deltas) {
-  constexpr int VEC = Vec16<T>::N;
-  constexpr int kMaxVec = 8;    // 16-byte vectors per thread per matrix: r * d / VEC <= 2048
   constexpr int kMaxSplit = 32;
   extern __shared__ __align__(16) float sm[];
   __shared__ float s_qk;
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.x;
-  const int b = h / hq, head = h % hq;
-  const int kvh = head / (hq / hkv);
-  const int ld = d + 1;
-  float* BQ = sm;                   // [32][d+1]  (rows >= r are zero)
-  float* BK = BQ + 32 * ld;         // [32][d+1]
-  float* qv = BK + 32 * ld;         // [d]
-  float* kv = qv + d;               // [d]
-  float* G = kv + d;                // [kGramNe] summed A^T [A | w]
+  float* G = sm;                    // [kGramNe] summed A^T [A | w]
   float* Mx = G + kGramNe;          // pivot-column exchange buffers of the inversion (16-byte aligned)
   float* GKi = Mx + 2 * 32 * kLdm;  // [32][kLdi]
   float* GQi = GKi + 32 * kLdi;     // [32][kLdi]
@@ -264,10 +355,12 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
   float* hat_q = hat_k + 32;
   float* new_k = hat_q + 32;
   float* tmp = new_k + 32;
-  float* cred = tmp + 32;           // [2 matrices][2 halves of d][32*32] MFMA tiles
+  float* cred = tmp + 32;           // [2 matrices][2 halves of d][32*32] MFMA tiles of B B^T (from the Gram launch)
+  (void)hat_k; (void)hat_q; (void)new_k; (void)tmp;
 
   // ---- every global load of the kernel is issued here, back to back
   const float* pin = part + (int64_t)h * S * kGramNe;
+  const float* pr = pre + (int64_t)h * kPreNe;
   constexpr int kPer = (kGramNe + kSolveThreads - 1) / kSolveThreads;  // 5 entries per thread
   float gsum[kPer];
   {
@@ -278,44 +371,12 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
 #pragma unroll
       for (int t = 0; t < kMaxSplit; ++t) x[u][t] = pin[(int64_t)min(t, S - 1) * kGramNe + min(e, kGramNe - 1)];
     }
-    const int vpr = 1 << vshift;
-    const int nvec = r << vshift;
-    Vec16<T> vq[kMaxVec], vk[kMaxVec];
+    float4 tl4[4];  // the four B B^T tiles: 4096 floats, 16 per thread
 #pragma unroll
-    for (int u = 0; u < kMaxVec; ++u) {
-      const int vi = min(tid + u * kSolveThreads, nvec - 1);
-      vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
-      vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
-    }
-    {
-      const int c = min(tid, d - 1);
-      const float qx = ld_f32<T>(q, (int64_t)h * d + c);
-      const float kx = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
-      if (tid < d) {
-        qv[tid] = qx;
-        kv[tid] = kx;
-      }
-    }
-    // zero the padded rows of BQ/BK, then scatter the vectors
-    for (int e = tid; e < (32 - r) * ld; e += kSolveThreads) {
-      BQ[r * ld + e] = 0.0f;
-      BK[r * ld + e] = 0.0f;
-    }
+    for (int u = 0; u < 4; ++u) tl4[u] = reinterpret_cast<const float4*>(pr)[tid + u * kSolveThreads];
+    const float pv = pr[4 * 1024 + min(tid, 64)];  // q B_Q^T [32] | k B_K^T [32] | q . k
 #pragma unroll
-    for (int u = 0; u < kMaxVec; ++u) {
-      const int vi = tid + u * kSolveThreads;
-      if (vi < nvec) {
-        const int row = vi >> vshift, c0 = (vi & (vpr - 1)) * VEC;
-        float fq[VEC], fk[VEC];
-        vq[u].unpack(fq);
-        vk[u].unpack(fk);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          BQ[row * ld + c0 + e] = fq[e];
-          BK[row * ld + c0 + e] = fk[e];
-        }
-      }
-    }
+    for (int u = 0; u < 4; ++u) reinterpret_cast<float4*>(cred)[tid + u * kSolveThreads] = tl4[u];
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
       float v = 0.0f;
@@ -325,44 +386,11 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const T* __res
       const int e = tid + u * kSolveThreads;
       if (e < kGramNe) G[e] = v;
     }
-  }
-  __syncthreads();
-  // ---- B_Q B_Q^T and B_K B_K^T on the matrix cores: wave -> (matrix, half of the d axis)
-  {
-    const int col = lane & 31, khalf = lane >> 5;
-    const int which = wave & 1, half = wave >> 1;
-    const float* B = (which ? BK : BQ) + col * ld + khalf;
-    v16f acc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-    const int k1 = (half + 1) * (d / 2);
-#pragma unroll 8
-    for (int kk = half * (d / 2); kk < k1; kk += 2)  // d >= 8 is a power of two
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(B[kk], B[kk], acc, 0, 0, 0);
-    float* mine = cred + (which * 2 + half) * 1024;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) mine[mfma_row(lane, v) * 32 + col] = acc[v];
-  }
-  // rhs_q = q B_Q^T + (q K^T) A ; kB = k B_K^T : thread -> (output i = tid >> 2, quarter of d)
-  {
-    const int i = tid >> 2, qtr = tid & 3;
-    const int which = i >> 5, row = i & 31;
-    const float* B = (which ? BK : BQ) + row * ld;
-    const float* vec = which ? kv : qv;
-    float v = 0.0f;
-#pragma unroll 8
-    for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], B[c], v);
-    v = group_sum(v, 4);
-    if (qtr == 0) {
-      if (which == 0) rhs_q[row] = v + G[32 * 32 + row];
-      else kB[row] = v;
-    }
-  }
-  if (wave == 0) {
-    float v = 0.0f;
-    for (int c = lane; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
-    v = wave_sum(v);
-    if (lane == 0) s_qk = v;
+    // rhs_q = q B_Q^T + (q K^T) A (entry 1024 + row of the summed partials belongs to thread row of u = 4);
+    // kB = k B_K^T
+    if (tid < 32) rhs_q[tid] = pv + gsum[4];
+    else if (tid < 64) kB[tid - 32] = pv;
+    else if (tid == 64) s_qk = pv;
   }
   __syncthreads();
   // columns of [G_K | I] (threads 0..63) and [G_Q | I] (threads 64..127), identity-padded beyond r
@@ -475,21 +503,29 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
   const int64_t a_rows = head_stride / r;
 
-  const size_t smem_solve = ((size_t)2 * 32 * (d + 1) + 2 * d + kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 +
-                             4 * 1024) * sizeof(float);
+  const size_t smem_solve = ((size_t)kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float);
   static size_t solve_allowed = 48 * 1024;
   if (smem_solve > solve_allowed) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_solve_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem_solve));
     solve_allowed = smem_solve;
   }
-  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kGramThreads), 0, st, (const T*)a_k,
-                     head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q, r, d,
-                     lpr_log2, part, S, ap);
+  // the Gram launch carries one more workgroup per head, which needs B_Q and B_K (fp32, padded rows) in LDS
+  const size_t smem_gram = ((size_t)2 * 32 * (d + 1) + 2 * d) * sizeof(float);
+  static size_t gram_allowed = 48 * 1024;
+  if (smem_gram > gram_allowed) {
+    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_gram_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem_gram));
+    gram_allowed = smem_gram;
+  }
+  if ((rc = ctx->als_pre.ensure((size_t)bh * kPreNe * sizeof(float)))) return rc;
+  float* pre = (float*)ctx->als_pre.p;
+  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S + 1, (unsigned)bh), dim3(kGramThreads), smem_gram, st,
+                     (const T*)a_k, head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q,
+                     r, d, lpr_log2, part, S, ap, (const T*)b_q, (const T*)b_k, (const T*)k_new, hq, hkv, pre);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const T*)b_q,
-                     (const T*)b_k, part, S, (const T*)q, (const T*)k_new, hq, hkv, r, d, lpr_log2, max_iter, iter_out,
-                     deltas);
+  hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const float*)pre,
+                     (const float*)part, S, r, max_iter, iter_out, deltas);
   LRQK_HIP_CHECK(hipGetLastError());
   FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
                 head_stride, append_row, nullptr, nullptr, nullptr, 0};

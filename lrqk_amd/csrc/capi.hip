@@ -47,6 +47,7 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->cand_cnt.release();
   ctx->attn_part.release();
   ctx->als_part.release();
+  ctx->als_pre.release();
   ctx->als_iter.release();
   ctx->prefill_ws.release();
   ctx->new_idx.release();

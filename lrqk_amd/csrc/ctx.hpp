@@ -50,6 +50,7 @@ struct lrqk_ctx {
   lrqk::DevBuf cand_cnt;    // per-chunk counts / thresholds
   lrqk::DevBuf attn_part;   // f32 [bh][S][d+2]
   lrqk::DevBuf als_part;    // f32 [bh][S][32*32 + 32]
+  lrqk::DevBuf als_pre;     // f32 [bh][4*1024 + 65]: what the solve needs from B_Q, B_K, q, k (formed beside the Gram pass)
   lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
