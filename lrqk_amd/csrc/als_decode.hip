@@ -50,96 +50,86 @@ struct GramAppend {
 
 // Everything the solve needs from B_Q, B_K, q and the new k -- B_Q B_Q^T and B_K B_K^T (four 32 x 32
 // MFMA tiles: matrix x half of the d axis), q B_Q^T, k B_K^T and q . k -- does not depend on the Gram
-// pass over the active rows, so one more workgroup per head of that launch forms it beside them.
+// pass over the active rows, so two more workgroups per head of that launch form it beside them.
 // out (kPreNe floats per head): tiles [4][1024] | q B_Q^T [32] | k B_K^T [32] | q . k.
 constexpr int kPreNe = 4 * 1024 + 32 + 32 + 1;
 template <typename T>
 __device__ __forceinline__ void als_bgram_body(const T* __restrict__ b_q, const T* __restrict__ b_k,
                                                const T* __restrict__ q, const T* __restrict__ k_new, int h, int hq,
                                                int hkv, int r, int d, int vshift, float* __restrict__ out,
-                                               float* __restrict__ sm) {
+                                               float* __restrict__ sm, int which) {
+  // Two workgroups per head, one per matrix (which = 0: B_Q with q, 1: B_K with k): waves 0 and 1 form the
+  // two half-sums of B B^T, waves 2 and 3 the 32 products with the vector, wave 0 of the first also q . k.
   constexpr int VEC = Vec16<T>::N;
-  constexpr int kMaxVec = 8;  // 16-byte vectors per thread per matrix: r * d / VEC <= 2048
+  constexpr int kMaxVec = 8;  // 16-byte vectors per thread: r * d / VEC <= 2048
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int b = h / hq, head = h % hq;
   const int kvh = head / (hq / hkv);
   const int ld = d + 1;
-  float* BQ = sm;            // [32][d+1]  (rows >= r are zero)
-  float* BK = BQ + 32 * ld;  // [32][d+1]
-  float* qv = BK + 32 * ld;  // [d]
-  float* kv = qv + d;        // [d]
+  float* B = sm;            // [32][d+1]  (rows >= r are zero)
+  float* vec = B + 32 * ld;  // [d]
+  float* oth = vec + d;      // [d] the other vector (for q . k)
+  const T* bsrc = which ? b_k : b_q;
   const int vpr = 1 << vshift;
   const int nvec = r << vshift;
-  Vec16<T> vq[kMaxVec], vk[kMaxVec];
+  Vec16<T> vb[kMaxVec];
 #pragma unroll
   for (int u = 0; u < kMaxVec; ++u) {
     const int vi = min(tid + u * kGramThreads, nvec - 1);
-    vq[u].load(b_q + (int64_t)h * r * d + (int64_t)vi * VEC);
-    vk[u].load(b_k + (int64_t)h * r * d + (int64_t)vi * VEC);
+    vb[u].load(bsrc + (int64_t)h * r * d + (int64_t)vi * VEC);
   }
   {
     const int c = min(tid, d - 1);
     const float qx = ld_f32<T>(q, (int64_t)h * d + c);
     const float kx = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
     if (tid < d) {
-      qv[tid] = qx;
-      kv[tid] = kx;
+      vec[tid] = which ? kx : qx;
+      oth[tid] = which ? qx : kx;
     }
   }
-  // zero the padded rows of BQ/BK, then scatter the vectors
-  for (int e = tid; e < (32 - r) * ld; e += kGramThreads) {
-    BQ[r * ld + e] = 0.0f;
-    BK[r * ld + e] = 0.0f;
-  }
+  for (int e = tid; e < (32 - r) * ld; e += kGramThreads) B[r * ld + e] = 0.0f;
 #pragma unroll
   for (int u = 0; u < kMaxVec; ++u) {
     const int vi = tid + u * kGramThreads;
     if (vi < nvec) {
       const int row = vi >> vshift, c0 = (vi & (vpr - 1)) * VEC;
-      float fq[VEC], fk[VEC];
-      vq[u].unpack(fq);
-      vk[u].unpack(fk);
+      float f[VEC];
+      vb[u].unpack(f);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        BQ[row * ld + c0 + e] = fq[e];
-        BK[row * ld + c0 + e] = fk[e];
-      }
+      for (int e = 0; e < VEC; ++e) B[row * ld + c0 + e] = f[e];
     }
   }
   __syncthreads();
-  // B_Q B_Q^T and B_K B_K^T on the matrix cores: wave -> (matrix, half of the d axis)
-  {
+  if (wave < 2) {
+    // B B^T on the matrix cores: wave -> half of the d axis
     const int col = lane & 31, khalf = lane >> 5;
-    const int which = wave & 1, half = wave >> 1;
-    const float* B = (which ? BK : BQ) + col * ld + khalf;
+    const int half = wave;
+    const float* Bp = B + col * ld + khalf;
     v16f acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
     const int k1 = (half + 1) * (d / 2);
 #pragma unroll 8
     for (int kk = half * (d / 2); kk < k1; kk += 2)  // d >= 8 is a power of two
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(B[kk], B[kk], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Bp[kk], Bp[kk], acc, 0, 0, 0);
     float* mine = out + (which * 2 + half) * 1024;
 #pragma unroll
     for (int v = 0; v < 16; ++v) mine[mfma_row(lane, v) * 32 + col] = acc[v];
-  }
-  // q B_Q^T and k B_K^T : thread -> (output i = tid >> 2, quarter of d)
-  {
-    const int i = tid >> 2, qtr = tid & 3;
-    const int which = i >> 5, row = i & 31;
-    const float* B = (which ? BK : BQ) + row * ld;
-    const float* vec = which ? kv : qv;
+    if (which == 0 && wave == 0) {
+      float v = 0.0f;
+      for (int c = lane; c < d; c += kWave) v = fmaf(vec[c], oth[c], v);
+      v = wave_sum(v);
+      if (lane == 0) out[4 * 1024 + 64] = v;
+    }
+  } else {
+    // vec B^T : thread -> (row = (tid - 128) >> 2, quarter of d)
+    const int i = (tid - 128) >> 2, qtr = tid & 3;
+    const float* Br = B + i * ld;
     float v = 0.0f;
 #pragma unroll 8
-    for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], B[c], v);
+    for (int c = qtr; c < d; c += 4) v = fmaf(vec[c], Br[c], v);
     v = group_sum(v, 4);
-    if (qtr == 0) out[4 * 1024 + which * 32 + row] = v;
-  }
-  if (wave == 0) {
-    float v = 0.0f;
-    for (int c = lane; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
-    v = wave_sum(v);
-    if (lane == 0) out[4 * 1024 + 64] = v;
+    if (qtr == 0) out[4 * 1024 + which * 32 + i] = v;
   }
 }
 
@@ -160,8 +150,8 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
   __shared__ float red[kGramWaves][kGramNe];
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.y, s = blockIdx.x;
-  if (s == S) {  // one workgroup per head beside the S splits
-    als_bgram_body<T>(b_q, b_k, q, k_new, h, hq, hkv, r, d, lpr_log2, pre + (int64_t)h * kPreNe, gram_dyn);
+  if (s >= S) {  // two workgroups per head beside the S splits
+    als_bgram_body<T>(b_q, b_k, q, k_new, h, hq, hkv, r, d, lpr_log2, pre + (int64_t)h * kPreNe, gram_dyn, s - S);
     return;
   }
   float* w_s = w_all[wave];
@@ -510,8 +500,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                                        (int)smem_solve));
     solve_allowed = smem_solve;
   }
-  // the Gram launch carries one more workgroup per head, which needs B_Q and B_K (fp32, padded rows) in LDS
-  const size_t smem_gram = ((size_t)2 * 32 * (d + 1) + 2 * d) * sizeof(float);
+  // the Gram launch carries two more workgroups per head, each with B_Q or B_K (fp32, padded rows) in LDS
+  const size_t smem_gram = ((size_t)32 * (d + 1) + 2 * d) * sizeof(float);
   static size_t gram_allowed = 48 * 1024;
   if (smem_gram > gram_allowed) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_gram_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -520,7 +510,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   }
   if ((rc = ctx->als_pre.ensure((size_t)bh * kPreNe * sizeof(float)))) return rc;
   float* pre = (float*)ctx->als_pre.p;
-  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S + 1, (unsigned)bh), dim3(kGramThreads), smem_gram, st,
+  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S + 2, (unsigned)bh), dim3(kGramThreads), smem_gram, st,
                      (const T*)a_k, head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q,
                      r, d, lpr_log2, part, S, ap, (const T*)b_q, (const T*)b_k, (const T*)k_new, hq, hkv, pre);
   LRQK_HIP_CHECK(hipGetLastError());
