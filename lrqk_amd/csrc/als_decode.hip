@@ -325,12 +325,15 @@ __device__ __forceinline__ float sum_lanes_0_31(float x) {
 
 // iter_out per head: [max_iter][2r] (q_hat then k_hat of each iteration);
 // deltas: [bh][max_iter] sum over r of (k_hat - k_hat')^2.
-template <typename T>
+// KS: compile-time bound of the number of Gram splits S (S <= KS): that many 16-byte loads per thread
+// are in flight for the partial sums, so the bound follows S closely.
+template <int KS>
 __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* __restrict__ pre,
                                                                   const float* __restrict__ part, int S, int r,
                                                                   int max_iter, float* __restrict__ iter_out,
                                                                   float* __restrict__ deltas) {
-  constexpr int kMaxSplit = 32;
+  static_assert(kGramNe % 4 == 0 && kGramNe / 4 - kSolveThreads <= kWave && kGramNe / 4 > kSolveThreads,
+                "a partial is one 16-byte vector per thread plus a few more for the first wave");
   extern __shared__ __align__(16) float sm[];
   __shared__ float s_qk;
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
@@ -351,15 +354,16 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
   // ---- every global load of the kernel is issued here, back to back
   const float* pin = part + (int64_t)h * S * kGramNe;
   const float* pr = pre + (int64_t)h * kPreNe;
-  constexpr int kPer = (kGramNe + kSolveThreads - 1) / kSolveThreads;  // 5 entries per thread
-  float gsum[kPer];
   {
-    float x[kPer][kMaxSplit];
+    // a partial is kGramNe / 4 = 264 vectors: one per thread, the last 8 (the A^T w column) in the first wave
+    constexpr int kVec = kGramNe / 4;
+    const float4* pin4 = reinterpret_cast<const float4*>(pin);
+    float4 x[KS], y[KS];
 #pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      const int e = tid + u * kSolveThreads;
+    for (int t = 0; t < KS; ++t) x[t] = pin4[(int64_t)min(t, S - 1) * kVec + tid];
+    if (wave == 0) {
 #pragma unroll
-      for (int t = 0; t < kMaxSplit; ++t) x[u][t] = pin[(int64_t)min(t, S - 1) * kGramNe + min(e, kGramNe - 1)];
+      for (int t = 0; t < KS; ++t) y[t] = pin4[(int64_t)min(t, S - 1) * kVec + min(kSolveThreads + tid, kVec - 1)];
     }
     float4 tl4[4];  // the four B B^T tiles: 4096 floats, 16 per thread
 #pragma unroll
@@ -367,22 +371,26 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
     const float pv = pr[4 * 1024 + min(tid, 64)];  // q B_Q^T [32] | k B_K^T [32] | q . k
 #pragma unroll
     for (int u = 0; u < 4; ++u) reinterpret_cast<float4*>(cred)[tid + u * kSolveThreads] = tl4[u];
+    auto sum_splits = [&](const float4 (&v)[KS]) {  // fixed order 0..S-1, element-wise
+      float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      float v = 0.0f;
-#pragma unroll
-      for (int t = 0; t < kMaxSplit; ++t) v += (t < S) ? x[u][t] : 0.0f;  // fixed order 0..S-1
-      gsum[u] = v;
-      const int e = tid + u * kSolveThreads;
-      if (e < kGramNe) G[e] = v;
-    }
-    // rhs_q = q B_Q^T + (q K^T) A (entry 1024 + row of the summed partials belongs to thread row of u = 4);
-    // kB = k B_K^T
-    if (tid < 32) rhs_q[tid] = pv + gsum[4];
+      for (int t = 0; t < KS; ++t) {
+        a.x += (t < S) ? v[t].x : 0.0f;
+        a.y += (t < S) ? v[t].y : 0.0f;
+        a.z += (t < S) ? v[t].z : 0.0f;
+        a.w += (t < S) ? v[t].w : 0.0f;
+      }
+      return a;
+    };
+    reinterpret_cast<float4*>(G)[tid] = sum_splits(x);
+    if (wave == 0 && kSolveThreads + tid < kVec) reinterpret_cast<float4*>(G)[kSolveThreads + tid] = sum_splits(y);
+    // rhs_q = q B_Q^T + (q K^T) A: the second term (G[1024 + i]) is added after the barrier; kB = k B_K^T
+    if (tid < 32) rhs_q[tid] = pv;
     else if (tid < 64) kB[tid - 32] = pv;
     else if (tid == 64) s_qk = pv;
   }
   __syncthreads();
+  if (tid < 32) rhs_q[tid] += G[32 * 32 + tid];  // (read again only after the barriers of the inversion)
   // columns of [G_K | I] (threads 0..63) and [G_Q | I] (threads 64..127), identity-padded beyond r
   {
     float colv[32];
@@ -404,7 +412,6 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
       const float eye = (i == jj) ? 1.0f : 0.0f;
       colv[i] = j < 32 ? ((i < r && j < r) ? g : eye) : eye;
     }
-    (void)gsum;
     invert_pair_regs(colv, Mx, GKi, GQi);
   }
   // ---- k_hat_0 and the alternating rank-1 solves, all inside the first wave: lane c (and c + 32)
@@ -494,12 +501,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   const int64_t a_rows = head_stride / r;
 
   const size_t smem_solve = ((size_t)kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float);
-  static size_t solve_allowed = 48 * 1024;
-  if (smem_solve > solve_allowed) {
-    LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_solve_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem_solve));
-    solve_allowed = smem_solve;
-  }
+  static_assert(((size_t)kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float) <= 48 * 1024,
+                "the solve kernel's LDS fits the default dynamic limit");
   // the Gram launch carries two more workgroups per head, each with B_Q or B_K (fp32, padded rows) in LDS
   const size_t smem_gram = ((size_t)32 * (d + 1) + 2 * d) * sizeof(float);
   static size_t gram_allowed = 48 * 1024;
@@ -514,8 +517,20 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                      (const T*)a_k, head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q,
                      r, d, lpr_log2, part, S, ap, (const T*)b_q, (const T*)b_k, (const T*)k_new, hq, hkv, pre);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((als_solve_kernel<T>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const float*)pre,
-                     (const float*)part, S, r, max_iter, iter_out, deltas);
+#define LRQK_SOLVE_CASE(KS)                                                                                     \
+  hipLaunchKernelGGL((als_solve_kernel<KS>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const float*)pre, \
+                     (const float*)part, S, r, max_iter, iter_out, deltas)
+  switch ((S + 3) / 4) {
+    case 1: LRQK_SOLVE_CASE(4); break;
+    case 2: LRQK_SOLVE_CASE(8); break;
+    case 3: LRQK_SOLVE_CASE(12); break;
+    case 4: LRQK_SOLVE_CASE(16); break;
+    case 5: LRQK_SOLVE_CASE(20); break;
+    case 6: LRQK_SOLVE_CASE(24); break;
+    case 7: LRQK_SOLVE_CASE(28); break;
+    default: LRQK_SOLVE_CASE(32); break;
+  }
+#undef LRQK_SOLVE_CASE
   LRQK_HIP_CHECK(hipGetLastError());
   FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
                 head_stride, append_row, nullptr, nullptr, nullptr, 0};

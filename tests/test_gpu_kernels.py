@@ -452,6 +452,17 @@ def _als_inputs(g, b, hq, hkv, n, d, r, cap, dtype):
                                                 (torch.bfloat16, 32, 8, 2112, 128, 32), (torch.float32, 2, 2, 70, 8, 3)])
 @pytest.mark.parametrize("max_iter,tol", [(1, 0.0), (2, 0.0), (3, 1e30), (4, 1e-6)])
 def test_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
+    _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol)
+
+
+@pytest.mark.parametrize("n", [1100, 2000, 2700, 3500, 4160, 6000])
+def test_als_decode_split_counts(ops, ws, oracle, n):
+    """The Gram sums arrive in ceil(n / 128) partials (at most 32) and the solve kernel is compiled per
+    group of four of that count: one case per group not met by the shapes above."""
+    _check_als_decode(ops, ws, oracle, torch.float32, 2, 1, n, 64, 16, 2, 0.0)
+
+
+def _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     _say("als_decode", dtype, hq, n, d, r, max_iter, tol)
     g = torch.Generator().manual_seed(n + r)
     b, cap = 1, 3 * n
