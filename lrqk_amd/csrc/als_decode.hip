@@ -317,6 +317,65 @@ __device__ __forceinline__ void invert_pair_regs(float (&colv)[32], float* cbuf,
   __syncthreads();
 }
 
+// Inverse of one SPD 32 x 32 matrix by one wave, as 32 symmetric sweeps on the matrix cores.  The
+// matrix sits in the accumulator layout of the 32x32x2 fp32 MFMA (acc[v] of lane l: row mfma_row(l, v),
+// column l % 32).  A sweep on pivot p (d = a_pp) maps
+//   a_ij -> a_ij - a_ip a_pj / d,   a_ip -> a_ip / d,   a_pj -> a_pj / d,   a_pp -> -1 / d,
+// keeps the matrix symmetric and, after all p, leaves -G^-1.  All four cases are one rank-2 update
+// acc -= A B with operands made from row p alone (held by the lanes of one half: by symmetry it is also
+// column p): A_i = a_pi / d, B_j = a_pj, except A_p = 1 - 1/d and B_p = d - 1 (which turn row and column p
+// into a_p. / d), and the second rank, supplied by the other half, subtracts 2 at (p, p).  B_p = d - 1
+// cancels badly for large d, so the matrix is first scaled to unit diagonal (then every pivot is <= 1);
+// the scaling is undone on the way out.  Rows and columns >= r are an identity block and are skipped.
+// g(i, j) returns element (i, j); sbuf: 32 floats of LDS owned by this wave; inv: [32][kLdi].
+template <typename GetG>
+__device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, float* inv) {
+  const int lane = lane_id();
+  const int col = lane & 31, half = lane >> 5;
+  v16f acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    const float x = g(i, col);
+    acc[v] = (i < r && col < r) ? x : (i == col ? 1.0f : 0.0f);
+  }
+  const float s_col = col < r ? __builtin_amdgcn_rsqf(g(col, col)) : 1.0f;
+  if (lane < 32) sbuf[lane] = s_col;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  float sc[16];  // s_row * s_col of every element this lane holds
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const float4 s4 = reinterpret_cast<const float4*>(sbuf)[2 * a + half];  // rows 8a + 4 half + 0..3
+    sc[4 * a + 0] = s4.x * s_col;
+    sc[4 * a + 1] = s4.y * s_col;
+    sc[4 * a + 2] = s4.z * s_col;
+    sc[4 * a + 3] = s4.w * s_col;
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] *= sc[v];
+#pragma unroll
+  for (int p = 0; p < 32; ++p) {
+    if (p < r) {  // (wave-uniform)
+      const int v = ((p >> 3) << 2) + (p & 3), hp = (p >> 2) & 1;
+      const float rv = acc[v];
+      const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rv), p + 32 * hp));
+      float rc = __builtin_amdgcn_rcpf(d);
+      rc = fmaf(fmaf(-d, rc, 1.0f), rc, rc);
+      const bool inhalf = half == hp, isp = col == p;
+      const float A = inhalf ? (isp ? 1.0f - rc : rv * rc) : (isp ? 2.0f : 0.0f);
+      const float B = inhalf ? (isp ? d - 1.0f : rv) : (isp ? 1.0f : 0.0f);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, B, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    inv[i * kLdi + col] = (i < r && col < r) ? -acc[v] * sc[v] : (i == col ? 1.0f : 0.0f);
+  }
+}
+
 // Sum of x over lanes 0..31 of the wave (the first two rows of 16 lanes); every lane must call it.
 __device__ __forceinline__ float sum_lanes_0_31(float x) {
   x = row_reduce(x, [](float a, float b) { return a + b; });
@@ -391,29 +450,14 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
   }
   __syncthreads();
   if (tid < 32) rhs_q[tid] += G[32 * 32 + tid];  // (read again only after the barriers of the inversion)
-  // columns of [G_K | I] (threads 0..63) and [G_Q | I] (threads 64..127), identity-padded beyond r
-  {
-    float colv[32];
-    const int mat = (tid >> 6) & 1, j = tid & 63;
-    // all LDS reads first (independent, so they pipeline), then the selects
-    const float* c0 = cred + (mat ? 0 : 2048);
-    const float gsel = mat ? 1.0f : 0.0f;
-    const int jj = j & 31;
-    float a0[32], a1[32], gg[32];
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      a0[i] = c0[i * 32 + jj];
-      a1[i] = c0[1024 + i * 32 + jj];
-      gg[i] = G[i * 32 + jj];
-    }
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      const float g = fmaf(gsel, gg[i], a0[i] + a1[i]);
-      const float eye = (i == jj) ? 1.0f : 0.0f;
-      colv[i] = j < 32 ? ((i < r && j < r) ? g : eye) : eye;
-    }
-    invert_pair_regs(colv, Mx, GKi, GQi);
+  // G_K = B_K B_K^T (first wave) and G_Q = B_Q B_Q^T + A^T A (second wave), each inverted by its wave
+  if (wave < 2) {
+    const float* c0 = cred + (wave ? 0 : 2048);
+    const float gsel = wave ? 1.0f : 0.0f;
+    auto elem = [&](int i, int j) { return fmaf(gsel, G[i * 32 + j], c0[i * 32 + j] + c0[1024 + i * 32 + j]); };
+    invert_sweep_mfma(elem, r, Mx + 32 * wave, wave ? GQi : GKi);
   }
+  __syncthreads();
   // ---- k_hat_0 and the alternating rank-1 solves, all inside the first wave: lane c (and c + 32)
   // holds column c of both inverses and element c of every vector; a vector element is
   // broadcast with readlane, so the chain of small solves needs no barrier and no LDS round trip.
