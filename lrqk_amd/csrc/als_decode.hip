@@ -21,10 +21,9 @@
 #include "common.hpp"
 #include "ctx.hpp"
 #include "als_finish.hpp"
+#include "small_inverse.hpp"
 
 namespace lrqk {
-
-typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGramThreads = 256;
 constexpr int kGramWaves = kGramThreads / kWave;
@@ -32,8 +31,6 @@ constexpr int kGramChunk = 32;  // tokens per wave per chunk = 16 MFMA steps
 constexpr int kGramNe = 32 * 32 + 32;
 constexpr int kSolveThreads = 256;
 
-// C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
-__device__ __forceinline__ int mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
 
 // Ring append folded into the Gram pass: slot `slot` (>= 0) of every head is the new token.  The
 // pass takes its K row from k_new and its token id from `token` instead of the buffers, and the
@@ -266,116 +263,6 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
 
 // Everything in the solve kernel works on 32 x 32 tiles padded with an identity block (rows
 // and columns >= r), so every loop has a compile-time trip count and its LDS reads pipeline.
-constexpr int kLdm = 65;  // row stride of an augmented [G | I] matrix (64 columns)
-constexpr int kLdi = 33;  // row stride of an inverse
-
-// Gauss-Jordan inversion of two SPD 32 x 32 matrices at once, no pivoting.  Threads 0..127:
-// thread (mat, j) keeps column j of the augmented matrix [G | I] of matrix `mat` in registers
-// (colv, rows 0..31); per pivot the pivot column is broadcast through LDS (cbuf: [2][2][32]
-// floats, 16-byte aligned) and the pivot row is normalised, so on return the identity half
-// holds the inverse: inv{0,1}[i][c] = colv[i] of thread (mat, 32 + c).  Every thread of the
-// workgroup must call it (one barrier per pivot).
-__device__ __forceinline__ void invert_pair_regs(float (&colv)[32], float* cbuf, float* inv0, float* inv1) {
-  const int tid = threadIdx.x;
-  const int mat = (tid >> 6) & 1, j = tid & 63;
-  const bool act = tid < 128;
-  // The rows are rotated by one after every pivot, so the pivot is always element 0 and the
-  // loop body is the same code for every p (a rolled loop: straight-line code for 32 pivots
-  // would be executed once per workgroup from a cold instruction cache).
-  // Each matrix belongs to one wave (64 columns), so the exchange needs no workgroup barrier.
-  // Four pivots per trip with static register indices, then one rotation by four rows.
-  if (act) {
-#pragma unroll 1
-    for (int p0 = 0; p0 < 32; p0 += 4) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        // the pivot column lives in lane p0 + q of this wave: broadcast it lane -> scalar registers
-        float cb[32];
-#pragma unroll
-        for (int i = 0; i < 32; ++i)
-          cb[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(colv[i]), p0 + q));
-        // reciprocal of the pivot: hardware estimate + one Newton step (error below 1 ulp)
-        float rc = __builtin_amdgcn_rcpf(cb[q]);
-        rc = fmaf(fmaf(-cb[q], rc, 1.0f), rc, rc);
-        const float mp = colv[q] * rc;
-#pragma unroll
-        for (int i = 0; i < 32; ++i)
-          if (i != q) colv[i] = fmaf(-cb[i], mp, colv[i]);
-        colv[q] = mp;
-      }
-      float t0 = colv[0], t1 = colv[1], t2 = colv[2], t3 = colv[3];
-#pragma unroll
-      for (int i = 0; i < 28; ++i) colv[i] = colv[i + 4];
-      colv[28] = t0; colv[29] = t1; colv[30] = t2; colv[31] = t3;
-    }
-  }
-  if (act && j >= 32) {
-    float* inv = mat ? inv1 : inv0;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) inv[i * kLdi + (j - 32)] = colv[i];
-  }
-  __syncthreads();
-}
-
-// Inverse of one SPD 32 x 32 matrix by one wave, as 32 symmetric sweeps on the matrix cores.  The
-// matrix sits in the accumulator layout of the 32x32x2 fp32 MFMA (acc[v] of lane l: row mfma_row(l, v),
-// column l % 32).  A sweep on pivot p (d = a_pp) maps
-//   a_ij -> a_ij - a_ip a_pj / d,   a_ip -> a_ip / d,   a_pj -> a_pj / d,   a_pp -> -1 / d,
-// keeps the matrix symmetric and, after all p, leaves -G^-1.  All four cases are one rank-2 update
-// acc -= A B with operands made from row p alone (held by the lanes of one half: by symmetry it is also
-// column p): A_i = a_pi / d, B_j = a_pj, except A_p = 1 - 1/d and B_p = d - 1 (which turn row and column p
-// into a_p. / d), and the second rank, supplied by the other half, subtracts 2 at (p, p).  B_p = d - 1
-// cancels badly for large d, so the matrix is first scaled to unit diagonal (then every pivot is <= 1);
-// the scaling is undone on the way out.  Rows and columns >= r are an identity block and are skipped.
-// g(i, j) returns element (i, j); sbuf: 32 floats of LDS owned by this wave; inv: [32][kLdi].
-template <typename GetG>
-__device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, float* inv) {
-  const int lane = lane_id();
-  const int col = lane & 31, half = lane >> 5;
-  v16f acc;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int i = mfma_row(lane, v);
-    const float x = g(i, col);
-    acc[v] = (i < r && col < r) ? x : (i == col ? 1.0f : 0.0f);
-  }
-  const float s_col = col < r ? __builtin_amdgcn_rsqf(g(col, col)) : 1.0f;
-  if (lane < 32) sbuf[lane] = s_col;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  float sc[16];  // s_row * s_col of every element this lane holds
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const float4 s4 = reinterpret_cast<const float4*>(sbuf)[2 * a + half];  // rows 8a + 4 half + 0..3
-    sc[4 * a + 0] = s4.x * s_col;
-    sc[4 * a + 1] = s4.y * s_col;
-    sc[4 * a + 2] = s4.z * s_col;
-    sc[4 * a + 3] = s4.w * s_col;
-  }
-#pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] *= sc[v];
-#pragma unroll
-  for (int p = 0; p < 32; ++p) {
-    if (p < r) {  // (wave-uniform)
-      const int v = ((p >> 3) << 2) + (p & 3), hp = (p >> 2) & 1;
-      const float rv = acc[v];
-      const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rv), p + 32 * hp));
-      float rc = __builtin_amdgcn_rcpf(d);
-      rc = fmaf(fmaf(-d, rc, 1.0f), rc, rc);
-      const bool inhalf = half == hp, isp = col == p;
-      const float A = inhalf ? (isp ? 1.0f - rc : rv * rc) : (isp ? 2.0f : 0.0f);
-      const float B = inhalf ? (isp ? d - 1.0f : rv) : (isp ? 1.0f : 0.0f);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, B, acc, 0, 0, 0);
-    }
-  }
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int i = mfma_row(lane, v);
-    inv[i * kLdi + col] = (i < r && col < r) ? -acc[v] * sc[v] : (i == col ? 1.0f : 0.0f);
-  }
-}
-
 // Sum of x over lanes 0..31 of the wave (the first two rows of 16 lanes); every lane must call it.
 __device__ __forceinline__ float sum_lanes_0_31(float x) {
   x = row_reduce(x, [](float a, float b) { return a + b; });
@@ -398,8 +285,8 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
   const int h = blockIdx.x;
   float* G = sm;                    // [kGramNe] summed A^T [A | w]
-  float* Mx = G + kGramNe;          // pivot-column exchange buffers of the inversion (16-byte aligned)
-  float* GKi = Mx + 2 * 32 * kLdm;  // [32][kLdi]
+  float* Mx = G + kGramNe;          // [2][32] row scales of the two inversions (16-byte aligned)
+  float* GKi = Mx + 2 * 32;         // [32][kLdi]
   float* GQi = GKi + 32 * kLdi;     // [32][kLdi]
   float* rhs_q = GQi + 32 * kLdi;   // 6 vectors of 32
   float* kB = rhs_q + 32;
@@ -544,8 +431,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
   const int64_t a_rows = head_stride / r;
 
-  const size_t smem_solve = ((size_t)kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float);
-  static_assert(((size_t)kGramNe + 2 * 32 * kLdm + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float) <= 48 * 1024,
+  const size_t smem_solve = ((size_t)kGramNe + 2 * 32 + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float);
+  static_assert(((size_t)kGramNe + 2 * 32 + 2 * 32 * kLdi + 6 * 32 + 4 * 1024) * sizeof(float) <= 48 * 1024,
                 "the solve kernel's LDS fits the default dynamic limit");
   // the Gram launch carries two more workgroups per head, each with B_Q or B_K (fp32, padded rows) in LDS
   const size_t smem_gram = ((size_t)32 * (d + 1) + 2 * d) * sizeof(float);

@@ -16,6 +16,7 @@
 
 #include "common.hpp"
 #include "ctx.hpp"
+#include "small_inverse.hpp"
 
 namespace lrqk {
 
@@ -506,39 +507,45 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_mfma_kernel(const T* __res
   }
 }
 
-// ---- small per-head systems, r <= 32: every thread keeps one column of the augmented matrix
-// [G (32 x 32, identity beyond r) | RHS (32 x d)] in registers; per pivot the pivot column is
-// broadcast through LDS.  No pivoting: G is a Gram matrix (plus B B^T), positive definite.
+// ---- small per-head systems, r <= 32: X = G^-1 RHS for a packed block [G (r x r) | RHS (r x d)] in LDS.
+// One wave inverts G (symmetric sweeps on the matrix cores); the product is formed 32 columns of the
+// right-hand side at a time, again on the matrix cores, by whichever wave takes the block.  No pivoting:
+// G is a Gram matrix (plus B B^T), positive definite.
 struct PfSmallShared {
-  __align__(16) float cbuf[2][32];
+  __align__(16) float scale[2][32];    // row scales of up to two inversions in flight
+  __align__(16) float inv[2][32 * kLdi];
 };
 
-// col[i], i < 32: this thread's column.  On return the RHS columns hold G^-1 RHS.
-__device__ __forceinline__ void pf_solve32(float (&colv)[32], PfSmallShared& sh) {
-  const int tid = threadIdx.x;
-  // The rows are rotated by one after every pivot, so the pivot is always element 0 and the
-  // loop body is the same code for every p (a rolled loop keeps the code small: it runs once
-  // per workgroup, from a cold instruction cache).
-#pragma unroll 1
-  for (int p = 0; p < 32; ++p) {
-    float4* cb4 = reinterpret_cast<float4*>(sh.cbuf[p & 1]);
-    if (tid == p) {
+// the inverse of the r x r block of G0 (row stride r + d), by the calling wave
+__device__ __forceinline__ void pf_invert(const float* G0, int r, int d, float* scale, float* inv) {
+  const int ld = r + d;
+  invert_sweep_mfma([&](int i, int j) { return G0[min(i, r - 1) * ld + min(j, r - 1)]; }, r, scale, inv);
+}
+
+// columns [32 cb, 32 cb + 32) of X = inv * RHS, by the calling wave; emit(i, j, x) for i < r, j < d
+template <typename Emit>
+__device__ __forceinline__ void pf_apply_inverse(const float* inv, const float* G0, int r, int d, int cb, Emit&& emit) {
+  const int lane = lane_id();
+  const int col = lane & 31, half = lane >> 5;
+  const int j = cb * 32 + col, ld = r + d;
+  float a[16], b[16];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) cb4[i] = make_float4(colv[4 * i], colv[4 * i + 1], colv[4 * i + 2], colv[4 * i + 3]);
-    }
-    __syncthreads();
-    float cb[32];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float4 t = cb4[i];
-      cb[4 * i] = t.x; cb[4 * i + 1] = t.y; cb[4 * i + 2] = t.z; cb[4 * i + 3] = t.w;
-    }
-    const float mp = colv[0] * (1.0f / cb[0]);
-#pragma unroll
-    for (int i = 0; i < 31; ++i) colv[i] = fmaf(-cb[i + 1], mp, colv[i + 1]);
-    colv[31] = mp;
+  for (int kk = 0; kk < 16; ++kk) {
+    const int k = 2 * kk + half;
+    a[kk] = inv[col * kLdi + k];
+    const float x = G0[min(k, r - 1) * ld + r + min(j, d - 1)];
+    b[kk] = (k < r && j < d) ? x : 0.0f;
   }
-  __syncthreads();
+  v16f acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+#pragma unroll
+  for (int kk = 0; kk < 16; ++kk) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc, 0, 0, 0);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    if (i < r && j < d) emit(i, j, acc[v]);
+  }
 }
 
 // sum of the S partial [r][r+d] blocks; 16 elements x 8 partials of loads in flight per thread
@@ -564,22 +571,6 @@ __device__ __forceinline__ void pf_reduce_part(const float* __restrict__ part, i
 #pragma unroll
     for (int q = 0; q < EB; ++q)
       if (e0 + q * kPfSmallThreads < ne) dst[e0 + q * kPfSmallThreads] = v[q];
-  }
-}
-
-// Column `tid` of [G | RHS] from a packed [r][r+d] block G0 (+ optional additions), identity-padded.
-__device__ __forceinline__ void pf_load_col(const float* G0, int r, int d, float (&colv)[32]) {
-  const int j = threadIdx.x;  // < 32: system column, else RHS column j - 32
-#pragma unroll
-  for (int i = 0; i < 32; ++i) {
-    float v = 0.0f;
-    if (j < 32) {
-      if (i < r && j < r) v = G0[i * (r + d) + j];
-      else if (i == j) v = 1.0f;
-    } else if (j - 32 < d && i < r) {
-      v = G0[i * (r + d) + r + (j - 32)];
-    }
-    colv[i] = v;
   }
 }
 
@@ -628,7 +619,9 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
   __shared__ float s_red[kPfSmallThreads / kWave][2];
   const int tid = threadIdx.x;
   const int h = blockIdx.x;
-  float colv[32];
+  const int wave = wave_id();
+  constexpr int kWaves = kPfSmallThreads / kWave;
+  const int nblk = (d + 31) / 32;  // 32-column blocks of a right-hand side
 
   if (stage == 0) {
     int done = 0;
@@ -675,24 +668,20 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
     pf_reduce_part(pq, S, ne, G1);
     pf_reduce_part(pk, S, ne, G2);
     __syncthreads();
-    // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q
-    pf_load_col(G1, r, d, colv);
-    pf_solve32(colv, sh);
-    if (tid >= 32 && tid - 32 < d) {
-#pragma unroll
-      for (int i = 0; i < 32; ++i)
-        if (i < r) {
-          Bs[i * (d + 4) + tid - 32] = colv[i];
-          b_q[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
-        }
-    }
-    // B_K
-    pf_load_col(G2, r, d, colv);
-    pf_solve32(colv, sh);
-    if (tid >= 32 && tid - 32 < d) {
-#pragma unroll
-      for (int i = 0; i < 32; ++i)
-        if (i < r) b_k[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
+    // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q and B_K likewise: the two inverses side by side, then all blocks
+    if (wave == 0) pf_invert(G1, r, d, sh.scale[0], sh.inv[0]);
+    else if (wave == 1) pf_invert(G2, r, d, sh.scale[1], sh.inv[1]);
+    __syncthreads();
+    for (int job = wave; job < 2 * nblk; job += kWaves) {
+      if (job < nblk) {
+        pf_apply_inverse(sh.inv[0], G1, r, d, job, [&](int i, int j, float x) {
+          Bs[i * (d + 4) + j] = x;
+          b_q[(int64_t)h * r * d + i * d + j] = x;
+        });
+      } else {
+        pf_apply_inverse(sh.inv[1], G2, r, d, job - nblk,
+                         [&](int i, int j, float x) { b_k[(int64_t)h * r * d + i * d + j] = x; });
+      }
     }
     if (stage == 2) return;
     __syncthreads();
@@ -706,13 +695,10 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
     pf_add_bbt(G1, Bs, r, d, G0);
   }
   __syncthreads();
-  pf_load_col(G0, r, d, colv);
-  pf_solve32(colv, sh);
-  if (tid >= 32 && tid - 32 < d) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i)
-      if (i < r) Mt[(int64_t)h * r * d + i * d + tid - 32] = colv[i];
-  }
+  if (wave == 0) pf_invert(G0, r, d, sh.scale[0], sh.inv[0]);
+  __syncthreads();
+  for (int job = wave; job < nblk; job += kWaves)
+    pf_apply_inverse(sh.inv[0], G0, r, d, job, [&](int i, int j, float x) { Mt[(int64_t)h * r * d + i * d + j] = x; });
 }
 
 template <typename T>

@@ -1,0 +1,74 @@
+// Inverse of a small symmetric positive definite matrix on the matrix cores, shared by the decode
+// and the prefill half of the factorisation.
+#pragma once
+#include "common.hpp"
+
+namespace lrqk {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// C tile of mfma_f32_32x32x2f32: lane l, element v -> row (the column is l & 31)
+__device__ __forceinline__ int mfma_row(int lane, int v) { return ((v >> 2) << 3) + ((lane >> 5) << 2) + (v & 3); }
+
+constexpr int kLdi = 33;  // row stride of an inverse in LDS
+
+// Inverse of one SPD 32 x 32 matrix by one wave, as 32 symmetric sweeps on the matrix cores.  The
+// matrix sits in the accumulator layout of the 32x32x2 fp32 MFMA (acc[v] of lane l: row mfma_row(l, v),
+// column l % 32).  A sweep on pivot p (d = a_pp) maps
+//   a_ij -> a_ij - a_ip a_pj / d,   a_ip -> a_ip / d,   a_pj -> a_pj / d,   a_pp -> -1 / d,
+// keeps the matrix symmetric and, after all p, leaves -G^-1.  All four cases are one rank-2 update
+// acc -= A B with operands made from row p alone (held by the lanes of one half: by symmetry it is also
+// column p): A_i = a_pi / d, B_j = a_pj, except A_p = 1 - 1/d and B_p = d - 1 (which turn row and column p
+// into a_p. / d), and the second rank, supplied by the other half, subtracts 2 at (p, p).  B_p = d - 1
+// cancels badly for large d, so the matrix is first scaled to unit diagonal (then every pivot is <= 1);
+// the scaling is undone on the way out.  Rows and columns >= r are an identity block and are skipped.
+// g(i, j) returns element (i, j); sbuf: 32 floats of LDS owned by this wave; inv: [32][kLdi].
+template <typename GetG>
+__device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, float* inv) {
+  const int lane = lane_id();
+  const int col = lane & 31, half = lane >> 5;
+  v16f acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    const float x = g(i, col);
+    acc[v] = (i < r && col < r) ? x : (i == col ? 1.0f : 0.0f);
+  }
+  const float s_col = col < r ? __builtin_amdgcn_rsqf(g(col, col)) : 1.0f;
+  if (lane < 32) sbuf[lane] = s_col;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  float sc[16];  // s_row * s_col of every element this lane holds
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const float4 s4 = reinterpret_cast<const float4*>(sbuf)[2 * a + half];  // rows 8a + 4 half + 0..3
+    sc[4 * a + 0] = s4.x * s_col;
+    sc[4 * a + 1] = s4.y * s_col;
+    sc[4 * a + 2] = s4.z * s_col;
+    sc[4 * a + 3] = s4.w * s_col;
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] *= sc[v];
+#pragma unroll
+  for (int p = 0; p < 32; ++p) {
+    if (p < r) {  // (wave-uniform)
+      const int v = ((p >> 3) << 2) + (p & 3), hp = (p >> 2) & 1;
+      const float rv = acc[v];
+      const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rv), p + 32 * hp));
+      float rc = __builtin_amdgcn_rcpf(d);
+      rc = fmaf(fmaf(-d, rc, 1.0f), rc, rc);
+      const bool inhalf = half == hp, isp = col == p;
+      const float A = inhalf ? (isp ? 1.0f - rc : rv * rc) : (isp ? 2.0f : 0.0f);
+      const float B = inhalf ? (isp ? d - 1.0f : rv) : (isp ? 1.0f : 0.0f);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, B, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    inv[i * kLdi + col] = (i < r && col < r) ? -acc[v] * sc[v] : (i == col ? 1.0f : 0.0f);
+  }
+}
+
+}  // namespace lrqk
