@@ -368,17 +368,21 @@ __global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* _
       return y0 + y1;
     };
     auto dot32 = [&](float a, float bb) { return sum_lanes_0_31(a * bb); };
-    // x = b (G + v^T v)^-1 from G^-1 (Sherman-Morrison): x = y - (y.v / (1 + z.v)) z, y = b G^-1, z = v G^-1
-    auto rank1 = [&](float bvec, float v, const float (&col)[32]) {
-      const float y = vecmat(bvec, col);
+    // x = b (G + v^T v)^-1 from G^-1 (Sherman-Morrison): x = y - (y.v / (1 + z.v)) z, y = b G^-1, z = v G^-1.
+    // Both right-hand sides have the form b = b0 + s v, so y = b0 G^-1 + s z: b0 G^-1 is formed once
+    // (for the k side it is k_hat_0 itself) and every solve costs one vector-matrix product.
+    auto rank1 = [&](float y0, float v, const float (&col)[32]) {
       const float z = vecmat(v, col);
+      const float y = fmaf(sqk, z, y0);
       const float alpha = dot32(y, v) / (1.0f + dot32(z, v));
       return fmaf(-alpha, z, y);
     };
-    float hk = vecmat(kb, cK);  // k_hat_0 = kB G_K^-1
+    const float hk0 = vecmat(kb, cK);  // k_hat_0 = kB G_K^-1
+    const float yq0 = vecmat(rq, cQ);  // rhs_q G_Q^-1
+    float hk = hk0;
     for (int it = 0; it < max_iter; ++it) {
-      const float hq = rank1(fmaf(sqk, hk, rq), hk, cQ);  // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
-      const float nk = rank1(fmaf(sqk, hq, kb), hq, cK);  // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat
+      const float hq = rank1(yq0, hk, cQ);  // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
+      const float nk = rank1(hk0, hq, cK);  // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat
       const float df = c < r ? hk - nk : 0.0f;
       const float dsq = dot32(df, df);
       if (lane == 0) deltas[(int64_t)h * max_iter + it] = dsq;
