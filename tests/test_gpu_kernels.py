@@ -487,6 +487,39 @@ def _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     assert torch.equal(ad[:, :, :cap - 1].cpu(), A[:, :, :cap - 1])         # nothing else touched
 
 
+def test_als_decode_ill_conditioned(ops, ws, oracle):
+    """Factors whose Gram matrices have condition numbers around 1e5 and entries far from 1 (what a real
+    stream produces: the r x r inverses run in fp32 without pivoting, on the matrix scaled to unit
+    diagonal).  The same bound against fp64 as for well-conditioned factors must hold."""
+    _say("als_decode ill-conditioned")
+    g = torch.Generator().manual_seed(77)
+    b, hq, hkv, n, d, r, cap = 1, 4, 2, 300, 64, 32, 640
+    x = _als_inputs(g, b, hq, hkv, n, d, r, cap, torch.float32)
+    spec = torch.logspace(0, -2.5, r)                      # singular values over 2.5 decades: cond(G) ~ 1e5
+    x["A"] = x["A"] * spec * 40.0                          # and a diagonal far above 1
+    x["B_Q"] = x["B_Q"] * spec.unsqueeze(-1) * 25.0
+    x["B_K"] = x["B_K"] * spec.unsqueeze(-1) * 25.0
+    idx = torch.stack([torch.randperm(cap - 1, generator=g)[:n] for _ in range(b * hq)]).view(b, hq, n)
+    A = x["A"].clone()
+    A[:, :, cap - 1] = 0
+    A_act = torch.take_along_dim(A, idx.unsqueeze(-1), 2)
+    G_Q = x["B_Q"].double() @ x["B_Q"].double().transpose(-1, -2) + A_act.double().transpose(-1, -2) @ A_act.double()
+    cond = torch.linalg.cond(G_Q).max().item()
+    assert 1e3 < cond < 1e7, cond
+    repk = oracle.repeat_kv(x["k"], hq // hkv)
+    ref = oracle.als_decode_w1(x["B_Q"].double(), A_act.double(), x["B_K"].double(), x["Kp"].double(),
+                               x["q"].double(), repk.double(), 2, 0.0)
+    bq, bk, ad = x["B_Q"].to(DEV), x["B_K"].to(DEV), A.to(DEV)
+    qh, kh = ops.als_decode(ws, bq, bk, ad, idx.to(torch.int32).to(DEV), x["Kp"].to(DEV), n, x["q"].to(DEV),
+                            x["k"].to(DEV), 2, 0.0, append_row=cap - 1)
+    lim = 2e-4  # as for well-conditioned factors (measured 1e-6 at cond 1.3e5)
+    for name, got, exp in (("q_hat", qh, ref[2]), ("k_hat", kh, ref[3])):
+        assert torch.isfinite(got).all(), name
+        rel = (got.cpu().double() - exp).norm() / exp.norm()
+        print(name, "cond %.2e rel %.2e lim %.2e" % (cond, float(rel), lim), flush=True)
+        assert rel < lim, (name, float(rel), cond)
+
+
 def test_als_decode_prefix_branch(ops, ws, oracle):
     """active_idx = NULL: rows 0..n-1 of A_K (the growing-prefix branch)."""
     _say("als_decode prefix")
