@@ -222,9 +222,14 @@ __device__ __forceinline__ void als_finish_body(const FinishArgs& fa, int h) {
       const int64_t off = (int64_t)h * r * d + (int64_t)vi * VEC;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        st_f32<T>(b_q, off + e, fq[e] - sq * err[0][cg * VEC + e]);
-        st_f32<T>(b_k, off + e, fk[e] - sk * err[1][cg * VEC + e]);
+        fq[e] -= sq * err[0][cg * VEC + e];
+        fk[e] -= sk * err[1][cg * VEC + e];
       }
+      Vec16<T> oq, ok;  // one 16-byte store per vector (b_q, b_k are 16-byte aligned: they are read that way)
+      oq.pack(fq);
+      ok.pack(fk);
+      oq.store(b_q + off);
+      ok.store(b_k + off);
     }
   }
   if (tid < r) {

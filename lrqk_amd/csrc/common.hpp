@@ -81,6 +81,8 @@ struct Vec16<float> {
   __device__ __forceinline__ void unpack(float* f) const {
     f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w;
   }
+  __device__ __forceinline__ void pack(const float* f) { raw = make_float4(f[0], f[1], f[2], f[3]); }
+  __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = raw; }
 };
 template <>
 struct Vec16<bf16_t> {
@@ -93,6 +95,14 @@ struct Vec16<bf16_t> {
     f[4] = __uint_as_float(raw.z << 16); f[5] = __uint_as_float(raw.z & 0xffff0000u);
     f[6] = __uint_as_float(raw.w << 16); f[7] = __uint_as_float(raw.w & 0xffff0000u);
   }
+  // rounds like st_f32 (to nearest even)
+  __device__ __forceinline__ void pack(const float* f) {
+    raw.x = (uint32_t)f32_to_bf16_bits(f[0]) | ((uint32_t)f32_to_bf16_bits(f[1]) << 16);
+    raw.y = (uint32_t)f32_to_bf16_bits(f[2]) | ((uint32_t)f32_to_bf16_bits(f[3]) << 16);
+    raw.z = (uint32_t)f32_to_bf16_bits(f[4]) | ((uint32_t)f32_to_bf16_bits(f[5]) << 16);
+    raw.w = (uint32_t)f32_to_bf16_bits(f[6]) | ((uint32_t)f32_to_bf16_bits(f[7]) << 16);
+  }
+  __device__ __forceinline__ void store(bf16_t* p) const { *reinterpret_cast<uint4*>(p) = raw; }
 };
 
 // ----------------------------------------------------------------------------- score keys
