@@ -65,6 +65,10 @@ def parse():
     p.add_argument("--batch", type=int, default=4, help="decoder mode: sequences")
     p.add_argument("--prompt", type=int, default=65536, help="decoder mode: prompt tokens per sequence")
     p.add_argument("--new-tokens", type=int, default=128, help="decoder mode: tokens decoded per sequence")
+    p.add_argument("--rotate", type=int, default=1,
+                   help="decode mode: step this many independent copies of the layer's state in turn (as the layers "
+                        "of a decoder do), so that no copy finds its buffers in the 256 MB last-level cache; the "
+                        "value stays the time per layer-step; counters and kernel timing are taken from the first copy")
     p.add_argument("--calib-copy-mb", type=int, default=0,
                    help="after the timed region, run one plain device copy of this many MiB (a known-size "
                         "kernel to scale hardware counters by)")
@@ -211,19 +215,27 @@ def main():
     Q, K, V, bases, gen = synth.prompt_qkv(w, a.seed, l, device=dev)
     A0 = synth.init_factors(w, l, a.seed + 1, device=dev)
     cls = lrqk_amd.LightAttentionIndicesNoHitMiss if a.variant == "no_hit_miss" else lrqk_amd.LightAttentionIndicesFactory
-    eng = cls(num_lite_tokens=w.lite_tokens, attn_topk=w.num_active_tokens, num_key_value_groups=w.groups, r=w.r,
-              max_iter=w.max_iter, tol=w.tol, capacity=4096)
-    eng.init_factors = A0
-    eng.attn_in_step = not a.no_attn
-    eng.fetch_mode = a.fetch
-    eng.use_score_index = not a.no_score_index
-    if a.victim_rows >= 0:
-        eng.victim_rows = a.victim_rows
+    def make_engine():
+        e_ = cls(num_lite_tokens=w.lite_tokens, attn_topk=w.num_active_tokens, num_key_value_groups=w.groups, r=w.r,
+                 max_iter=w.max_iter, tol=w.tol, capacity=4096)
+        e_.init_factors = A0
+        e_.attn_in_step = not a.no_attn
+        e_.fetch_mode = a.fetch
+        e_.use_score_index = not a.no_score_index
+        if a.victim_rows >= 0:
+            e_.victim_rows = a.victim_rows
+        return e_
+    eng = make_engine()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     eng.prefill(Q, K, V)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
+    others = []
+    for _ in range(max(1, a.rotate) - 1):  # further copies of the same layer state, each with buffers of its own
+        o_ = make_engine()
+        o_.prefill(Q, K, V)
+        others.append(o_)
     del A0
     stream = synth.DecodeStream(w, Q[:, :, -1:], bases, gen)
     total = a.warmup + a.steps
@@ -234,14 +246,17 @@ def main():
     del Q, K, V
     torch.cuda.empty_cache()
     # reserve so that no step of the timed region allocates or grows a buffer
-    eng.ws.reserve(w.batch * w.num_heads, l + total + 64, w.num_active_tokens,
-                   w.num_active_tokens + w.lite_tokens, w.r, w.head_dim)
+    for e_ in [eng] + others:
+        e_.ws.reserve(w.batch * w.num_heads, l + total + 64, w.num_active_tokens,
+                      w.num_active_tokens + w.lite_tokens, w.r, w.head_dim)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
 
     miss = sel = 0
     for i in range(a.warmup):
         eng.decode(qs[i], ks[i], vs[i])
+        for o_ in others:
+            o_.decode(qs[i], ks[i], vs[i])
     torch.cuda.synchronize()
     cap_before = (eng._A_K.capacity, eng.KVcpu.capacity)
     m_first = eng.lite_indices[eng.lite_len] - 1
@@ -255,8 +270,10 @@ def main():
     for i in range(a.warmup, total):
         eng.decode(qs[i], ks[i], vs[i])
         counts.append(eng.last_miss_count)
+        for o_ in others:
+            o_.decode(qs[i], ks[i], vs[i])
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    elapsed = (time.perf_counter() - t0) / (1 + len(others))
     kern_ms, launches = eng.ws.timing_read()
     eng.ws.timing_enable(0)
     sel_fast, sel_full = eng.ws.select_stats()
@@ -284,6 +301,8 @@ def main():
 
     sidx_on = (not a.no_score_index) and w.r in (16, 32, 64)
     traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) if a.context is None and a.variant == "default" else None
+    if others:
+        traffic = None  # the counters were read on a single copy
 
     if a.calib_copy_mb > 0:
         src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -320,7 +339,8 @@ def main():
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
                    "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
-                   "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last]},
+                   "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last],
+                   "layer_copies": 1 + len(others)},
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
