@@ -507,6 +507,251 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_mfma_kernel(const T* __res
   }
 }
 
+// ---- the same pass for bf16 input on the bf16 matrix cores (16 x the fp32 MFMA rate), without giving up
+// fp32 accuracy: an fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8 mantissa bits, by
+// truncation), a product of two bf16 numbers is exact in fp32, and the MFMA accumulates in fp32.  So
+//   apply:  C = X Mt^T            = X (Mt_hi + Mt_mid + Mt_lo)^T            (X is bf16 as it is: 3 products)
+//   gram:   G_AX += C^T X         = (C_hi + C_mid + C_lo)^T X                (3 products)
+//           G_AA += C^T C         ~ all piece pairs except mid*lo, lo*mid, lo*lo (6 products, error 2^-24)
+// with 32x32x16 tiles.  The Gram products sum over the rows of the tile, and C comes out of the apply in
+// the accumulator layout (lane l, element v: row pf_mfma_row(l, v), column l % 32), where a lane holds
+// rows 4 h .. 4 h + 3 (+ 8, 16, 24) of its column, h = l / 32: taken eight at a time these are the k
+// elements of an MFMA operand, in an order that does not matter as long as the other operand uses the
+// same one.  X gets into that layout by a product with the identity (2 MFMAs per 32 columns, exact).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// the three bf16 pieces of x (as the upper halves of fp32 bit patterns)
+__device__ __forceinline__ void pf_split3(float x, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+  hi = __float_as_uint(x) & 0xffff0000u;
+  const float r1 = x - __uint_as_float(hi);  // exact
+  mid = __float_as_uint(r1) & 0xffff0000u;
+  const float r2 = r1 - __uint_as_float(mid);  // exact, at most 8 significant bits
+  lo = __float_as_uint(r2) & 0xffff0000u;
+}
+// two bf16 values (upper halves of a, b) in one word, a first
+__device__ __forceinline__ uint32_t pf_pack2(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
+__device__ __forceinline__ bf16x8 pf_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  return __builtin_bit_cast(bf16x8, make_uint4(a, b, c, d));
+}
+
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* __restrict__ X, int xh, int hq,
+                                                                  int64_t l, int r, int d,
+                                                                  const float* __restrict__ Mt, float* __restrict__ A,
+                                                                  float* __restrict__ part,
+                                                                  float* __restrict__ delta_part,
+                                                                  const int* __restrict__ done_flag, int S) {
+  if (done_flag && *done_flag) return;
+  constexpr int LDB = 32 * NB + 8;  // row stride of a bf16 tile (elements)
+  constexpr int KB = 2 * NB;        // 16-column blocks of X
+  constexpr int VEC = 8;
+  constexpr int NL = 32 * 32 * NB / (kWave * VEC);
+  constexpr int NT = NW * kWave;
+  extern __shared__ __align__(16) float sm[];
+  __shared__ float red[NW];
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int col = lane & 31, half = lane >> 5;
+  uint16_t* x_s = reinterpret_cast<uint16_t*>(sm) + wave * 32 * LDB;           // this wave's rows of X
+  uint16_t* mt_s = reinterpret_cast<uint16_t*>(sm) + NW * 32 * LDB;            // [3][32][LDB] pieces of Mt
+  const int h = blockIdx.y, s = blockIdx.x;
+  const int b = h / hq, head = h % hq;
+  const int64_t xhead = (int64_t)b * xh + head / (hq / xh);
+  const bf16_t* Xh = X + xhead * l * d;
+  float* Ah = A + (int64_t)h * l * r;
+  const bool apply = Mt != nullptr;
+  const bool full_rows = d == 32 * NB;
+
+  if (apply) {
+    const float* Mh = Mt + (int64_t)h * r * d;
+    for (int e = tid; e < 32 * 32 * NB; e += NT) {
+      const int n = e / (32 * NB), k = e % (32 * NB);
+      const float v = Mh[min(n, r - 1) * d + min(k, d - 1)];
+      uint32_t p0, p1, p2;
+      pf_split3((n < r && k < d) ? v : 0.0f, p0, p1, p2);
+      mt_s[(0 * 32 + n) * LDB + k] = (uint16_t)(p0 >> 16);
+      mt_s[(1 * 32 + n) * LDB + k] = (uint16_t)(p1 >> 16);
+      mt_s[(2 * 32 + n) * LDB + k] = (uint16_t)(p2 >> 16);
+    }
+  }
+  for (int e = lane; e < 32 * LDB / 2; e += kWave) reinterpret_cast<uint32_t*>(x_s)[e] = 0u;
+
+  const int64_t rows_per_split = (((l + S - 1) / S) + 31) / 32 * 32;
+  const int64_t r0 = (int64_t)s * rows_per_split;
+  const int64_t r1 = min(l, r0 + rows_per_split);
+
+  floatx16 gAA;
+  floatx16 gAX[NB];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) gAA[v] = 0.0f;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) gAX[nb][v] = 0.0f;
+  float dsum = 0.0f;
+  // B operand of the identity product for the two 16-column halves of a 32-column block: element j of
+  // lane (col, half) is row 16 kb2 + 8 half + j of the identity, column col
+  bf16x8 ident[2];
+#pragma unroll
+  for (int kb2 = 0; kb2 < 2; ++kb2) {
+    uint32_t w[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int k0 = 16 * kb2 + 8 * half + 2 * jj;
+      w[jj] = (col == k0 ? 0x3f80u : 0u) | (col == k0 + 1 ? 0x3f800000u : 0u);  // bf16 1.0 = 0x3f80
+    }
+    ident[kb2] = pf_bf16x8(w[0], w[1], w[2], w[3]);
+  }
+
+  uint4 pre[NL];
+  auto issue = [&](int64_t t0) {
+    const int nvalid = t0 < r1 ? (int)min((int64_t)32, r1 - t0) * d : 0;
+    const int64_t base = (t0 < r1 ? t0 : r0) * d;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int e = (i * kWave + lane) * VEC;
+      pre[i] = *reinterpret_cast<const uint4*>(Xh + base + (e < nvalid ? e : 0));
+    }
+  };
+  if (r0 + (int64_t)wave * 32 < r1) issue(r0 + (int64_t)wave * 32);
+  __syncthreads();  // Mt staged, tiles cleared
+
+  for (int64_t t0 = r0 + (int64_t)wave * 32; t0 < r1; t0 += 32 * NW) {
+    const int rows = (int)min((int64_t)32, r1 - t0);
+    {
+      const int nvalid = rows * d;
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int e = (i * kWave + lane) * VEC;
+        if (e < 32 * d) {
+          const int row = full_rows ? e / (32 * NB) : e / d;
+          const int c0 = full_rows ? e % (32 * NB) : e - row * d;
+          *reinterpret_cast<uint4*>(&x_s[row * LDB + c0]) = e < nvalid ? pre[i] : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+    pf_wave_sync();
+    if (t0 + 32 * NW < r1) issue(t0 + 32 * NW);
+
+    floatx16 c;
+    float old[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
+      old[v] = Ah[rr * r + min(col, r - 1)];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) c[v] = 0.0f;
+    auto x_op = [&](int kb) {  // rows of X as an A operand: row col, columns 16 kb + 8 half .. + 7
+      return *reinterpret_cast<const bf16x8*>(&x_s[col * LDB + kb * 16 + 8 * half]);
+    };
+    if (apply) {
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        const bf16x8 a = x_op(kb);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+          const bf16x8 m = *reinterpret_cast<const bf16x8*>(&mt_s[(p * 32 + col) * LDB + kb * 16 + 8 * half]);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, m, c, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = pf_mfma_row(lane, v);
+        if (row < rows && col < r) {
+          const float df = old[v] - c[v];
+          dsum = fmaf(df, df, dsum);
+          Ah[(t0 + row) * r + col] = c[v];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) c[v] = (pf_mfma_row(lane, v) < rows && col < r) ? old[v] : 0.0f;
+    }
+    // the three pieces of C, eight rows (one k block) at a time
+    bf16x8 cp[3][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      uint32_t pc[3][8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pf_split3(c[8 * kb + j], pc[0][j], pc[1][j], pc[2][j]);
+#pragma unroll
+      for (int p = 0; p < 3; ++p)
+        cp[p][kb] = pf_bf16x8(pf_pack2(pc[p][0], pc[p][1]), pf_pack2(pc[p][2], pc[p][3]), pf_pack2(pc[p][4], pc[p][5]),
+                              pf_pack2(pc[p][6], pc[p][7]));
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[0][kb], gAA, 0, 0, 0);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[1][kb], gAA, 0, 0, 0);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[0][kb], gAA, 0, 0, 0);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[1][kb], gAA, 0, 0, 0);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[2][kb], gAA, 0, 0, 0);
+      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[2][kb], cp[0][kb], gAA, 0, 0, 0);
+    }
+    // per 32 columns of X: the block in the accumulator layout (identity product), packed to bf16 --
+    // xb[kb] = this lane's eight rows of k block kb, column 32 nb + col -- then its Gram products
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      floatx16 xa;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) xa[v] = 0.0f;
+      xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb), ident[0], xa, 0, 0, 0);
+      xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb + 1), ident[1], xa, 0, 0, 0);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const bf16x8 xb =
+            pf_bf16x8(pf_pack2(__float_as_uint(xa[8 * kb + 0]), __float_as_uint(xa[8 * kb + 1])),
+                      pf_pack2(__float_as_uint(xa[8 * kb + 2]), __float_as_uint(xa[8 * kb + 3])),
+                      pf_pack2(__float_as_uint(xa[8 * kb + 4]), __float_as_uint(xa[8 * kb + 5])),
+                      pf_pack2(__float_as_uint(xa[8 * kb + 6]), __float_as_uint(xa[8 * kb + 7])));
+#pragma unroll
+        for (int p = 0; p < 3; ++p) gAX[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[p][kb], xb, gAX[nb], 0, 0, 0);
+      }
+    }
+    pf_wave_sync();  // this wave's reads of the tile precede its next staging writes
+  }
+  __syncthreads();  // every wave is done with its tile (and with Mt): the LDS is reused below
+
+  // reduce the waves' tiles through LDS, one 32 x 32 block at a time (tile nb of G_AX: columns 32 nb + n)
+  const int ne = r * (r + d);
+  float* out = part + ((int64_t)h * S + s) * ne;
+  for (int blk = 0; blk <= NB; ++blk) {
+    float* mine = sm + wave * 1024;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      float val = gAA[v];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        if (blk == nb + 1) val = gAX[nb][v];
+      mine[pf_mfma_row(lane, v) * 32 + col] = val;
+    }
+    __syncthreads();
+    for (int e = tid; e < 1024; e += NT) {
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v += sm[w * 1024 + e];
+      const int m = e >> 5, n = e & 31;
+      if (blk == 0) {
+        if (m < r && n < r) out[m * (r + d) + n] = v;
+      } else {
+        const int cx = 32 * (blk - 1) + n;
+        if (m < r && cx < d) out[m * (r + d) + r + cx] = v;
+      }
+    }
+    __syncthreads();
+  }
+  if (apply) {
+    dsum = wave_sum(dsum);
+    if (lane == 0) red[wave] = dsum;
+    __syncthreads();
+    if (tid == 0) {
+      float t = 0.0f;
+      for (int w = 0; w < NW; ++w) t += red[w];
+      delta_part[(int64_t)h * S + s] = t;
+    }
+  }
+}
+
 // ---- small per-head systems, r <= 32: X = G^-1 RHS for a packed block [G (r x r) | RHS (r x d)] in LDS.
 // One wave inverts G (symmetric sweeps on the matrix cores); the product is formed 32 columns of the
 // right-hand side at a time, again on the matrix cores, by whichever wave takes the block.  No pivoting:
@@ -742,6 +987,12 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
     const int nw = nb == 8 ? 4 : 8;
     pass_threads = nw * kWave;
     smem_pass = std::max((size_t)(nw + (nb == 8 ? 0 : 1)) * 32 * (32 * nb + 4), (size_t)nw * 1024) * sizeof(float);
+    if constexpr (sizeof(T) == 2) {
+      if (nb <= 4) {  // bf16 input: the pass on the bf16 matrix cores (three-piece split, fp32 accuracy)
+        pass = nb == 1 ? pf_pass_bf16_kernel<1, 8> : nb == 2 ? pf_pass_bf16_kernel<2, 8> : pf_pass_bf16_kernel<4, 8>;
+        smem_pass = std::max((size_t)(8 + 3) * 32 * (32 * nb + 8) * sizeof(uint16_t), (size_t)8 * 1024 * sizeof(float));
+      }
+    }
   }
   auto small = small32 ? pf_small32_kernel : pf_small_generic_kernel;
   const size_t smem_small = small32 ? ((size_t)3 * ne + 4 + (size_t)r * (d + 4)) * sizeof(float)
