@@ -143,8 +143,8 @@ def prefill_als(a):
         # bf16 input: the passes run on the bf16 matrix cores (fp32 operands as three bf16 pieces), where the
         # arithmetic is far from any limit; what bounds them is the stream over X and A
         gbs = bytes_ / (ms * 1e-3) / 1e9
-        # executed bf16 flops: per 32 rows 24 (apply) + 8 (identity) + 24 + 12 (Grams) MFMAs of 32x32x16
-        mf_apply, mf_gram = 68, 44
+        # executed bf16 flops: per 32 rows 24 (apply) + 8 (identity) + 24 + 16 (Grams) MFMAs of 32x32x16
+        mf_apply, mf_gram = 72, 48
         exec_flops = bh * (l / 32.0) * (2 * mf_gram + iters * 2 * mf_apply) * 2.0 * 32 * 32 * 16
         roof = {"bound": "hbm", "kernel": "pf_pass_bf16_kernel", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,

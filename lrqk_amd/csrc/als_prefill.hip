@@ -512,7 +512,9 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_mfma_kernel(const T* __res
 // truncation), a product of two bf16 numbers is exact in fp32, and the MFMA accumulates in fp32.  So
 //   apply:  C = X Mt^T            = X (Mt_hi + Mt_mid + Mt_lo)^T            (X is bf16 as it is: 3 products)
 //   gram:   G_AX += C^T X         = (C_hi + C_mid + C_lo)^T X                (3 products)
-//           G_AA += C^T C         ~ all piece pairs except mid*lo, lo*mid, lo*lo (6 products, error 2^-24)
+//           G_AA += C^T C         = all piece pairs except lo*lo (8 products, error 2^-32; the pieces of a number
+//                                   share its sign, so dropping mid*lo as well would bias the diagonal by ~2^-24,
+//                                   which the r x r systems amplify by their condition number)
 // with 32x32x16 tiles.  The Gram products sum over the rows of the tile, and C comes out of the apply in
 // the accumulator layout (lane l, element v: row pf_mfma_row(l, v), column l % 32), where a lane holds
 // rows 4 h .. 4 h + 3 (+ 8, 16, 24) of its column, h = l / 32: taken eight at a time these are the k
@@ -679,14 +681,31 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
         cp[p][kb] = pf_bf16x8(pf_pack2(pc[p][0], pc[p][1]), pf_pack2(pc[p][2], pc[p][3]), pf_pack2(pc[p][4], pc[p][5]),
                               pf_pack2(pc[p][6], pc[p][7]));
     }
+    // The matrix cores do not round to nearest when they add to their accumulator: over thousands of
+    // additions to a growing sum that is a bias (measured: -2e-5 relative on a sum of 16K squares, ten times
+    // the fp32 pipe's).  So a tile's products are summed in a fresh accumulator, smallest pieces first, and
+    // the tile's sum joins the running total by an ordinary fp32 addition.
+    {
+      floatx16 t;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[0][kb], gAA, 0, 0, 0);
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[1][kb], gAA, 0, 0, 0);
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[0][kb], gAA, 0, 0, 0);
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[1][kb], gAA, 0, 0, 0);
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[2][kb], gAA, 0, 0, 0);
-      gAA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[2][kb], cp[0][kb], gAA, 0, 0, 0);
+      for (int v = 0; v < 16; ++v) t[v] = 0.0f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[2][kb], t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[2][kb], cp[1][kb], t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[2][kb], t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[2][kb], cp[0][kb], t, 0, 0, 0);
+      }
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[1][kb], t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[1][kb], t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[1][kb], cp[0][kb], t, 0, 0, 0);
+      }
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[0][kb], cp[0][kb], t, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) gAA[v] += t[v];
     }
     // per 32 columns of X: the block in the accumulator layout (identity product), packed to bf16 --
     // xb[kb] = this lane's eight rows of k block kb, column 32 nb + col -- then its Gram products
@@ -697,16 +716,22 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       for (int v = 0; v < 16; ++v) xa[v] = 0.0f;
       xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb), ident[0], xa, 0, 0, 0);
       xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb + 1), ident[1], xa, 0, 0, 0);
+      bf16x8 xb[2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const bf16x8 xb =
-            pf_bf16x8(pf_pack2(__float_as_uint(xa[8 * kb + 0]), __float_as_uint(xa[8 * kb + 1])),
-                      pf_pack2(__float_as_uint(xa[8 * kb + 2]), __float_as_uint(xa[8 * kb + 3])),
-                      pf_pack2(__float_as_uint(xa[8 * kb + 4]), __float_as_uint(xa[8 * kb + 5])),
-                      pf_pack2(__float_as_uint(xa[8 * kb + 6]), __float_as_uint(xa[8 * kb + 7])));
+      for (int kb = 0; kb < 2; ++kb)
+        xb[kb] = pf_bf16x8(pf_pack2(__float_as_uint(xa[8 * kb + 0]), __float_as_uint(xa[8 * kb + 1])),
+                           pf_pack2(__float_as_uint(xa[8 * kb + 2]), __float_as_uint(xa[8 * kb + 3])),
+                           pf_pack2(__float_as_uint(xa[8 * kb + 4]), __float_as_uint(xa[8 * kb + 5])),
+                           pf_pack2(__float_as_uint(xa[8 * kb + 6]), __float_as_uint(xa[8 * kb + 7])));
+      floatx16 t;
 #pragma unroll
-        for (int p = 0; p < 3; ++p) gAX[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[p][kb], xb, gAX[nb], 0, 0, 0);
-      }
+      for (int v = 0; v < 16; ++v) t[v] = 0.0f;
+#pragma unroll
+      for (int p = 2; p >= 0; --p)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[p][kb], xb[kb], t, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) gAX[nb][v] += t[v];
     }
     pf_wave_sync();  // this wave's reads of the tile precede its next staging writes
   }

@@ -538,6 +538,26 @@ def test_als_decode_prefix_branch(ops, ws, oracle):
 
 # ---------------------------------------------------------------- ALS prefill
 
+def test_als_prefill_long_sums(ops, ws, oracle):
+    """The Gram sums of a 128K prompt, bf16 input: the first B factors (no iteration: two Gram passes and the
+    r x r solves, on well-conditioned random factors) against fp64.  The matrix cores do not round to nearest
+    when they accumulate, which biases long sums of squares (2.2e-6 here when a whole split of the long axis
+    is summed inside one accumulator); summed tile by tile the result stays below the fp32 pipe's 8.4e-7."""
+    _say("als_prefill long sums")
+    g = torch.Generator().manual_seed(5)
+    b, hq, hkv, l, d, r = 1, 2, 1, 131072, 128, 32
+    Q = torch.randn((b, hq, l, d), generator=g).to(torch.bfloat16)
+    K = torch.randn((b, hkv, l, d), generator=g).to(torch.bfloat16)
+    A_Q0 = torch.randn((b, hq, l, r), generator=g)
+    A_K0 = torch.randn((b, hq, l, r), generator=g)
+    ref = oracle.als_prefill_w1(Q.double(), oracle.repeat_kv(K, hq // hkv).double(), A_Q0.double(), A_K0.double(), 0, 0.0)
+    got = ops.als_prefill(ws, Q.to(DEV), K.to(DEV), A_Q0.to(DEV), A_K0.to(DEV), 0, 0.0)
+    for name, x, y in (("B_Q", got[1], ref[1]), ("B_K", got[3], ref[3])):
+        rel = float((x.cpu().double() - y).norm() / y.norm())
+        print(name, "rel err %.3e" % rel, flush=True)
+        assert rel < 7e-7, (name, rel)
+
+
 @pytest.mark.parametrize("dtype,hq,hkv,l,d,r,iters,tol",
                          [(torch.float32, 4, 2, 40, 16, 4, 2, 0.0), (torch.float32, 4, 2, 700, 16, 4, 0, 0.0),
                           (torch.float32, 28, 4, 1024, 128, 16, 1, 1e-2), (torch.bfloat16, 8, 2, 3000, 128, 32, 3, 0.0),
