@@ -563,7 +563,11 @@ def test_als_prefill_long_sums(ops, ws, oracle):
                           (torch.float32, 28, 4, 1024, 128, 16, 1, 1e-2), (torch.bfloat16, 8, 2, 3000, 128, 32, 3, 0.0),
                           (torch.float32, 2, 1, 333, 8, 3, 6, 1e30), (torch.float32, 2, 1, 333, 8, 3, 6, 5e-2),
                           (torch.bfloat16, 4, 2, 1500, 64, 8, 2, 0.0), (torch.bfloat16, 2, 2, 777, 256, 32, 2, 0.0),
-                          (torch.bfloat16, 2, 1, 500, 12, 4, 2, 0.0), (torch.float32, 2, 1, 4500, 96, 24, 2, 0.0)])
+                          (torch.bfloat16, 2, 1, 500, 12, 4, 2, 0.0), (torch.float32, 2, 1, 4500, 96, 24, 2, 0.0),
+                          # bf16 input on the bf16 matrix cores: d = 96 (rows not a whole number of 32-column
+                          # blocks), one block, a prompt shorter than one tile, a ragged last tile per split
+                          (torch.bfloat16, 2, 1, 1000, 96, 24, 2, 0.0), (torch.bfloat16, 2, 2, 333, 32, 16, 2, 0.0),
+                          (torch.bfloat16, 2, 1, 37, 64, 8, 1, 0.0), (torch.bfloat16, 4, 1, 20011, 128, 32, 2, 0.0)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
