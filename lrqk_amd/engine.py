@@ -238,7 +238,10 @@ class LightAttentionIndicesFactory:
             self._hit_len = k
         else:
             self.KVcpu.append(key_states, value_states)
-            hit = self.compute_hit_indices(query_states=A_Q[:, :, -1:, :], key_states=A_K[:, :, 0:seq_len - L, :])
+            # the rows are scanned where they will live (same values as A_K, which sync_cache copied there): the
+            # score index that this first scan builds then stays valid for the decode steps
+            hit = self.compute_hit_indices(query_states=A_Q[:, :, -1:, :],
+                                           key_states=self._A_K.data.narrow(2, 0, seq_len - L))
             self._hit_len = hit.shape[2]
             self._active_idx[:, :, :self._hit_len] = hit[..., 0].to(torch.int32)
             self.fetch_by_hit(dst=self.Kgpu_topk_area, src=key_states, hit_indices=hit)
