@@ -283,13 +283,14 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     marks = []
+    chunk = max(8, 64 // (1 + len(others)))  # (64 layer-steps per chunk, however many copies take turns)
     for i in range(a.warmup, total):
         # The host enqueues a step in less than half the time the GPU needs for it.  Left alone it runs thousands
         # of launches ahead, and once the runtime's launch queue is full (at about 2000 launches here) every
         # further launch waits in a way that leaves gaps on the GPU (512 steps: 128 us per step instead of 86).
         # So the host stays at most 128 steps ahead: it waits for the mark recorded two chunks of 64 steps ago,
         # which the GPU passed long before, and the GPU never runs dry.
-        if (i - a.warmup) % 64 == 0:
+        if (i - a.warmup) % chunk == 0:
             marks.append(torch.cuda.Event())
             marks[-1].record()
             if len(marks) > 2:
