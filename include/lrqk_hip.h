@@ -165,6 +165,17 @@ int lrqk_flush_ring(const void* k_act, const void* v_act, int n_slots, int slot0
 int lrqk_attention(lrqk_ctx* ctx, const void* q, const void* k_act, const void* v_act, int n_slots,
                    int n_valid, void* out, int bh, int d, int dtype, void* stream);
 
+/* No counterpart in the reference.  The same attention as lrqk_attention for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops and harnesses that forbid
+ * hipMalloc): it takes no ctx and allocates nothing; its split partial results live in a fixed
+ * 4 MiB block of the library's own device memory (one per GPU, held until the process ends).
+ * Limit: bh * min(64, ceil(n_valid / 64)) * (d + 2) <= 1048576, else LRQK_ELIMIT.  All calls on one
+ * GPU share that block: calls that overlap on one GPU (different streams or threads) race; calls on
+ * one stream are ordered.  The block needs no clearing between calls (every entry that is read was
+ * written by the same call). */
+int lrqk_attention_static(const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
+                          void* out, int bh, int d, int dtype, void* stream);
+
 /* py:803-839 cast_lrqk_decode -> py:529-628 _lrqk_decode_inv_w1 + py:651-665 -- the per-step
  * factor update.  b_q,b_k: [bh][r][d] storage dtype, updated in place.  The active A_K rows
  * are gathered from a_k (heads of head_stride elements) at active_idx[bh][0..n) (py:1156-1171);

@@ -59,6 +59,7 @@ def _sig(lib):
         "lrqk_append_token": ([vp, vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_flush_ring": ([vp, vp, i32, i32, i32, vp, i64, i64, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_attention": ([vp, vp, vp, vp, i32, i32, vp, i32, i32, i32, vp], i32),
+        "lrqk_attention_static": ([vp, vp, vp, i32, i32, vp, i32, i32, i32, vp], i32),
         "lrqk_als_decode": ([vp, vp, vp, vp, i64, vp, i64, vp, i32, i32, vp, vp, i32, i32, i32, i32, i32, i32, f32,
                              vp, vp, i64, i32, vp], i32),
         "lrqk_als_prefill": ([vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i64, i32, i32, i32, f32, i32, vp], i32),

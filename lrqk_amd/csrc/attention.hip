@@ -10,6 +10,8 @@
 // kernel then adds the freshly fetched slots of its head before merging.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "ctx.hpp"
 #include "rows.hpp"
@@ -492,25 +494,80 @@ static int attn_shape(int d, int vec, int* lpr_log2) {
   return LRQK_OK;
 }
 
+// Number of slot-axis splits of the stand-alone attention.
+static int attn_splits(int n_valid) {
+  int S = (n_valid + 63) / 64;
+  if (S < 1) S = 1;
+  if (S > 64) S = 64;
+  return S;
+}
+
+// The two launches of the stand-alone attention; `part` holds bh * S * (d + 2) floats.  Every triple of
+// `part` is written by the first launch (an empty split writes an empty triple), so it needs no clearing.
+template <typename T>
+static int attention_launch(const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid, void* out,
+                            int bh, int d, int lpr_log2, int S, float* part, hipStream_t st) {
+  const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
+  hipLaunchKernelGGL((attn_partial_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kAttnThreads), 0, st,
+                     (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, n_valid, d, lpr_log2, scale_log2e, part, S);
+  LRQK_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st, (const float*)part, S, d,
+                     (T*)out);
+  LRQK_HIP_CHECK(hipGetLastError());
+  return LRQK_OK;
+}
+
 template <typename T>
 static int attention_impl(lrqk_ctx* ctx, const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
                           void* out, int bh, int d, hipStream_t st) {
   int lpr_log2 = 0;
   int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
   if (rc) return rc;
-  int S = (n_valid + 63) / 64;
-  if (S < 1) S = 1;
-  if (S > 64) S = 64;
+  const int S = attn_splits(n_valid);
   if ((rc = ctx->attn_part.ensure((size_t)bh * S * (d + 2) * sizeof(float)))) return rc;
-  const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
-  hipLaunchKernelGGL((attn_partial_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kAttnThreads), 0, st,
-                     (const T*)q, (const T*)k_act, (const T*)v_act, n_slots, n_valid, d, lpr_log2, scale_log2e,
-                     (float*)ctx->attn_part.p, S);
-  LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
-                     (const float*)ctx->attn_part.p, S, d, (T*)out);
-  LRQK_HIP_CHECK(hipGetLastError());
+  return attention_launch<T>(q, k_act, v_act, n_slots, n_valid, out, bh, d, lpr_log2, S, (float*)ctx->attn_part.p, st);
+}
+
+// ----------------------------------------------------------------------------- attention without allocation
+// Split partials of lrqk_attention_static: a fixed block in the code object's own device memory, one copy per
+// GPU the library runs on, held until the process ends.
+constexpr size_t kStaticPartFloats = (size_t)1 << 20;  // 4 MiB
+static __device__ __align__(256) float g_attn_static_part[kStaticPartFloats];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_static_mu;
+static float* g_static_part_ptr[kMaxDevices];  // device address of the block on each GPU (nullptr: not asked yet)
+
+// Device address of g_attn_static_part on the current GPU (resolved once per device).
+static int static_part(float** out) {
+  int dev = 0;
+  LRQK_HIP_CHECK(hipGetDevice(&dev));
+  LRQK_REQUIRE(dev >= 0 && dev < kMaxDevices, LRQK_ELIMIT, "device ordinal %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_part_ptr[dev]) {
+    float* p = nullptr;
+    LRQK_HIP_CHECK(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(g_attn_static_part)));
+    LRQK_REQUIRE(p != nullptr, LRQK_EHIP, "hipGetSymbolAddress returned a null address");
+    g_static_part_ptr[dev] = p;
+  }
+  *out = g_static_part_ptr[dev];
   return LRQK_OK;
+}
+
+template <typename T>
+static int attention_static_impl(const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
+                                 void* out, int bh, int d, hipStream_t st) {
+  int lpr_log2 = 0;
+  int rc = attn_shape(d, Vec16<T>::N, &lpr_log2);
+  if (rc) return rc;
+  const int S = attn_splits(n_valid);
+  const size_t need = (size_t)bh * S * (d + 2);
+  LRQK_REQUIRE(need <= kStaticPartFloats, LRQK_ELIMIT,
+               "bh=%d x %d splits x (d+2)=%d floats of partial results exceed the static block of %zu floats", bh, S, d + 2,
+               kStaticPartFloats);
+  float* part = nullptr;
+  if ((rc = static_part(&part))) return rc;
+  return attention_launch<T>(q, k_act, v_act, n_slots, n_valid, out, bh, d, lpr_log2, S, part, st);
 }
 
 template <typename T>
@@ -603,4 +660,17 @@ extern "C" int lrqk_attention(lrqk_ctx* ctx, const void* q, const void* k_act, c
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LRQK_F32) return attention_impl<float>(ctx, q, k_act, v_act, n_slots, n_valid, out, bh, d, st);
   return attention_impl<bf16_t>(ctx, q, k_act, v_act, n_slots, n_valid, out, bh, d, st);
+}
+
+extern "C" int lrqk_attention_static(const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
+                                     void* out, int bh, int d, int dtype, void* stream) {
+  LRQK_REQUIRE(q && k_act && v_act && out, LRQK_EINVAL, "null pointer");
+  LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
+  LRQK_REQUIRE(bh > 0 && bh <= 65535 && d > 0, LRQK_EINVAL, "bad sizes bh=%d d=%d", bh, d);
+  LRQK_REQUIRE(n_valid > 0 && n_valid <= n_slots, LRQK_EINVAL, "n_valid=%d outside 1..%d", n_valid, n_slots);
+  LRQK_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)k_act % 16 == 0) && ((uintptr_t)v_act % 16 == 0), LRQK_EINVAL,
+               "pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LRQK_F32) return attention_static_impl<float>(q, k_act, v_act, n_slots, n_valid, out, bh, d, st);
+  return attention_static_impl<bf16_t>(q, k_act, v_act, n_slots, n_valid, out, bh, d, st);
 }

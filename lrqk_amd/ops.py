@@ -276,6 +276,20 @@ def attention(ws: Workspace, q: torch.Tensor, k_act: torch.Tensor, v_act: torch.
     return out
 
 
+def attention_static(q: torch.Tensor, k_act: torch.Tensor, v_act: torch.Tensor, out: torch.Tensor,
+                     n_valid: Optional[int] = None) -> torch.Tensor:
+    """The same attention through the entry point that allocates nothing: no workspace, the caller
+    passes ``out`` [b,H,1,d] and a contiguous q; partial results go to a fixed block inside the library."""
+    _need_cuda(q, k_act, v_act, out)
+    b, H, n, d = k_act.shape
+    n_valid = n if n_valid is None else n_valid
+    assert k_act.is_contiguous() and v_act.is_contiguous() and q.is_contiguous() and out.is_contiguous()
+    assert q.dtype == k_act.dtype == v_act.dtype == out.dtype and out.numel() == b * H * d
+    check(_lib.load().lrqk_attention_static(q.data_ptr(), k_act.data_ptr(), v_act.data_ptr(), n, n_valid,
+                                            out.data_ptr(), b * H, d, _dt(q), _stream(q)))
+    return out
+
+
 def als_decode(ws: Workspace, b_q, b_k, a_k, active_idx: Optional[torch.Tensor], k_prev, n: int, q, k_new,
                max_iter: int, tol: float, append_row: int = -1) -> Tuple[torch.Tensor, torch.Tensor]:
     """In-place factor update.  b_q,b_k [b,H,r,d]; a_k [b,H,cap,r]; active_idx int32 [b,H,>=n] or None;
