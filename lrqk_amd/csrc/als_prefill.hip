@@ -778,44 +778,29 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
 }
 
 // ---- small per-head systems, r <= 32: X = G^-1 RHS for a packed block [G (r x r) | RHS (r x d)] in LDS.
-// One wave inverts G (symmetric sweeps on the matrix cores); the product is formed 32 columns of the
-// right-hand side at a time, again on the matrix cores, by whichever wave takes the block.  No pivoting:
-// G is a Gram matrix (plus B B^T), positive definite.
+// Gauss-Jordan elimination of [G | RHS] as symmetric sweeps on the matrix cores, 64 columns of the
+// right-hand side per wave (every wave repeats the sweeps of G itself).  No pivoting: G is a Gram matrix
+// (plus B B^T), positive definite.
 struct PfSmallShared {
-  __align__(16) float scale[2][32];    // row scales of up to two inversions in flight
-  __align__(16) float inv[2][32 * kLdi];
+  __align__(16) float scale[kPfSmallThreads / kWave][32];  // row scales of the solve each wave has in flight
 };
 
-// the inverse of the r x r block of G0 (row stride r + d), by the calling wave
-__device__ __forceinline__ void pf_invert(const float* G0, int r, int d, float* scale, float* inv) {
-  const int ld = r + d;
-  invert_sweep_mfma([&](int i, int j) { return G0[min(i, r - 1) * ld + min(j, r - 1)]; }, r, scale, inv);
-}
-
-// columns [32 cb, 32 cb + 32) of X = inv * RHS, by the calling wave; emit(i, j, x) for i < r, j < d
+// X = G^-1 RHS for the packed block G0 = [G (r x r) | RHS (r x d)] in LDS: the waves of the workgroup share
+// the 32-column blocks of the right-hand side, two per solve; emit(i, j, x) for i < r, j < d.
 template <typename Emit>
-__device__ __forceinline__ void pf_apply_inverse(const float* inv, const float* G0, int r, int d, int cb, Emit&& emit) {
-  const int lane = lane_id();
-  const int col = lane & 31, half = lane >> 5;
-  const int j = cb * 32 + col, ld = r + d;
-  float a[16], b[16];
-#pragma unroll
-  for (int kk = 0; kk < 16; ++kk) {
-    const int k = 2 * kk + half;
-    a[kk] = inv[col * kLdi + k];
-    const float x = G0[min(k, r - 1) * ld + r + min(j, d - 1)];
-    b[kk] = (k < r && j < d) ? x : 0.0f;
-  }
-  v16f acc;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-#pragma unroll
-  for (int kk = 0; kk < 16; ++kk) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc, 0, 0, 0);
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int i = mfma_row(lane, v);
-    if (i < r && j < d) emit(i, j, acc[v]);
-  }
+__device__ __forceinline__ void pf_solve_blocks(const float* G0, int r, int d, int cb0, float* scale, Emit&& emit) {
+  const int ld = r + d;
+  solve_sweep_mfma<2>([&](int i, int j) { return G0[min(i, r - 1) * ld + min(j, r - 1)]; },
+                      [&](int b, int i, int col) {
+                        const int j = (cb0 + b) * 32 + col;
+                        const float x = G0[min(i, r - 1) * ld + r + min(j, d - 1)];
+                        return j < d ? x : 0.0f;
+                      },
+                      r, scale,
+                      [&](int b, int i, int col, float x) {
+                        const int j = (cb0 + b) * 32 + col;
+                        if (j < d) emit(i, j, x);
+                      });
 }
 
 // sum of the S partial [r][r+d] blocks; 16 elements x 8 partials of loads in flight per thread
@@ -891,7 +876,7 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
   const int h = blockIdx.x;
   const int wave = wave_id();
   constexpr int kWaves = kPfSmallThreads / kWave;
-  const int nblk = (d + 31) / 32;  // 32-column blocks of a right-hand side
+  const int njob = (d + 63) / 64;  // pairs of 32-column blocks of a right-hand side
 
   if (stage == 0) {
     int done = 0;
@@ -938,19 +923,16 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
     pf_reduce_part(pq, S, ne, G1);
     pf_reduce_part(pk, S, ne, G2);
     __syncthreads();
-    // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q and B_K likewise: the two inverses side by side, then all blocks
-    if (wave == 0) pf_invert(G1, r, d, sh.scale[0], sh.inv[0]);
-    else if (wave == 1) pf_invert(G2, r, d, sh.scale[1], sh.inv[1]);
-    __syncthreads();
-    for (int job = wave; job < 2 * nblk; job += kWaves) {
-      if (job < nblk) {
-        pf_apply_inverse(sh.inv[0], G1, r, d, job, [&](int i, int j, float x) {
+    // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q and B_K likewise: both systems side by side, two column blocks per wave
+    for (int job = wave; job < 2 * njob; job += kWaves) {
+      if (job < njob) {
+        pf_solve_blocks(G1, r, d, 2 * job, sh.scale[wave], [&](int i, int j, float x) {
           Bs[i * (d + 4) + j] = x;
           b_q[(int64_t)h * r * d + i * d + j] = x;
         });
       } else {
-        pf_apply_inverse(sh.inv[1], G2, r, d, job - nblk,
-                         [&](int i, int j, float x) { b_k[(int64_t)h * r * d + i * d + j] = x; });
+        pf_solve_blocks(G2, r, d, 2 * (job - njob), sh.scale[wave],
+                        [&](int i, int j, float x) { b_k[(int64_t)h * r * d + i * d + j] = x; });
       }
     }
     if (stage == 2) return;
@@ -965,10 +947,9 @@ __global__ __launch_bounds__(kPfSmallThreads) void pf_small32_kernel(int stage, 
     pf_add_bbt(G1, Bs, r, d, G0);
   }
   __syncthreads();
-  if (wave == 0) pf_invert(G0, r, d, sh.scale[0], sh.inv[0]);
-  __syncthreads();
-  for (int job = wave; job < nblk; job += kWaves)
-    pf_apply_inverse(sh.inv[0], G0, r, d, job, [&](int i, int j, float x) { Mt[(int64_t)h * r * d + i * d + j] = x; });
+  for (int job = wave; job < njob; job += kWaves)
+    pf_solve_blocks(G0, r, d, 2 * job, sh.scale[wave],
+                    [&](int i, int j, float x) { Mt[(int64_t)h * r * d + i * d + j] = x; });
 }
 
 template <typename T>

@@ -71,4 +71,77 @@ __device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, 
   }
 }
 
+// X = G^-1 RHS for NB blocks of 32 right-hand-side columns, by one wave: the same 32 sweeps, applied to
+// the augmented matrix [G | RHS] (Gauss-Jordan elimination of the right-hand side, no explicit inverse).
+// For a positive definite G this is backward stable: the residual RHS - G X stays at 2^-24 relative however
+// badly G is conditioned, as with a factorisation-based solve, whereas a product with a computed inverse
+// leaves cond(G) * 2^-24.  At pivot p the right-hand side takes the same rank-1 update as G, with row p of
+// the block as the B operand: r_ij -= (a_ip / d) r_pj, r_pj -= (1 - 1/d) r_pj.  G is scaled to unit diagonal
+// as in invert_sweep_mfma: the rows of RHS are scaled on the way in and the rows of X on the way out.
+// g(i, j): element of G (any i, j < 32; values outside r x r are ignored); rhs(b, i, col): element (i, col)
+// of block b (0 outside the matrix); emit(b, i, col, x) receives X for i < r.  sbuf: 32 floats of LDS
+// owned by this wave.
+template <int NB, typename GetG, typename GetR, typename Emit>
+__device__ __forceinline__ void solve_sweep_mfma(GetG&& g, GetR&& rhs, int r, float* sbuf, Emit&& emit) {
+  const int lane = lane_id();
+  const int col = lane & 31, half = lane >> 5;
+  v16f acc, xr[NB];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int i = mfma_row(lane, v);
+    const float x = g(i, col);
+    acc[v] = (i < r && col < r) ? x : (i == col ? 1.0f : 0.0f);
+  }
+  const float s_col = col < r ? __builtin_amdgcn_rsqf(g(col, col)) : 1.0f;
+  __builtin_amdgcn_wave_barrier();  // (an earlier use of sbuf by this wave is complete)
+  if (lane < 32) sbuf[lane] = s_col;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  float sr[16];  // s_row of every element this lane holds
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const float4 s4 = reinterpret_cast<const float4*>(sbuf)[2 * a + half];  // rows 8a + 4 half + 0..3
+    sr[4 * a + 0] = s4.x;
+    sr[4 * a + 1] = s4.y;
+    sr[4 * a + 2] = s4.z;
+    sr[4 * a + 3] = s4.w;
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] *= sr[v] * s_col;
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int i = mfma_row(lane, v);
+      xr[b][v] = i < r ? rhs(b, i, col) * sr[v] : 0.0f;
+    }
+#pragma unroll
+  for (int p = 0; p < 32; ++p) {
+    if (p < r) {  // (wave-uniform)
+      const int v = ((p >> 3) << 2) + (p & 3), hp = (p >> 2) & 1;
+      const float rv = acc[v];
+      const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rv), p + 32 * hp));
+      float rc = __builtin_amdgcn_rcpf(d);
+      rc = fmaf(fmaf(-d, rc, 1.0f), rc, rc);
+      const bool inhalf = half == hp, isp = col == p;
+      const float A = inhalf ? (isp ? 1.0f - rc : rv * rc) : (isp ? 2.0f : 0.0f);
+      const float B = inhalf ? (isp ? d - 1.0f : rv) : (isp ? 1.0f : 0.0f);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const float BR = inhalf ? xr[b][v] : 0.0f;
+        xr[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, BR, xr[b], 0, 0, 0);
+      }
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, B, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int i = mfma_row(lane, v);
+      if (i < r) emit(b, i, col, xr[b][v] * sr[v]);
+    }
+}
+
 }  // namespace lrqk

@@ -362,6 +362,7 @@ class LightAttentionIndicesFactory:
                                   evict.shape[2])
         else:
             ops.fetch_rows(self.KVcpu.data, self.Kgpu, self.Vgpu, self._active_idx, slots, count, evict.shape[2])
+        self.last_attn = ops.attention(self.ws, q, self.Kgpu, self.Vgpu) if self.attn_in_step else None
         return self.Kgpu, self.Vgpu
 
     # ------------------------------------------------------------------ statistics

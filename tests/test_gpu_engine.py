@@ -31,78 +31,183 @@ def _rel(a, b):
     return float((a - b).norm() / (b.norm() + 1e-300))
 
 
+# Largest deviation seen per (trace, quantity) in this session: printed (and written next to the other GPU
+# results when that folder exists) so that every tolerance below can be read against what was measured.
+DEVIATIONS = {}
+
+
+def _note(tag, name, value, limit):
+    """Record a measured relative deviation and require it below ``limit``."""
+    key = f"{tag}:{name}"
+    DEVIATIONS[key] = max(DEVIATIONS.get(key, 0.0), value)
+    assert value < limit, (tag, name, "measured %.3e" % value, "limit %.1e" % limit)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _report_deviations():
+    yield
+    if not DEVIATIONS:
+        return
+    import json
+    import os
+    lines = [f"  {k}: {v:.3e}" for k, v in sorted(DEVIATIONS.items())]
+    print("\nmeasured deviations (max over steps):\n" + "\n".join(lines), flush=True)
+    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    if os.path.isdir(out):
+        with open(os.path.join(out, "parity_deviations_engine.json"), "w") as f:
+            json.dump(DEVIATIONS, f, indent=1, sort_keys=True)
+
+
+def _check_prefill_products(oracle, tag, Q, K, g, A_Q0, A_K0, r, max_iter, tol, got32, heads):
+    """The factorisation as the kernel returns it (fp32, before the engine rounds it to the storage type)
+    against the fp64 oracle on the query heads ``heads``.  The individual factors are only defined up to the
+    conditioning of the r x r systems (an fp32 LAPACK run of the same algorithm is itself percents away from
+    fp64 on rank-r data, which tests/test_oracle_als.py measures on the CPU), so what is compared is what the
+    path uses: the fits A_K B_K and A_Q B_Q and the first proxy scores A_Q[-1] A_K^T.  The limit is derived:
+    three times what the oracle's own fp32 run deviates from its fp64 run on the same heads, at least 1e-3."""
+    hs = list(heads)
+    Qs = Q[:, hs]
+    Ks = oracle.repeat_kv(K, g)[:, hs]
+    a0, k0 = A_Q0[:, hs], A_K0[:, hs]
+    ref = oracle.als_prefill_w1(Qs.double(), Ks.double(), a0.double(), k0.double(), max_iter, tol)
+    r32 = oracle.als_prefill_w1(Qs.float(), Ks.float(), a0.float(), k0.float(), max_iter, tol)
+    AQ, BQ, AK, BK = [t[:, hs].cpu().double() for t in got32]
+
+    def products(aq, bq, ak, bk):
+        aq, bq, ak, bk = aq.double(), bq.double(), ak.double(), bk.double()
+        return {"A_K B_K": ak @ bk, "A_Q B_Q": aq @ bq, "A_Q[-1] A_K^T": aq[:, :, -1:] @ ak.transpose(-1, -2)}
+
+    exp, own, got = products(*ref), products(*r32), products(AQ, BQ, AK, BK)
+    for name in exp:
+        base = _rel(own[name], exp[name])
+        dev = _rel(got[name], exp[name])
+        _say(f"{tag} prefill {name}: kernel vs fp64 {dev:.2e}; fp32 oracle vs fp64 {base:.2e}")
+        _note(tag, "prefill " + name, dev, max(1e-3, 3.0 * base))
+    return ref
+
+
 def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter, tol, rho, cls=None, capacity=64,
-              seed=0, fp_tol=None, no_hit_miss=False, sigma=0.01, compare_factors=True):
+              seed=0, fp_tol=None, no_hit_miss=False, sigma=0.01, compare_factors=True, attn_in_step=True,
+              gpu_draw=False, oracle_heads=None, tag=None, configure=None, attn_tol=None, compare_every=1):
+    """One seeded prefill + decode trace on the GPU engine and on the oracle.
+
+    compare_factors   compare the engine's stored factors with an fp64 oracle prefill element by element
+                      (well-conditioned traces); otherwise the kernel's fp32 factors are compared through
+                      their products on ``oracle_heads`` (see _check_prefill_products)
+    attn_in_step      the fused step computes the attention; False takes the path of a reference-style
+                      caller (the step returns K, V and the caller runs the attention itself)
+    gpu_draw          draw the inputs on the GPU (long contexts; a host draw would take minutes)
+    """
     from lrqk_amd import synth, ops
+    tag = tag or f"b{b}h{hq}l{l}r{r}k{k}"
     g = hq // hkv
-    gen = torch.Generator().manual_seed(seed)
-    Q, WQ = synth.low_rank_noise(gen, b, hq, l, d, rho, sigma, dtype)
-    K, WK = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
-    V, WV = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
-    A_Q0 = torch.randn((b, hq, l, r), generator=gen)
-    A_K0 = torch.randn((b, hq, l, r), generator=gen)
+    if gpu_draw:
+        gen = torch.Generator(device=DEV).manual_seed(seed)
+        Qd, WQ = synth.low_rank_noise(gen, b, hq, l, d, rho, sigma, dtype)
+        Kd, WK = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
+        Vd, WV = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
+        A_Q0d = torch.randn((b, hq, l, r), generator=gen, device=DEV)
+        A_K0d = torch.randn((b, hq, l, r), generator=gen, device=DEV)
+        Q, K, V, A_Q0, A_K0 = Qd.cpu(), Kd.cpu(), Vd.cpu(), A_Q0d.cpu(), A_K0d.cpu()
+    else:
+        gen = torch.Generator().manual_seed(seed)
+        Q, WQ = synth.low_rank_noise(gen, b, hq, l, d, rho, sigma, dtype)
+        K, WK = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
+        V, WV = synth.low_rank_noise(gen, b, hkv, l, d, rho, sigma, dtype)
+        A_Q0 = torch.randn((b, hq, l, r), generator=gen)
+        A_K0 = torch.randn((b, hq, l, r), generator=gen)
+        Qd, Kd, Vd = Q.to(DEV), K.to(DEV), V.to(DEV)
     cls = cls or lrqk.LightAttentionIndicesFactory
     eng = cls(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=r, max_iter=max_iter, tol=tol,
               capacity=capacity)
     eng.init_factors = (A_Q0, A_K0)
-    eng.attn_in_step = True
+    eng.attn_in_step = attn_in_step
+    if configure:
+        configure(eng)
     orc = oracle.OracleLayer(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=r, max_iter=max_iter, tol=tol,
                              capacity=capacity, compute_dtype=torch.float64, no_hit_miss=no_hit_miss)
-    # default tolerance of the small traces: their data has rank rho == r, so the r x r Gram
-    # systems are ill-conditioned (cond ~ 1e4-1e5) and fp32 carries 1e-3..1e-2; the
-    # full-shape traces below pass explicit, tighter limits
-    lim = fp_tol or (2e-2 if dtype == torch.bfloat16 else 1e-2)
+    # Limits on the per-step factor outputs (q_hat, k_hat, B_Q, B_K; both sides rounded to the storage type):
+    # the larger of a floor and four times what the oracle's own fp32 run of the same step deviates from its
+    # fp64 run (derived per step below).  Floors: fp32 storage 1e-4 (measured 2e-7..3e-5 on well-conditioned
+    # traces); bf16 storage 1e-3: the outputs agree except where the two roundings to bf16 fall on different
+    # sides (one unit in the last place = 2^-8 relative on that element).  Every measured value is recorded.
+    # Traces on data of rank rho <= r (the tiny ones): r x r systems of condition 1e5 and beyond, where single
+    # steps of any fp32 evaluation order scatter by factors: floor 1e-3 there too.
+    lim = fp_tol or (1e-3 if (dtype == torch.bfloat16 or rho <= r) else 1e-4)
 
     # ---- prefill
-    eng.prefill(Q.to(DEV), K.to(DEV), V.to(DEV))
-    ref = oracle.cast_lrqk_prefill(Q, oracle.repeat_kv(K, g), r, max_iter[0], tol[0], A_Q0=A_Q0, A_K0=A_K0,
-                                   compute_dtype=torch.float64)
-    # fp32 kernels vs the fp64 oracle, both rounded to the storage dtype afterwards: most
-    # elements agree exactly, a few differ by one unit in the last place
+    eng.prefill(Qd, Kd, Vd)
     gA_K, gB_K, gB_Q = eng.A_K.cpu(), eng.B_K.cpu(), eng.B_Q.cpu()
     gA_Qrow = eng.last_A_Q_row.cpu()
+    # the same kernel call the engine made, kept in fp32: products against fp64 on a head subset, and the
+    # engine's stored factors must be exactly these, rounded to the storage type
+    got32 = ops.als_prefill(ops.Workspace(), Qd, Kd, A_Q0.to(DEV).clone(), A_K0.to(DEV).clone(), max_iter[0], tol[0])
+    heads = oracle_heads if oracle_heads is not None else range(min(hq, 2))
+    _check_prefill_products(oracle, tag, Q, K, g, A_Q0, A_K0, r, max_iter[0], tol[0], got32, heads)
+    assert torch.equal(got32[2].to(dtype).cpu(), gA_K) and torch.equal(got32[3].to(dtype).cpu(), gB_K), tag
+    assert torch.equal(got32[1].to(dtype).cpu(), gB_Q), tag
+    assert torch.equal(got32[0][:, :, -1:].to(dtype).cpu(), gA_Qrow), tag
+    del got32
     if compare_factors:
+        # element by element as well (small traces).  Their data has rank rho == r, so the r x r systems are
+        # badly conditioned and the factors themselves carry cond * 2^-24: measured up to 6e-3 -> 2e-2
+        ref = oracle.cast_lrqk_prefill(Q, oracle.repeat_kv(K, g), r, max_iter[0], tol[0], A_Q0=A_Q0, A_K0=A_K0,
+                                       compute_dtype=torch.float64)
         for name, got, exp in (("A_K", gA_K, ref[2]), ("B_K", gB_K, ref[3]), ("B_Q", gB_Q, ref[1]),
                                ("A_Q[-1]", gA_Qrow, ref[0][:, :, -1:])):
-            assert _rel(got, exp) < lim, ("prefill", name, _rel(got, exp))
-    # what the factors are for: the fit K ~ A_K B_K and the last query row q ~ a_q B_Q.  These
-    # are well determined even where the individual factors are not (badly scaled r x r
-    # systems: fp32 LAPACK itself is several percent away from fp64 there)
-    K4 = oracle.repeat_kv(K, g).double()
-    fit_g = _rel(gA_K.double() @ gB_K.double(), K4)
-    fit_o = _rel(ref[2].double() @ ref[3].double(), K4)
-    assert abs(fit_g - fit_o) < 2e-3 + 0.05 * fit_o, ("prefill fit K", fit_g, fit_o)
-    qfit_g = _rel(gA_Qrow.double() @ gB_Q.double(), Q[:, :, -1:].double())
-    qfit_o = _rel(ref[0][:, :, -1:].double() @ ref[1].double(), Q[:, :, -1:].double())
-    assert abs(qfit_g - qfit_o) < 2e-2 + 0.1 * qfit_o, ("prefill fit q", qfit_g, qfit_o)
+            _note(tag, "prefill " + name, _rel(got, exp), 2e-2)
     # continue the oracle from the GPU's factors
     A_Q_full = torch.zeros((b, hq, l, r), dtype=dtype)
     A_Q_full[:, :, -1:] = gA_Qrow
     orc.prefill(Q, K, V, als_result=(A_Q_full, gB_Q, gA_K, gB_K))
+    del A_Q_full, Qd, Kd, Vd
     _compare_state(eng, orc, k, "prefill")
 
     # ---- decode
     stream = synth.DecodeStream(synth.Workload("t", hq, hkv, d, b, dtype, l, r, k, L, max_iter, tol, steps, rho, sigma),
-                                Q[:, :, -1:], (WQ, WK, WV), gen)
+                                Q[:, :, -1:].to(gen.device), (WQ, WK, WV), gen)
     n_miss_total = 0
+    # attention against the textbook softmax in fp64, rounded to the storage type like the kernel's output
+    # (else the comparison measures the output rounding itself, 1.1e-3..2.2e-3 in bf16): measured 2e-7 in
+    # fp32; in bf16 what remains are elements whose rounding fell on the other side
+    a_lim = attn_tol or (1e-3 if dtype == torch.bfloat16 else 1e-5)
     for step in range(steps):
-        q, kk, vv = stream.next()
+        q, kk, vv = [t.cpu() for t in stream.next()]
         Kg, Vg = eng.decode(q.to(DEV), kk.to(DEV), vv.to(DEV))
         oB_Q, oB_K, ohq, ohk = orc.begin_decode(q, kk, vv)
-        for name, got, exp in (("q_hat", eng.last_q_hat, ohq), ("k_hat", eng.last_k_hat, ohk),
-                               ("B_Q", eng.B_Q, oB_Q), ("B_K", eng.B_K, oB_K)):
-            assert _rel(got, exp) < lim, (step, name, _rel(got, exp))
+        # the oracle's own fp32 run of the same update (same inputs: begin_decode has not changed the factors
+        # yet): what fp32 arithmetic is entitled to on this step's r x r systems
+        if orc.current_len <= orc.n:
+            a_in, k_in = orc.A_K, orc.Kgpu.narrow(2, 0, orc.current_len - 1)
+        else:
+            a_in, k_in = orc._A_K_hitted_with_lite(), orc.Kgpu
+        o32 = oracle.cast_lrqk_decode(orc.B_Q, a_in, orc.B_K, k_in, q, oracle.repeat_kv(kk, g), max_iter[1], tol[1],
+                                      torch.float32)
+        for name, got, exp, own in (("q_hat", eng.last_q_hat, ohq, o32[2]), ("k_hat", eng.last_k_hat, ohk, o32[3]),
+                                    ("B_Q", eng.B_Q, oB_Q, o32[0]), ("B_K", eng.B_K, oB_K, o32[1])):
+            key = f"{tag}:{name} (fp32 oracle)"
+            DEVIATIONS[key] = max(DEVIATIONS.get(key, 0.0), _rel(own, exp))
+            _note(tag, name, _rel(got, exp), max(lim, 4.0 * DEVIATIONS[key]))   # (largest of the trace so far)
         oK, oV = orc.finish_decode(eng.B_Q.cpu(), eng.B_K.cpu(), eng.last_q_hat.cpu(), eng.last_k_hat.cpu())
         assert Kg.shape == oK.shape, (step, Kg.shape, oK.shape)
-        assert torch.equal(Kg.cpu(), oK) and torch.equal(Vg.cpu(), oV), step
-        _compare_state(eng, orc, k, f"step {step}")
+        if step % compare_every == 0 or step == steps - 1:
+            assert torch.equal(Kg.cpu(), oK) and torch.equal(Vg.cpu(), oV), step
+            _compare_state(eng, orc, k, f"step {step}")
+        else:
+            assert torch.equal(eng.hit_indices.cpu(), orc.hit_indices), step
         if orc.current_len > orc.n:
             assert torch.equal(eng.last_evict.cpu().bool(), orc.last_evict), step
             assert torch.equal(eng.last_miss_count.cpu().long(), orc.last_evict.sum(-1)), step
             n_miss_total += int(orc.last_evict.sum())
-            if eng.last_attn is not None:
-                exp = oracle.attention(q, oK, oV)
-                assert _rel(eng.last_attn, exp) < (8e-3 if dtype == torch.bfloat16 else 1e-4), step
+            exp = oracle.attention(q, oK, oV).to(dtype)
+            if attn_in_step:
+                assert eng.last_attn is not None
+                _note(tag, "attention", _rel(eng.last_attn, exp), a_lim)
+            else:
+                # reference-style caller: the step hands back K, V and the caller attends (py:2326)
+                assert eng.last_attn is None
+                out = ops.attention(eng.ws, q.to(DEV), Kg, Vg)
+                _note(tag, "attention (caller)", _rel(out, exp), a_lim)
     return eng, orc, n_miss_total
 
 
@@ -135,7 +240,7 @@ def test_tiny_fp32_trace(lrqk, oracle):
 def test_tiny_bf16_trace(lrqk, oracle):
     _say("tiny bf16 trace")
     _lockstep(lrqk, oracle, b=1, hq=4, hkv=1, d=16, l=50, r=8, k=16, L=4, steps=24, dtype=torch.bfloat16,
-              max_iter=(2, 2), tol=(1e-8, 1e-8), rho=8, capacity=32, fp_tol=2e-2)
+              max_iter=(2, 2), tol=(1e-8, 1e-8), rho=8, capacity=32)
 
 
 def test_buffer_growth_during_decode(lrqk, oracle):
@@ -154,7 +259,7 @@ def test_growth_with_score_index_and_victim_cache(lrqk, oracle):
     re-sized; the trace must stay in lock step with the oracle throughout."""
     _say("growth trace, score index on")
     eng, orc, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=32, l=300, r=16, k=64, L=8, steps=400,
-                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=24, capacity=64, fp_tol=3e-2,
+                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=24, capacity=64,
                             compare_factors=False)
     assert n > 0 and eng._A_K.capacity == orc._A_K.capacity and eng._A_K.capacity >= 675   # 450 -> 675 (-> 1012)
 
@@ -297,16 +402,157 @@ def test_qwen_shape_fp32_short(lrqk, oracle):
     max_iter (1,1)) at a reduced context so the oracle finishes in seconds."""
     _say("qwen shape trace")
     _, _, n = _lockstep(lrqk, oracle, b=1, hq=28, hkv=4, d=128, l=1536, r=16, k=512, L=32, steps=40,
-                        dtype=torch.float32, max_iter=(1, 1), tol=(1e-2, 1e-2), rho=32, capacity=4096, fp_tol=2e-3)
+                        dtype=torch.float32, max_iter=(1, 1), tol=(1e-2, 1e-2), rho=32, capacity=4096)
     assert n > 0
 
 
 def test_llama_shape_bf16_short(lrqk, oracle):
     """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, r 32, k 2048, L 64, bf16) at an
-    8K context."""
+    8K context, long enough (70 steps) for the 64-token ring to be flushed to the host store once."""
     _say("llama shape trace")
-    _lockstep(lrqk, oracle, b=1, hq=32, hkv=8, d=128, l=8192, r=32, k=2048, L=64, steps=6, dtype=torch.bfloat16,
-              max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096, fp_tol=3e-2, compare_factors=False)
+    eng, orc, n = _lockstep(lrqk, oracle, b=1, hq=32, hkv=8, d=128, l=8192, r=32, k=2048, L=64, steps=70,
+                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096,
+                            compare_factors=False, oracle_heads=(0, 13, 31), tag="llama8k",
+                            compare_every=8)
+    assert n > 0 and len(eng.KVcpu) == 8192 + 64
+
+
+def test_llama_shape_128k_lockstep(lrqk, oracle):
+    """The configuration the headline metric is quoted on (Llama-3-8B shape, 128K context, bf16, r 32, k 2048,
+    lite 64), with the engine's defaults -- score index on, victim cache on, attention inside the step -- in
+    lock step with the oracle: prefill selection, resident rows and host store, then every decode step's
+    ids, evicted slots and refetched rows bit for bit, factors and attention within tolerance."""
+    _say("llama shape 128K trace")
+    oracle.set_threads(16)
+    try:
+        eng, orc, n = _lockstep(lrqk, oracle, b=1, hq=32, hkv=8, d=128, l=131072, r=32, k=2048, L=64, steps=10,
+                                dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096,
+                                compare_factors=False, oracle_heads=(3, 28), tag="llama128k",
+                                gpu_draw=True, compare_every=3)
+    finally:
+        oracle.set_threads(1)
+    assert eng.use_score_index and eng.victim_rows_effective == 8192 and n > 0
+    fast, full = eng.ws.select_stats()
+    _say("selector heads from the candidate list / rescanned:", fast, full)
+    assert fast > 0     # the filtered (score index) path served heads in this trace
+
+
+def test_llama_shape_batch4_short(lrqk, oracle):
+    """Batch 4 of the Llama shape (128 heads in one launch, the full-decoder configuration's width)."""
+    _say("llama shape, batch 4")
+    _, _, n = _lockstep(lrqk, oracle, b=4, hq=32, hkv=8, d=128, l=4096, r=32, k=2048, L=64, steps=5,
+                        dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096,
+                        compare_factors=False, oracle_heads=(5, 30), tag="llama_b4", gpu_draw=True)
+    assert n > 0
+
+
+def test_poster_operating_point(lrqk, oracle):
+    """r 16, k 1024, lite 16 on the Llama shape: the setting behind the reference's published tokens/s table
+    (tps_estimate.py:20-29).  24 steps: the 16-token ring wraps and is flushed once."""
+    _say("r16 / k1024 / lite16 trace")
+    eng, _, n = _lockstep(lrqk, oracle, b=1, hq=32, hkv=8, d=128, l=6000, r=16, k=1024, L=16, steps=24,
+                          dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, capacity=4096,
+                          compare_factors=False, oracle_heads=(0, 31), tag="poster_r16")
+    assert n > 0 and len(eng.KVcpu) == 6000 + 16
+
+
+@pytest.mark.parametrize("r,k,L,l,dtype", [(32, 512, 16, 3000, torch.bfloat16), (8, 256, 8, 2000, torch.bfloat16),
+                                             (16, 128, 8, 1000, torch.float32)])
+def test_eight_iterations_tight_tolerance(lrqk, oracle, r, k, L, l, dtype):
+    """max_iter (8, 8) with tol 1e-8, the setting of the reference's accuracy configurations
+    (eval_configs_lrqk): more decode iterations than the scan can take over from the solve kernel, so the
+    step finishes the factor update in a launch of its own.  Also the smallest rank the reference sweeps (8)."""
+    _say("max_iter 8 / tol 1e-8 trace", r, k, L, l, dtype)
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=8, hkv=2, d=64, l=l, r=r, k=k, L=L, steps=20, dtype=dtype,
+                        max_iter=(8, 8), tol=(1e-8, 1e-8), rho=2 * r, sigma=0.05, capacity=1024,
+                        compare_factors=False,
+                        oracle_heads=(0, 5), tag=f"iter8_r{r}")
+    assert n > 0
+
+
+def test_reference_style_caller(lrqk, oracle):
+    """The step as a reference-style caller drives it (DynamicLRQKCache.update returns K, V and the caller
+    runs the attention, py:2284-2290, 2326): no attention inside the step, hence the separate fetch launch
+    and no victim cache.  Same lock-step comparison, ring flush included."""
+    _say("reference-style caller trace (attention outside the step)")
+    _, _, n = _lockstep(lrqk, oracle, b=2, hq=8, hkv=2, d=64, l=1500, r=16, k=256, L=8, steps=30,
+                        dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, sigma=0.05, capacity=512,
+                        compare_factors=False, attn_in_step=False, tag="caller_attn")
+    assert n > 0
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=16, l=40, r=4, k=8, L=4, steps=20, dtype=torch.float32,
+                        max_iter=(2, 2), tol=(1e-8, 1e-8), rho=4, capacity=16, attn_in_step=False, tag="caller_attn_tiny")
+    assert n > 0
+
+
+def test_store_tail_is_never_read(lrqk, oracle, monkeypatch):
+    """The host store is not cleared when it is allocated or grown (the reference zero-fills it,
+    py:888, 913).  Poison every fresh block with NaN: a lock-step trace that grows the store twice must
+    stay bit-identical to the oracle, i.e. no row at or beyond the rows written so far is ever read."""
+    _say("poisoned store tail trace")
+    from lrqk_amd import buffers
+
+    def poisoned(self, shape):
+        pin = bool(self.pin_memory) and torch.cuda.is_available()
+        t = torch.empty(shape, device=self.device, dtype=self.dtype, pin_memory=pin)
+        return t.fill_(float("nan"))
+
+    monkeypatch.setattr(buffers.AutoIncreaseTensorSharedKV, "_alloc", poisoned)
+    eng, orc, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=32, l=300, r=16, k=64, L=8, steps=400,
+                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=24, capacity=64,
+                            compare_factors=False, tag="poison", compare_every=16)
+    assert n > 0 and eng.KVcpu.capacity >= 675
+    assert torch.isnan(eng.KVcpu.data[:, :, len(eng.KVcpu):].float()).all()      # the tail is still poison
+    assert torch.isfinite(eng.Kgpu.float()).all() and torch.isfinite(eng.Vgpu.float()).all()
+
+
+def test_independent_runs_agree(lrqk, oracle):
+    """No hand-over of factors: the GPU engine and an fp64 oracle run the whole trace (their own prefill
+    factorisation, their own factor updates) on the Qwen-shaped fp32 configuration, whose r x r systems are
+    well conditioned.  Differences are then fp32 rounding only, so the resident sets must coincide almost
+    everywhere after every step and the attention outputs must agree."""
+    _say("independent GPU / oracle runs")
+    from lrqk_amd import synth, ops
+    b, hq, hkv, d, l, r, k, L, steps = 1, 28, 4, 128, 1536, 16, 512, 32, 40
+    g = hq // hkv
+    gen = torch.Generator().manual_seed(3)
+    Q, WQ = synth.low_rank_noise(gen, b, hq, l, d, 32, 0.01, torch.float32)
+    K, WK = synth.low_rank_noise(gen, b, hkv, l, d, 32, 0.01, torch.float32)
+    V, WV = synth.low_rank_noise(gen, b, hkv, l, d, 32, 0.01, torch.float32)
+    A_Q0 = torch.randn((b, hq, l, r), generator=gen)
+    A_K0 = torch.randn((b, hq, l, r), generator=gen)
+    eng = lrqk.LightAttentionIndicesFactory(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=r,
+                                            max_iter=(1, 1), tol=(1e-2, 1e-2), capacity=4096)
+    eng.init_factors = (A_Q0, A_K0)
+    eng.attn_in_step = True
+    eng.prefill(Q.to(DEV), K.to(DEV), V.to(DEV))
+    orc = oracle.OracleLayer(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=r, max_iter=(1, 1),
+                             tol=(1e-2, 1e-2), capacity=4096, compute_dtype=torch.float64)
+    orc.prefill(Q, K, V, A_Q0=A_Q0, A_K0=A_K0)
+
+    def overlap():
+        a, o = eng.hit_indices.cpu()[..., 0], orc.hit_indices[..., 0]
+        same = 0
+        for h in range(hq):
+            same += len(set(a[0, h].tolist()) & set(o[0, h].tolist()))
+        return same / (hq * k)
+
+    ov = overlap()
+    _say("resident-set overlap after prefill: %.4f" % ov)
+    assert ov > 0.995, ov
+    stream = synth.DecodeStream(synth.Workload("t", hq, hkv, d, b, torch.float32, l, r, k, L, (1, 1), (1e-2, 1e-2),
+                                               steps, 32, 0.01), Q[:, :, -1:], (WQ, WK, WV), gen)
+    worst_ov, worst_attn = 1.0, 0.0
+    for step in range(steps):
+        q, kk, vv = stream.next()
+        eng.decode(q.to(DEV), kk.to(DEV), vv.to(DEV))
+        oK, oV = orc.decode(q, kk, vv)
+        worst_ov = min(worst_ov, overlap())
+        worst_attn = max(worst_attn, _rel(eng.last_attn, oracle.attention(q, oK, oV)))
+    _say("worst overlap %.4f, worst attention deviation %.2e over %d steps" % (worst_ov, worst_attn, steps))
+    DEVIATIONS["independent:1-overlap"] = 1.0 - worst_ov
+    DEVIATIONS["independent:attention"] = worst_attn
+    assert worst_ov > 0.99, worst_ov
+    assert worst_attn < 1e-3, worst_attn
 
 
 def test_cache_front_door(lrqk, oracle):
@@ -373,9 +619,23 @@ def test_cast_functions(lrqk, oracle):
     A_Q, B_Q, A_K, B_K = out          # a generator, unpacked like the reference's callers do
     ref = oracle.als_prefill_w1(Q.double(), K.double(), A0.double(), A0.flip(2).double(), 3, 0.0)
     assert _rel(A_K @ B_K, ref[2] @ ref[3]) < 1e-3 and _rel(A_Q @ B_Q, ref[0] @ ref[1]) < 1e-3
+    from lrqk_amd import factor
     for m in ("top", "topcol", lrqk.InitAQAK.randn):
         o = tuple(lrqk.cast_lrqk_prefill(Q.to(DEV), K.to(DEV), r, max_iter=1, tol=0.0, init_method=m))
         assert o[0].shape == (b, H, l, r) and torch.isfinite(o[3]).all()
+        if m == lrqk.InitAQAK.randn:
+            continue
+        # the column-picking initialisers (py:154-185) against the oracle's: the same columns, hence the same
+        # initial factors bit for bit, and the factorisation started from them against fp64
+        a0, k0 = factor._init_AQ_AK(Q.to(DEV), K.to(DEV), r, m)
+        e0, f0 = oracle.init_aq_ak(Q, K, r, m)
+        assert torch.equal(a0.cpu(), e0) and torch.equal(k0.cpu(), f0), m
+        ref = oracle.cast_lrqk_prefill(Q, K, r, 1, 0.0, init_method=m, compute_dtype=torch.float64)
+        for name, x, y in (("A_K B_K", o[2].cpu() @ o[3].cpu(), ref[2] @ ref[3]),
+                           ("A_Q B_Q", o[0].cpu() @ o[1].cpu(), ref[0] @ ref[1]),
+                           ("A_Q A_K^T", o[0].cpu()[:, :, -1:] @ o[2].cpu().transpose(-1, -2),
+                            ref[0][:, :, -1:] @ ref[2].transpose(-1, -2))):
+            _note("init_" + m, name, _rel(x, y), 1e-3)
     with pytest.raises(ValueError):
         tuple(lrqk.cast_lrqk_prefill(Q.to(DEV), K.to(DEV), r, init_method="nope"))
     # decode cast: inputs untouched, outputs match the oracle

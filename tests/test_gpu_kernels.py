@@ -104,6 +104,36 @@ def test_score_select_full_size(ops, ws, oracle, dtype, r):
         assert torch.all(got[..., 1:] > got[..., :-1]) and int(got.max()) < m
 
 
+@pytest.mark.parametrize("H,m", [(4, 131072 - 65), (32, 270000)])
+def test_score_select_full_size_with_score_index(ops, oracle, H, m):
+    """The default scan of the decode step (8-bit score index, bf16, r 32, k 2048) at the full 128K range,
+    and beyond it at the width of the Llama shape (32 heads x 270K rows: each workgroup of the scan walks
+    more than its usual two tiles).  First call: no threshold carried yet, every head rescans; later calls
+    with a drifting query: the prefiltered list.  Bit-exact against the oracle's full sort each time."""
+    _say("score_select full size with score index", H, m)
+    from lrqk_amd import synth
+    ws = ops.Workspace()
+    ws.score_index(True)
+    g = torch.Generator().manual_seed(70 + H)
+    r, k, cap = 32, 2048, m + 64
+    A = (torch.randn((1, H, cap, r), generator=g) * 0.7).bfloat16()
+    q = torch.randn((1, H, 1, r), generator=g)
+    Ad = A.to(DEV)
+    oracle.set_threads(16)
+    try:
+        for step in range(3):
+            qb = q.bfloat16()
+            exp = oracle.compute_hit_indices(qb, A[:, :, :m + step], k, True)[..., 0].to(torch.int32)
+            got = ops.score_select(ws, Ad, qb.to(DEV), m + step, k, True).cpu()
+            assert torch.equal(got, exp), step
+            q = synth.rotate_query(g, q, 0.05)
+    finally:
+        oracle.set_threads(1)
+    fast, full = ws.select_stats()
+    _say("heads from the prefiltered list / rescanned:", fast, full)
+    assert full >= H and fast >= H, (fast, full)
+
+
 def test_score_select_filtered_path(ops, oracle):
     """Repeated calls on one workspace with a slowly drifting query: after the first call the
     heads are served from the candidate list of the streaming filter; every result must
@@ -589,3 +619,40 @@ def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
         rel = (x - y).norm() / y.norm()
         # the individual factors depend on the conditioning of the r x r systems: 5e-3
         assert rel < (5e-3 if name in ("A_K", "B_K", "A_Q", "B_Q") else 1e-3), (name, float(rel))
+
+
+def test_als_prefill_benchmark_configuration(ops, ws, oracle):
+    """The prefill-factorisation benchmark exactly as it is specified: 32 query / 8 kv heads, 32768 tokens,
+    d 128, bf16 rows of rank 48 plus N(0, 0.05) noise, r 32, max_iter 4, tol 1e-8 -- against the fp64 oracle
+    on four query heads (of different kv groups), together with both fit residuals."""
+    _say("als_prefill benchmark configuration")
+    from lrqk_amd import synth
+    w = synth.WORKLOADS["llama8b_32k_prefill_als"]
+    l, r, d = w.context, w.r, w.head_dim
+    assert (w.num_heads, w.num_kv_heads, l, r, w.max_iter[0], w.tol[0], w.rho, w.sigma) == (32, 8, 32768, 32, 4, 1e-8, 48, 0.05)
+    Qd, Kd, _, _, _ = synth.prompt_qkv(w, 0, l, device=DEV)
+    A0 = synth.init_factors(w, l, 1, device=DEV)
+    got = ops.als_prefill(ws, Qd, Kd, A0[0].clone(), A0[1].clone(), w.max_iter[0], w.tol[0])
+    heads = [0, 9, 22, 31]
+    g = w.groups
+    Q = Qd[:, heads].cpu().double()
+    K = Kd[:, [h // g for h in heads]].cpu().double()
+    ref = oracle.als_prefill_w1(Q, K, A0[0][:, heads].cpu().double(), A0[1][:, heads].cpu().double(), w.max_iter[0], w.tol[0])
+    AQ, BQ, AK, BK = [t[:, heads].cpu().double() for t in got]
+
+    def rel(x, y):
+        return float((x - y).norm() / y.norm())
+
+    # fp32 arithmetic (bf16 matrix cores on three-way split operands) against fp64: 1e-3 on what the path uses,
+    # 5e-3 on the individual factors (conditioning of the r x r systems)
+    for name, x, y, lim in (("A_K B_K", AK @ BK, ref[2] @ ref[3], 1e-3), ("A_Q B_Q", AQ @ BQ, ref[0] @ ref[1], 1e-3),
+                            ("A_Q[-1] A_K^T", AQ[:, :, -1:] @ AK.transpose(-1, -2), ref[0][:, :, -1:] @ ref[2].transpose(-1, -2), 1e-3),
+                            ("A_K", AK, ref[2], 5e-3), ("B_K", BK, ref[3], 5e-3), ("A_Q", AQ, ref[0], 5e-3), ("B_Q", BQ, ref[1], 5e-3)):
+        dev = rel(x, y)
+        print("  %-14s deviation from fp64 %.2e (limit %.0e)" % (name, dev, lim), flush=True)
+        assert dev < lim, (name, dev)
+    res_g, res_o = rel(AK @ BK, K), rel(ref[2] @ ref[3], K)
+    resq_g, resq_o = rel(AQ @ BQ, Q), rel(ref[0] @ ref[1], Q)
+    print("  residual K: kernel %.6f oracle %.6f; residual Q: kernel %.6f oracle %.6f" % (res_g, res_o, resq_g, resq_o),
+          flush=True)
+    assert abs(res_g - res_o) < 1e-4 and abs(resq_g - resq_o) < 1e-4

@@ -208,3 +208,41 @@ def test_attention_vs_sdpa(oracle, dtype):
     assert torch.allclose(out, ref, atol=1e-12)
     # one key: the output is that value row
     assert torch.allclose(oracle.attention(q, K[:, :, :1], V[:, :, :1]), V[:, :, :1].double())
+
+
+def test_fp32_run_against_fp64_run_on_rank_r_data(oracle):
+    """How far an fp32 run of the prefill factorisation is from an fp64 run of the same algorithm on the
+    decode benchmark's data (rows of rank 32 plus N(0, 0.01) noise, bf16, r 32, max_iter 2, Llama head
+    size): the r x r systems reach condition numbers of 1e5..1e6, so the individual factors of the two runs
+    differ by percents, while everything the path uses them for (the fits A_K B_K, A_Q B_Q and the proxy
+    scores A_Q[-1] A_K^T) agrees to better than 2e-3.  This is why the GPU traces at that shape compare
+    products, with a limit of three times this deviation, and not the factors element by element.  On the
+    prefill benchmark's data (rank 48 + 0.05 noise) the systems are benign and the factors agree as well."""
+    from lrqk_amd import synth
+    orc = oracle
+
+    def run(rho, sigma, iters):
+        g = torch.Generator().manual_seed(0)
+        b, hq, hkv, l, d, r = 1, 4, 1, 8192, 128, 32
+        Q, _ = synth.low_rank_noise(g, b, hq, l, d, rho, sigma, torch.bfloat16)
+        K, _ = synth.low_rank_noise(g, b, hkv, l, d, rho, sigma, torch.bfloat16)
+        A_Q0 = torch.randn((b, hq, l, r), generator=g)
+        A_K0 = torch.randn((b, hq, l, r), generator=g)
+        Kr = orc.repeat_kv(K, hq // hkv)
+        r64 = orc.als_prefill_w1(Q.double(), Kr.double(), A_Q0.double(), A_K0.double(), iters, 0.0)
+        r32 = orc.als_prefill_w1(Q.float(), Kr.float(), A_Q0.float(), A_K0.float(), iters, 0.0)
+        rel = lambda x, y: float((x.double() - y).norm() / y.norm())
+        factors = {n: rel(x, y) for n, x, y in zip(("A_Q", "B_Q", "A_K", "B_K"), r32, r64)}
+        prods = {"A_K B_K": rel(r32[2] @ r32[3], r64[2] @ r64[3]), "A_Q B_Q": rel(r32[0] @ r32[1], r64[0] @ r64[1]),
+                 "scores": rel(r32[0][:, :, -1:] @ r32[2].transpose(-1, -2), r64[0][:, :, -1:] @ r64[2].transpose(-1, -2))}
+        cond = float(torch.linalg.cond(r64[0].transpose(-1, -2) @ r64[0]).max())
+        return factors, prods, cond
+
+    factors, prods, cond = run(32, 0.01, 2)
+    print("rank-32 data: cond %.1e factors %s products %s" % (cond, factors, prods))
+    assert cond > 1e4
+    assert max(factors.values()) > 5e-3          # the factors themselves are not comparable at 1e-3 ...
+    assert max(prods.values()) < 2e-3            # ... their products are
+    factors, prods, cond = run(48, 0.05, 4)
+    print("rank-48 data: cond %.1e factors %s products %s" % (cond, factors, prods))
+    assert cond < 1e4 and max(factors.values()) < 1e-4 and max(prods.values()) < 1e-4
