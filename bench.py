@@ -46,9 +46,10 @@ def parse():
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--cpu-steps", type=int, default=3, help="oracle steps timed for cpu_baseline (0 = skip)")
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
-    p.add_argument("--event-every", type=int, default=8,
+    p.add_argument("--event-every", type=int, default=0,
                    help="bracket every n-th proxy-score launch of the timed region with HIP events (each pair "
-                        "of event packets delays its step by ~10 us, so every launch would inflate the step time)")
+                        "of event packets delays its step by ~10 us, so every launch would inflate the step time); "
+                        "0 = every 8th, or more often so that at least 32 launches are bracketed")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
@@ -56,7 +57,7 @@ def parse():
     p.add_argument("--no-score-index", action="store_true",
                    help="scan the bf16 A_K rows directly instead of their 8-bit score index")
     p.add_argument("--victim-rows", type=int, default=-1,
-                   help="rows per head of the device-side cache of evicted K/V rows (-1: k, 0: off)")
+                   help="rows per head of the device-side cache of evicted K/V rows (-1: 4 k, 0: off)")
     p.add_argument("--mode", default="decode", choices=["decode", "prefill_als", "decoder"],
                    help="prefill_als: time the prefill factorisation alone (workload llama8b_32k_prefill_als unless "
                         "--workload is given); a step is one whole factorisation.  decoder: greedy decoding with a "
@@ -69,10 +70,16 @@ def parse():
                    help="decode mode: further untimed steps before the warm-up steps.  The first process on a box "
                         "enqueues its first few hundred steps several times slower than later ones (cold host-side "
                         "launch path), slower than the GPU executes them, and 16 warm-up steps do not get past that")
-    p.add_argument("--rotate", type=int, default=1,
+    p.add_argument("--rotate", type=int, default=4,
                    help="decode mode: step this many independent copies of the layer's state in turn (as the layers "
                         "of a decoder do), so that no copy finds its buffers in the 256 MB last-level cache; the "
-                        "value stays the time per layer-step; counters and kernel timing are taken from the first copy")
+                        "value is the time per layer-step; kernel timing is taken from the first copy.  1 = one "
+                        "copy stepped back to back (its score index stays in that cache)")
+    p.add_argument("--warm-steps", type=int, default=128,
+                   help="decode mode: after the timed region, step the first copy alone this many times and report "
+                        "that (cache-warm) time per step as a secondary figure; 0 = skip")
+    p.add_argument("--probe-mb", type=int, default=1024,
+                   help="decode mode: size of the plain read / copy kernels whose rates are reported beside the scan's")
     p.add_argument("--calib-copy-mb", type=int, default=0,
                    help="after the timed region, run one plain device copy of this many MiB (a known-size "
                         "kernel to scale hardware counters by)")
@@ -137,6 +144,23 @@ def prefill_als(a):
         num_q += float((Qh - AQ[:, h] @ BQ[:, h]).pow(2).sum()); den_q += float(Qh.pow(2).sum())
     bh = w.batch * w.num_heads
     r, d = w.r, w.head_dim
+    cpu = None
+    if a.cpu_steps > 0:
+        # the oracle's fp32 run of the same factorisation on a few heads, scaled to all heads
+        from oracle import lrqk_oracle as orc
+        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        hs = list(range(0, w.num_heads, max(1, w.num_heads // 4)))[:4]
+        Qc = Q[:, hs].float().cpu()
+        Kc = K[:, [h // g for h in hs]].float().cpu()
+        a0, k0 = A0[0][:, hs].cpu(), A0[1][:, hs].cpu()
+        orc.als_prefill_w1(Qc[:, :1], Kc[:, :1], a0[:, :1], k0[:, :1], 1, tol)   # untimed warm-up
+        t0 = time.perf_counter()
+        orc.als_prefill_w1(Qc, Kc, a0, k0, iters, tol)
+        cpu_ms = (time.perf_counter() - t0) * 1e3 * (w.batch * w.num_heads / len(hs))
+        cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": threads, "kind": "port",
+               "sample": f"fp32 torch-CPU factorisation of {len(hs)} of the {w.num_heads} heads at the full length "
+                         f"on {threads} threads, scaled to all heads"}
     # one pass = apply (2 l d r) + Grams (2 l r (r + d)); 2 initial Gram passes + 2 passes per iteration
     flops = bh * (2 * 2.0 * l * r * (r + d) + iters * 2 * (2.0 * l * d * r + 2.0 * l * r * (r + d)))
     e = 2 if w.dtype == torch.bfloat16 else 4
@@ -168,7 +192,7 @@ def prefill_als(a):
                       "max_iter": iters, "tol": tol, "input_dtype": "bf16" if e == 2 else "f32"},
            "rel_residual_K": round((num_k / den_k) ** 0.5, 6), "rel_residual_Q": round((num_q / den_q) ** 0.5, 6),
            "roofline": roof,
-           "cpu_baseline": None}
+           "cpu_baseline": cpu}
     print(json.dumps(out))
 
 
@@ -220,6 +244,7 @@ def main():
     from lrqk_amd import synth
     import lrqk_amd
     from lrqk_amd import _lib
+    from lrqk_amd import ops as ops_mod
     _lib.load()  # fail loudly if the HIP library is missing
     if a.mode == "prefill_als":
         return prefill_als(a)
@@ -259,7 +284,9 @@ def main():
     stream = synth.DecodeStream(w, Q[:, :, -1:], bases, gen)
     a.warmup_asked = a.warmup
     a.warmup += max(0, a.settle)  # all untimed alike; the line reports both numbers
-    total = a.warmup + a.steps
+    copies = 1 + len(others)
+    warm_steps = max(0, a.warm_steps) if copies > 1 else 0
+    total = a.warmup + a.steps + warm_steps
     qs, ks, vs = [], [], []
     for _ in range(total):
         q, k, v = stream.next()
@@ -273,7 +300,6 @@ def main():
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
 
-    miss = sel = 0
     for i in range(a.warmup):
         eng.decode(qs[i], ks[i], vs[i])
         for o_ in others:
@@ -284,40 +310,73 @@ def main():
     cap_before = (eng._A_K.capacity, eng.KVcpu.capacity)
     m_first = eng.lite_indices[eng.lite_len] - 1
 
-    eng.ws.timing_enable(a.steps, every=max(1, a.event_every))
+    # at least 32 bracketed launches (when there are that many steps), at most every 8th
+    every = a.event_every if a.event_every > 0 else max(1, min(8, a.steps // 32))
+    eng.ws.timing_enable(a.steps, every=every)
     eng.ws.select_stats(reset=True)
     eng.ws.victim_stats(reset=True)
     counts = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    # The host enqueues a step in less than half the time the GPU needs for it.  Left alone it runs thousands
+    # of launches ahead, and once the runtime's launch queue is full (at about 2000 launches here) every
+    # further launch waits in a way that leaves gaps on the GPU.  So the host stays at most 128 layer-steps
+    # ahead: it waits for a mark recorded that long ago, which the GPU passed long before, and the GPU never
+    # runs dry.  The same marks (one per 32 layer-steps) give the spread of the step time.
+    mark_every = max(1, 32 // copies)   # engine iterations between marks
+    ahead = max(2, 128 // (mark_every * copies))
     marks = []
-    chunk = max(8, 64 // (1 + len(others)))  # (64 layer-steps per chunk, however many copies take turns)
-    for i in range(a.warmup, total):
-        # The host enqueues a step in less than half the time the GPU needs for it.  Left alone it runs thousands
-        # of launches ahead, and once the runtime's launch queue is full (at about 2000 launches here) every
-        # further launch waits in a way that leaves gaps on the GPU (512 steps: 128 us per step instead of 86).
-        # So the host stays at most 128 steps ahead: it waits for the mark recorded two chunks of 64 steps ago,
-        # which the GPU passed long before, and the GPU never runs dry.
-        if (i - a.warmup) % chunk == 0:
-            marks.append(torch.cuda.Event())
-            marks[-1].record()
-            if len(marks) > 2:
-                marks[-3].synchronize()
-        eng.decode(qs[i], ks[i], vs[i])
-        counts.append(eng.last_miss_count)
-        for o_ in others:
-            o_.decode(qs[i], ks[i], vs[i])
+
+    def timed_loop(first, count, engines):
+        for i in range(first, first + count):
+            if (i - first) % mark_every == 0:
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[-1].record()
+                if len(marks) > ahead:
+                    marks[-1 - ahead].synchronize()
+            for j, e_ in enumerate(engines):
+                e_.decode(qs[i], ks[i], vs[i])
+                if j == 0:
+                    counts.append(e_.last_miss_count)
+        marks.append(torch.cuda.Event(enable_timing=True))
+        marks[-1].record()
+
+    timed_loop(a.warmup, a.steps, [eng] + others)
     torch.cuda.synchronize()
-    elapsed = (time.perf_counter() - t0) / (1 + len(others))
+    elapsed = (time.perf_counter() - t0) / copies
     kern_ms, launches = eng.ws.timing_read()
     eng.ws.timing_enable(0)
+    # per-mark-interval time per layer-step (the last interval may be shorter)
+    spans = []
+    for j in range(len(marks) - 1):
+        n_it = min(mark_every, a.steps - j * mark_every)
+        if n_it > 0:
+            spans.append(marks[j].elapsed_time(marks[j + 1]) * 1e3 / (n_it * copies))
+    spans.sort()
+
+    def pct(p_):
+        return round(spans[min(len(spans) - 1, int(p_ * len(spans)))], 2) if spans else None
+
     sel_fast, sel_full = eng.ws.select_stats()
     sel_short, sel_over = eng.ws.select_stats_detail()
     host_rows = eng.ws.victim_stats()
+    rows_scanned, rows_rescored = eng.ws.scan_stats()
     vic_on = eng.victim_rows_effective > 0 and a.fetch == "direct" \
         and not a.no_attn and a.variant == "default"
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
+    n_timed = len(counts)
+
+    # the same state stepped back to back: its score index largely stays in the last-level cache
+    warm_us = None
+    if warm_steps:
+        marks.clear()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        timed_loop(a.warmup + a.steps, warm_steps, [eng])
+        torch.cuda.synchronize()
+        warm_us = (time.perf_counter() - t1) / warm_steps * 1e6
+    counts = counts[:n_timed]
 
     n_miss = int(torch.stack(counts).sum())
     n_sel = len(counts) * w.batch * w.num_heads * w.num_active_tokens
@@ -325,19 +384,28 @@ def main():
     row_bytes = 2 * w.head_dim * e
     us_step = elapsed / a.steps * 1e6
     m_avg = (m_first + m_last) / 2.0
-    scan_bytes = w.batch * w.num_heads * m_avg * w.r * e
-    kern_us = kern_ms * 1e3 / max(launches, 1)
-    achieved = scan_bytes / (kern_us * 1e-6) / 1e9 if launches else 0.0
-    n_act = w.num_active_tokens + w.lite_tokens
     bh = w.batch * w.num_heads
+    scan_bytes = bh * m_avg * w.r * e            # what the reference's scan reads: r values per cached token and head
+    kern_us = kern_ms * 1e3 / max(launches, 1)
+    n_act = w.num_active_tokens + w.lite_tokens
     step_bytes = (scan_bytes + (0 if a.no_attn else 2 * bh * n_act * w.head_dim * e) + bh * n_act * w.head_dim * e
                   + bh * n_act * w.r * e + 4 * bh * w.r * w.head_dim * e + 3 * bh * w.num_active_tokens * 4
                   + n_miss / a.steps * row_bytes)
 
     sidx_on = (not a.no_score_index) and w.r in (16, 32, 64)
+    # Bytes one launch of the scan has to move.  Without the score index: the A_K rows.  With it: the 8-bit copy
+    # (r + 4 bytes per row) plus the rows it rescores exactly from A_K (counted by the kernel; last launch) plus
+    # the candidate pairs it writes -- fewer bytes than the reference's scan reads, which is the point of it.
+    if sidx_on and rows_scanned:
+        must_move = bh * m_avg * (w.r + 4) + rows_rescored * w.r * e + 8.0 * rows_rescored
+    else:
+        must_move = scan_bytes
+    achieved = must_move / (kern_us * 1e-6) / 1e9 if launches else 0.0
     traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) if a.context is None and a.variant == "default" else None
-    if others:
-        traffic = None  # the counters were read on a single copy
+
+    read_gbs = copy_gbs = None
+    if a.probe_mb > 0:
+        read_gbs, copy_gbs = ops_mod.probe_bandwidth(a.probe_mb << 20, 10, dev)
 
     if a.calib_copy_mb > 0:
         src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -376,7 +444,11 @@ def main():
         "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
                    "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
                    "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last],
-                   "layer_copies": 1 + len(others)},
+                   "layer_copies": copies,
+                   "cache": "cold: %d copies of the layer state take turns, as the layers of a decoder do" % copies
+                   if copies > 1 else "warm: one copy stepped back to back"},
+        "us_per_step_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
+        "us_per_step_one_copy_back_to_back": round(warm_us, 2) if warm_us else None,
         "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
@@ -386,15 +458,21 @@ def main():
                          "served": round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0},
         "step_algorithmic_bytes": round(step_bytes),
         "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-        # achieved = algorithmic bytes of the scan (r values of the storage type per cached token and head) over
-        # the kernel's duration; with the score index the kernel moves fewer bytes than that (see traffic), so
-        # the algorithmic rate can exceed what the memory system actually delivered (traffic_gbs).
+        # achieved = bytes the scan kernel has to move per launch (see must_move above) over its duration, so
+        # frac is a fraction of the HBM peak; algorithmic_equiv_gbs prices the same duration at the bytes the
+        # reference's scan reads (r values of the storage type per cached token and head), which the score
+        # index undercuts; traffic = HBM bytes per launch read from hardware counters (profiles/).
         "roofline": {"bound": "hbm", "kernel": "score_prefilter_kernel" if sidx_on else "score_filter_kernel",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": round(traffic) if traffic else None,
                      "traffic_gbs": round(traffic / (kern_us * 1e-6) / 1e9, 1) if traffic and launches else None,
-                     "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(scan_bytes)},
+                     "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(must_move),
+                     "rows_rescored_per_launch": rows_rescored,
+                     "algorithmic_bytes_per_launch": round(scan_bytes),
+                     "algorithmic_equiv_gbs": round(scan_bytes / (kern_us * 1e-6) / 1e9, 1) if launches else None,
+                     "measured_read_gbs": round(read_gbs, 1) if read_gbs else None,
+                     "measured_copy_gbs": round(copy_gbs, 1) if copy_gbs else None},
         "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full, "list_short": sel_short,
                            "list_overflow": sel_over},
         "cpu_baseline": cpu,

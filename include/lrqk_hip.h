@@ -76,6 +76,11 @@ int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads, int reset
  * than k candidates, lists that overflowed. */
 int lrqk_select_stats_detail(lrqk_ctx* ctx, int* list_short, int* list_overflow);
 
+/* Work of the last scan that went through the score index: rows it covered (all heads) and rows whose
+ * bound reached the threshold and were rescored exactly from a_k (0 / 0 if the last scan read a_k itself).
+ * Copies from the device (synchronises).  No counterpart in the reference. */
+int lrqk_scan_stats(lrqk_ctx* ctx, int64_t* rows_scanned, int64_t* rows_rescored);
+
 /* py:1275-1315 only_indices_in_cpu -- hit/miss diff, in place.
  * hit: [bh][hit_stride] current GPU-resident token ids (first k used), any order, unique.
  * new_idx: [bh][new_stride] ascending, unique.  On return the j-th evicted slot (ascending
@@ -228,6 +233,14 @@ int lrqk_timing_enable(lrqk_ctx* ctx, int max_launches);
  * them by a few microseconds, which a sampled measurement keeps out of most steps. */
 int lrqk_timing_stride(lrqk_ctx* ctx, int every);
 int lrqk_timing_read(lrqk_ctx* ctx, double* total_ms, int* launches);
+
+/* No counterpart in the reference.  Plain streaming kernels of known size on the caller's stream: `reps`
+ * reads of src[0, bytes) and `reps` copies of it to dst, each series timed with HIP events; returns the
+ * average milliseconds per pass (waits for the stream).  What the memory system delivers on the GPU at
+ * hand, to read the scan's rate against, and a transfer of known size to scale hardware counters by.
+ * src, dst: device memory, 16-byte aligned, bytes a multiple of 16. */
+int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, int reps, double* read_ms, double* copy_ms,
+                         void* stream);
 
 /* Host-side row gathers with the reference's native signatures (the staged fetch path
  * and API parity); multi-threaded memcpy.

@@ -66,10 +66,12 @@ def _sig(lib):
         "lrqk_decode_step": ([vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32,
                               i32, i32, i64, i64, i32, f32, i32, i32, vp, vp, vp, vp, vp, i32, vp], i32),
         "lrqk_select_stats": ([vp, c.POINTER(i32), c.POINTER(i32), i32], i32),
+        "lrqk_scan_stats": ([vp, c.POINTER(c.c_int64), c.POINTER(c.c_int64)], i32),
         "lrqk_select_stats_detail": ([vp, c.POINTER(i32), c.POINTER(i32)], i32),
         "lrqk_timing_enable": ([vp, i32], i32),
         "lrqk_timing_stride": ([vp, i32], i32),
         "lrqk_timing_read": ([vp, c.POINTER(c.c_double), c.POINTER(i32)], i32),
+        "lrqk_probe_bandwidth": ([vp, vp, i64, i32, c.POINTER(c.c_double), c.POINTER(c.c_double), vp], i32),
         "lrqk_d0_indices_select": ([vp, vp, vp, i64, i64, i64, i32], i32),
         "lrqk_take_along_dim_with_mask": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32], i64),
     }

@@ -89,6 +89,8 @@ struct lrqk_ctx {
   int tev_seen = 0;    // launches seen since timing was enabled
   int sel_bh = 0;      // head count the selector state (t_low, counters) was initialised for
   int last_short = 0, last_overflow = 0;  // split of the rescans seen by the last lrqk_select_stats
+  int scan_wgs = 0;        // workgroups of the last scan through the score index (0: the last scan read A_K itself)
+  int64_t scan_rows = 0;   // rows that scan covered (all heads)
 };
 
 namespace lrqk {

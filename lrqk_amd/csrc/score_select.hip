@@ -20,6 +20,8 @@
 //                  occupied range fills the 4096 bins: one or two passes instead of three.
 //                  The selected ids are emitted in order through two bitmaps (key > T,
 //                  key == T) and, when asked, diffed in place against the resident set.
+#include <vector>
+
 #include "common.hpp"
 #include "ctx.hpp"
 #include "als_finish.hpp"
@@ -158,6 +160,8 @@ struct SelState {
   float* q_cur;
   int* cand_count;
   int* stats;
+  int* rescored;     // per workgroup of the last index scan: rows whose bound passed (rescored exactly)
+  int rescored_cap;
 };
 
 __global__ void init_select_state_kernel(SelState st, int bh) {
@@ -494,6 +498,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
   };
   // A workgroup takes tiles_per_wg consecutive tiles (2 unless the context is so long that the launch
   // would otherwise hold more workgroups than the GPU does at a time).
+  int resc_total = 0;  // (thread 0) rows handed to the exact rescoring so far
 #pragma unroll 1
   for (int tile = 0; tile < tiles_per_wg; ++tile) {
     const int64_t base = base0 + (int64_t)tile * kFiltRows;
@@ -503,7 +508,10 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
       if (m_count > kFiltTiles * kFiltRows - kFiltRows) {
         rescore();
         flush_hits(false);
-        if (tid == 0) m_count = 0;
+        if (tid == 0) {
+          resc_total += m_count;
+          m_count = 0;
+        }
         __syncthreads();
       }
     }
@@ -537,6 +545,10 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     }
   }
   __syncthreads();
+  if (tid == 0) {
+    const int slot = h * (int)gridDim.x + (int)blockIdx.x;
+    if (slot < st.rescored_cap) st.rescored[slot] = resc_total + m_count;
+  }
   rescore();
   flush_hits(true);
 }
@@ -1104,7 +1116,8 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
   // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | cand_count i32 [bh] |
   // stats i32 [3]: served from the list, rescans because the list was too short, because it overflowed
   void* before = ctx->cand_cnt.p;
-  if ((rc = ctx->cand_cnt.ensure((size_t)(5 * bh + 3) * 4))) return rc;
+  constexpr int kRescSlots = 8192;  // workgroups of one index scan (never more than the GPU holds at a time)
+  if ((rc = ctx->cand_cnt.ensure((size_t)(5 * bh + 3 + bh + kRescSlots) * 4))) return rc;
   uint32_t* base = (uint32_t*)ctx->cand_cnt.p;
   sb->st.t_low = base;
   sb->st.q_norm = (float*)(base + bh);
@@ -1112,6 +1125,8 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
   sb->st.q_cur = (float*)(base + 3 * bh);
   sb->st.cand_count = (int*)(base + 4 * bh);
   sb->st.stats = (int*)(base + 5 * bh);
+  sb->st.rescored = (int*)(base + 5 * bh + 3);
+  sb->st.rescored_cap = bh + kRescSlots;
   if (before != ctx->cand_cnt.p || ctx->sel_bh != bh) {
     hipLaunchKernelGGL(init_select_state_kernel, dim3((unsigned)((bh + 255) / 256)), dim3(256), 0, st, sb->st, bh);
     LRQK_HIP_CHECK(hipGetLastError());
@@ -1176,8 +1191,11 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
                          head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six,
                          tiles_per_wg);
       via_index = true;
+      ctx->scan_wgs = (int)std::min<int64_t>((int64_t)grid_ix.x * bh, sb.st.rescored_cap);
+      ctx->scan_rows = (int64_t)bh * m;
     }
   }
+  if (!via_index) ctx->scan_wgs = 0;
   if (!via_index)
     hipLaunchKernelGGL((score_filter_kernel<T, R>), grid, dim3(kFiltThreads), filt_smem, st, (const T*)a_k, head_stride,
                        (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq);
@@ -1337,6 +1355,20 @@ extern "C" int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int b
                      topk, out_idx, out_stride, df);
   LRQK_HIP_CHECK(hipGetLastError());
   return topk;
+}
+
+extern "C" int lrqk_scan_stats(lrqk_ctx* ctx, int64_t* rows_scanned, int64_t* rows_rescored) {
+  LRQK_REQUIRE(ctx && rows_scanned && rows_rescored, LRQK_EINVAL, "null pointer");
+  *rows_scanned = *rows_rescored = 0;
+  if (!ctx->cand_cnt.p || ctx->sel_bh <= 0 || ctx->scan_wgs <= 0) return LRQK_OK;
+  std::vector<int> v((size_t)ctx->scan_wgs);
+  LRQK_HIP_CHECK(hipMemcpy(v.data(), (int*)ctx->cand_cnt.p + 5 * ctx->sel_bh + 3, v.size() * sizeof(int),
+                           hipMemcpyDeviceToHost));
+  int64_t t = 0;
+  for (int x : v) t += x;
+  *rows_scanned = ctx->scan_rows;
+  *rows_rescored = t;
+  return LRQK_OK;
 }
 
 extern "C" int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads, int reset) {

@@ -83,6 +83,12 @@ class Workspace:
         check(_lib.load().lrqk_select_stats(self._h, ctypes.byref(a), ctypes.byref(b), 1 if reset else 0))
         return a.value, b.value
 
+    def scan_stats(self):
+        """(rows covered, rows rescored exactly) by the last scan through the score index; (0, 0) otherwise."""
+        a, b = ctypes.c_int64(), ctypes.c_int64()
+        check(_lib.load().lrqk_scan_stats(self._h, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
     def select_stats_detail(self):
         """(lists too short, lists overflowed) among the rescans of the last select_stats()."""
         a, b = ctypes.c_int(), ctypes.c_int()
@@ -347,6 +353,16 @@ def decode_step(ws: Workspace, b_q, b_k, a_k, active_idx, k_act, v_act, kv_store
         r, d, topk, lite, ring_slot, token, m, flush_row0, int(max_iter), float(tol),
         1 if (round_scores and b_q.dtype == torch.bfloat16) else 0, 1 if no_hit_miss else 0, q_hat.data_ptr(),
         k_hat.data_ptr(), _ptr(attn_out), _ptr(evict), _ptr(miss_count), _dt(b_q), _stream(b_q)))
+
+
+def probe_bandwidth(nbytes: int, reps: int = 10, device="cuda:0"):
+    """(read GB/s, copy GB/s of bytes read + bytes written) of plain streaming kernels over ``nbytes``."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    r_ms, c_ms = ctypes.c_double(), ctypes.c_double()
+    check(_lib.load().lrqk_probe_bandwidth(src.data_ptr(), dst.data_ptr(), nbytes, reps, ctypes.byref(r_ms),
+                                           ctypes.byref(c_ms), _stream(src)))
+    return nbytes / (r_ms.value * 1e-3) / 1e9, 2 * nbytes / (c_ms.value * 1e-3) / 1e9
 
 
 # --------------------------------------------------------------------------- host gathers
