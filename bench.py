@@ -66,6 +66,9 @@ def parse():
     p.add_argument("--batch", type=int, default=4, help="decoder mode: sequences")
     p.add_argument("--prompt", type=int, default=65536, help="decoder mode: prompt tokens per sequence")
     p.add_argument("--new-tokens", type=int, default=128, help="decoder mode: tokens decoded per sequence")
+    p.add_argument("--seqs", type=int, default=0,
+                   help="decode mode: sequences stepped together (the batch of the layer-step; 0 = the workload's "
+                        "own, 1 for the 128K configuration); value stays the time of one layer-step of the whole batch")
     p.add_argument("--settle", type=int, default=512,
                    help="decode mode: further untimed steps before the warm-up steps.  The first process on a box "
                         "enqueues its first few hundred steps several times slower than later ones (cold host-side "
@@ -253,6 +256,9 @@ def main():
 
     dev = torch.device("cuda:0")
     w = synth.WORKLOADS[a.workload]
+    if a.seqs > 0 and a.seqs != w.batch:
+        import dataclasses
+        w = dataclasses.replace(w, batch=a.seqs)
     l = a.context or w.context
     t_setup = time.perf_counter()
     # synthetic prompt, drawn on the GPU (128K x 48 heads x 128 would take minutes on the host)
@@ -401,7 +407,8 @@ def main():
     else:
         must_move = scan_bytes
     achieved = must_move / (kern_us * 1e-6) / 1e9 if launches else 0.0
-    traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) if a.context is None and a.variant == "default" else None
+    traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) \
+        if a.context is None and a.variant == "default" and w.batch == 1 else None
 
     read_gbs = copy_gbs = None
     if a.probe_mb > 0:
@@ -441,15 +448,16 @@ def main():
         "ms_per_step": round(us_step / 1e3, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
-        "config": {"workload": f"{w.name}@{l}", "heads": [w.num_heads, w.num_kv_heads], "head_dim": w.head_dim,
-                   "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
+        "config": {"workload": f"{w.name}@{l}", "batch": w.batch, "heads": [w.num_heads, w.num_kv_heads],
+                   "head_dim": w.head_dim, "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
                    "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last],
                    "layer_copies": copies,
                    "cache": "cold: %d copies of the layer state take turns, as the layers of a decoder do" % copies
                    if copies > 1 else "warm: one copy stepped back to back"},
         "us_per_step_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
         "us_per_step_one_copy_back_to_back": round(warm_us, 2) if warm_us else None,
-        "tokens_per_s_32_layers": round(1e6 / (32 * us_step), 2),
+        "us_per_sequence_layer_step": round(us_step / w.batch, 2),
+        "tokens_per_s_32_layers": round(w.batch * 1e6 / (32 * us_step), 2),
         "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
         "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
         "missed_bytes_per_step": round(n_miss / a.steps * row_bytes),

@@ -128,7 +128,8 @@ int lrqk_fetch_rows_staged(lrqk_ctx* ctx, const void* kv_store, int64_t cap, voi
  * host_threads gather threads (<= 0 keeps the current count).  No counterpart in the reference. */
 int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
 
-/* Score index for the scan (no counterpart in the reference; off by default).  The ctx keeps an
+/* Score index for the scan (no counterpart in the reference; a new ctx has it off, the Python
+ * engine switches it on).  The ctx keeps an
  * 8-bit copy of the A_K rows (one scale per row, 36 instead of 64 bytes per row for r = 32) and the
  * scan of lrqk_score_select / lrqk_score_select_diff / lrqk_decode_step reads that copy: it bounds
  * every row's score and rescores exactly, from a_k itself, only the rows whose bound reaches the
@@ -137,7 +138,8 @@ int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
  * in place call this again (any value) to drop it.  Applies to r = 16, 32, 64. */
 int lrqk_ctx_score_index(lrqk_ctx* ctx, int enable);
 
-/* Victim cache for lrqk_decode_step (no counterpart in the reference; off by default).  K/V rows
+/* Victim cache for lrqk_decode_step (no counterpart in the reference; a new ctx has it off, the
+ * Python engine gives it 4 k rows per head).  K/V rows
  * that leave the top-k slots are kept in a per-head FIFO of rows_per_head rows on the device
  * (tokens near the selection threshold return within a few steps); a missed row that is still
  * there is copied from the FIFO instead of over the host link.  Results are identical: a token's
@@ -199,8 +201,9 @@ int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head
  * a_q,a_k: [bh][l][r] fp32 work buffers holding the initial factors on entry and the
  * result on return; b_q,b_k out: [bh][r][d] fp32.  The stopping test (batch-wide mean squared
  * change of A_Q and A_K below tol) is evaluated on the device: once it fires the remaining
- * launches return at once, and the host never waits.  r <= 32 and head dimensions that are a
- * multiple of 16 bytes run on fp32 MFMA tiles, other shapes on a generic kernel.  Returns 0. */
+ * launches return at once, and the host never waits.  r <= 32: bf16 input with d <= 128 runs on
+ * the bf16 matrix cores (fp32 operands as three bf16 pieces each, fp32 accumulation), fp32 input
+ * or d = 256 on fp32 MFMA tiles, other shapes on a generic kernel.  Returns 0. */
 int lrqk_als_prefill(lrqk_ctx* ctx, const void* q, const void* k, float* a_q, float* a_k, float* b_q,
                      float* b_k, int b, int hq, int hkv, int64_t l, int r, int d, int max_iter, float tol,
                      int dtype, void* stream);

@@ -132,42 +132,41 @@ class AutoIncreaseTensorSharedKV(AutoIncreaseTensor):
 
 
 class PreAllocatedTensor:
-    """Fixed-capacity buffer; overflow raises ValueError (lrqk_attention.py:966-1011)."""
+    """Bounded buffer along ``dim`` (interface of lrqk_attention.py:966-1011: ``capacity``, ``dim``,
+    ``dtype``, ``device``, ``data``, ``current_len``; ``append`` past the capacity raises ``ValueError``).
+    Storage appears with the first piece and takes its shape, dtype and device from it unless given."""
 
     def __init__(self, capacity: int, dim: int, dtype: torch.dtype = None, device: torch.device = None):
-        self.capacity = capacity
-        self.dim = dim
-        self.dtype = dtype
-        self.device = device
-        self.data = None
-        self.current_len = 0
+        self.capacity, self.dim = capacity, dim
+        self.dtype, self.device = dtype, device
+        self.data, self.current_len = None, 0
 
     @classmethod
     def from_tensor(cls, capacity: int, dim: int, data: torch.Tensor):
-        out = cls(capacity, dim, data.dtype, data.device)
-        out.append(data)
-        return out
+        buf = cls(capacity, dim, dtype=data.dtype, device=data.device)
+        buf.append(data)
+        return buf
+
+    def _window(self, start: int, length: int) -> torch.Tensor:
+        return self.data.narrow(self.dim, start, length)
 
     def append(self, x: torch.Tensor):
-        if self.dtype is None:
-            self.dtype = x.dtype
-        if self.device is None:
-            self.device = x.device
-        n = x.shape[self.dim]
+        self.dtype = x.dtype if self.dtype is None else self.dtype
+        self.device = x.device if self.device is None else self.device
         if self.data is None:
-            shape = list(x.shape)
-            shape[self.dim] = self.capacity
-            self.data = torch.empty(shape, dtype=self.dtype, device=self.device)
-        if self.current_len + n > self.capacity:
+            full = [self.capacity if ax == self.dim else size for ax, size in enumerate(x.shape)]
+            self.data = torch.empty(full, dtype=self.dtype, device=self.device)
+        end = self.current_len + x.shape[self.dim]
+        if end > self.capacity:
             raise ValueError("Not enough capacity to store the tensor")
-        self.data.narrow(self.dim, self.current_len, n).copy_(x)
-        self.current_len += n
+        self._window(self.current_len, end - self.current_len).copy_(x)
+        self.current_len = end
 
     def has_data(self):
         return self.data is not None
 
     def tensor(self) -> torch.Tensor:
-        return self.data.narrow(self.dim, 0, self.current_len)
+        return self._window(0, self.current_len)
 
     def __len__(self):
         return self.current_len
@@ -177,18 +176,23 @@ class PreAllocatedTensor:
 
 
 class _CacheQKV:
-    """Prompt pieces shorter than the active set wait here (lrqk_attention.py:1014-1028)."""
+    """The pieces of a prompt that is still shorter than the active set (interface of
+    lrqk_attention.py:1014-1028: members ``Q``, ``K``, ``V``; ``append`` returns what has been
+    collected so far; ``len`` is the number of positions held)."""
+
+    _NAMES = ("Q", "K", "V")
 
     def __init__(self, capacity: int, dim: int, dtype: torch.dtype = None, device: torch.device = None):
-        self.Q = PreAllocatedTensor(capacity, dim, dtype, device)
-        self.K = PreAllocatedTensor(capacity, dim, dtype, device)
-        self.V = PreAllocatedTensor(capacity, dim, dtype, device)
+        for name in self._NAMES:
+            setattr(self, name, PreAllocatedTensor(capacity, dim, dtype, device))
 
-    def append(self, Q, K, V):
-        self.Q.append(Q)
-        self.K.append(K)
-        self.V.append(V)
-        return self.Q.tensor(), self.K.tensor(), self.V.tensor()
+    def append(self, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor):
+        held = []
+        for name, piece in zip(self._NAMES, (Q, K, V)):
+            buf = getattr(self, name)
+            buf.append(piece)
+            held.append(buf.tensor())
+        return tuple(held)
 
     def __len__(self):
-        return self.Q.current_len
+        return len(self.Q)

@@ -248,10 +248,14 @@ extern "C" int lrqk_gather_rows(const void* src, int64_t src_len, const int32_t*
   LRQK_REQUIRE(count >= 0 && count <= n_slots && idx_stride >= count && src_len > 0, LRQK_EINVAL, "bad sizes");
   LRQK_REQUIRE(aligned16(src) && aligned16(dst), LRQK_EINVAL, "pointers must be 16-byte aligned");
   if (count == 0) return LRQK_OK;
+  // src may be pinned host memory (the reference's host branch of fetch_by_hit): read through its mapping
+  const void* dev_src = nullptr;
+  rc = lrqk::resolve_store(src, &dev_src);
+  if (rc) return rc;
   int64_t blocks = ((int64_t)count * cpr + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)blocks, (unsigned)(b * hq)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4*)src, src_len, idx, idx_stride, count, (uint4*)dst, n_slots, hq, hkv, cpr);
+                     (const uint4*)dev_src, src_len, idx, idx_stride, count, (uint4*)dst, n_slots, hq, hkv, cpr);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }

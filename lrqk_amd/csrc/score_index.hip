@@ -284,5 +284,6 @@ extern "C" int lrqk_ctx_score_index(lrqk_ctx* ctx, int enable) {
   ctx->sidx_enabled = enable != 0;
   ctx->sidx_a_k = nullptr;  // whatever was indexed is dropped; the next scan rebuilds what it needs
   ctx->sidx_valid = 0;
+  ctx->sel_bh = 0;  // the bound a scan carries to the next one is in the units of the scan that made it
   return LRQK_OK;
 }

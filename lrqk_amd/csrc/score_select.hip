@@ -410,15 +410,9 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     rs.init_from_lanes(qv, r, round_bf16);
     q_lane = sizeof(T) == 2 ? round_to_bf16_f32(qv) : qv;
   }
-  const float qn = rs.q_norm();
-  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn, round_bf16);
-  if (tid == 0 && blockIdx.x == 0) {
-    st.t_used[h] = tl;
-    st.q_cur[h] = qn;
-  }
   // q' from W q' = q, last unknown first; lane i keeps the residual of equation i
   float qc[R];
-  float qsum = 0.0f, ql1 = 0.0f;
+  float qsum = 0.0f, ql1 = 0.0f, ql2 = 0.0f;
   {
     float resid = q_lane;
 #pragma unroll
@@ -431,7 +425,17 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     for (int j = 0; j < R; ++j) {
       qsum += qc[j];
       ql1 += fabsf(qc[j]);
+      ql2 = fmaf(qc[j], qc[j], ql2);
     }
+  }
+  // The rows are white in the index's coordinates, so the scores of a head spread like |q'|, whatever
+  // the direction of the proxy query: the carried bound follows that norm (the plain scan, which has
+  // no transform, follows |q_hat|).
+  const float qn = sqrtf(ql2);
+  const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn, round_bf16);
+  if (tid == 0 && blockIdx.x == 0) {
+    st.t_used[h] = tl;
+    st.q_cur[h] = qn;
   }
   const float dfac = ql1 * kSidxDFactor;
   // float threshold; an unset bound (no key passes) keeps the list empty exactly like the plain filter
@@ -554,7 +558,10 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
 }
 
 // --------------------------------------------------------------------------- select (+ diff)
-constexpr int kSelThreads = 1024;
+#ifndef LRQK_SEL_THREADS
+#define LRQK_SEL_THREADS 1024
+#endif
+constexpr int kSelThreads = LRQK_SEL_THREADS;
 // The bound carried to the next call is the key of rank 1.5 k: the list then holds ~1.5 k candidates per
 // head and stays usable as long as the number of rows above the (rescaled) bound does not drop by a third
 // from one call to the next.  (2 k: 1.3 us slower per 128K step; 1.25 k: 3 rescans in 16384 head-steps.)
@@ -563,6 +570,8 @@ constexpr int kSelWaves = kSelThreads / kWave;
 constexpr int kChunkBits = 262144;            // token ids covered by one bitmap pass
 constexpr int kChunkWords = kChunkBits / 32;  // 8192 words = 32 KB per bitmap
 constexpr int kBins = 4096;
+constexpr int kBinsPT = kBins / kSelThreads;          // histogram bins per thread
+constexpr int kWordsPT = kChunkWords / kSelThreads;   // bitmap words per thread
 constexpr int kFusedDiffMaxK = 4096;          // LDS budget of the in-kernel diff
 
 // Inclusive block scan of two counters at once.  scratch: 2 * kSelWaves ints.  Two barriers.
@@ -620,17 +629,17 @@ __device__ __forceinline__ void block_rank2(bool pa, bool pb, int* scratch, int&
   tot_b = tb;
 }
 
-// From two histograms of kBins bins (4 bins per thread): the digit of the need_a-th largest
+// From two histograms of kBins bins (kBinsPT bins per thread): the digit of the need_a-th largest
 // element of hist_a and of the need_b-th largest of hist_b, with the ranks inside those
 // digits.  s_res: 4 shared ints.  Three barriers.
 __device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32_t* hist_b, int need_a, int need_b,
                                             int* scratch, int* s_res, int& dig_a, int& rem_a, int& dig_b, int& rem_b) {
   const int tid = threadIdx.x;
-  int ca[4], cb[4], la = 0, lb = 0;
+  int ca[kBinsPT], cb[kBinsPT], la = 0, lb = 0;
 #pragma unroll
-  for (int x = 0; x < 4; ++x) {
-    ca[x] = (int)hist_a[tid * 4 + x];
-    cb[x] = (int)hist_b[tid * 4 + x];
+  for (int x = 0; x < kBinsPT; ++x) {
+    ca[x] = (int)hist_a[tid * kBinsPT + x];
+    cb[x] = (int)hist_b[tid * kBinsPT + x];
     la += ca[x];
     lb += cb[x];
   }
@@ -640,9 +649,9 @@ __device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32
   if (above_a < need_a && need_a <= above_a + la) {
     int c = above_a;
 #pragma unroll
-    for (int x = 3; x >= 0; --x) {
+    for (int x = kBinsPT - 1; x >= 0; --x) {
       if (c < need_a && c + ca[x] >= need_a) {
-        s_res[0] = tid * 4 + x;
+        s_res[0] = tid * kBinsPT + x;
         s_res[1] = need_a - c;
       }
       c += ca[x];
@@ -651,9 +660,9 @@ __device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32
   if (above_b < need_b && need_b <= above_b + lb) {
     int c = above_b;
 #pragma unroll
-    for (int x = 3; x >= 0; --x) {
+    for (int x = kBinsPT - 1; x >= 0; --x) {
       if (c < need_b && c + cb[x] >= need_b) {
-        s_res[2] = tid * 4 + x;
+        s_res[2] = tid * kBinsPT + x;
         s_res[3] = need_b - c;
       }
       c += cb[x];
@@ -665,6 +674,12 @@ __device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32
   dig_b = s_res[2];
   rem_b = s_res[3];
 }
+
+#ifdef LRQK_SEL_STAMPS
+#define SEL_STAMP(i) do { if (threadIdx.x == 0) s_stamp[i] = wall_clock64(); } while (0)
+#else
+#define SEL_STAMP(i) do { } while (0)
+#endif
 
 struct DiffArgs {
   int32_t* hit;        // [bh][hit_stride] resident token ids, nullptr = no diff
@@ -698,6 +713,12 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   __shared__ uint32_t wred[2 * kSelWaves];
   __shared__ int s_res[4];
   __shared__ int s_n;
+#ifdef LRQK_SEL_STAMPS
+  __shared__ uint64_t s_stamp[16];
+  if (threadIdx.x < 16) s_stamp[threadIdx.x] = 0;
+  __syncthreads();
+#endif
+  SEL_STAMP(0);
   uint32_t* gt = dyn;
   uint32_t* eq = dyn + kChunkWords;
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
@@ -725,6 +746,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       st.cand_count[h] = 0;  // re-arm for the next call
     }
     __syncthreads();
+    SEL_STAMP(1);
     const int n = s_n;
     fast = n >= k && n <= cand_cap;
     if (fast) {
@@ -742,7 +764,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   }
   // The candidate list is read once into registers (one batch of independent loads); the
   // rescan path walks the key array in batches of 8 independent loads per thread.
-  constexpr int kRegCand = 8;
+  constexpr int kRegCand = 8192 / kSelThreads;
   const bool in_regs = fast && N <= (int64_t)kRegCand * kSelThreads;
   uint2 creg[kRegCand];
   if (in_regs) {
@@ -808,6 +830,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   }
   if (tid == 0) s_res[0] = s_res[1] = s_res[2] = s_res[3] = 0;
   __syncthreads();
+  SEL_STAMP(2);
   vmax = 0u;
   vor = 0u;
 #pragma unroll
@@ -824,8 +847,10 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   // ---- pass 1 (both ranks share it)
   for_each([&](uint32_t key, int64_t) { atomicAdd(&hist[((key - lo) >> tz) >> s1], 1u); });
   __syncthreads();
+  SEL_STAMP(3);
   int D1, need1, E1, needE;
   find_digits(hist, hist, k, k2, scratch, s_res, D1, need1, E1, needE);
+  SEL_STAMP(4);
   uint32_t offT = (uint32_t)D1 << s1, offE = (uint32_t)E1 << s1;
   int need_eq = need1;
   if (s1 > 0) {
@@ -865,6 +890,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       need_eq = need3;
     }
   }
+  SEL_STAMP(5);
   const uint32_t Tk = lo + (offT << tz);
   if (tid == 0) {
     st.t_low[h] = lo + (offE << tz);  // rank >= 1.5k (rounded down to the resolved bits)
@@ -890,15 +916,17 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       }
     }
     __syncthreads();
+    SEL_STAMP(6);
     for_each([&](uint32_t key, int64_t idx) {
       const int64_t rel = idx - c0;
       if (key >= Tk && rel >= 0 && rel < span) atomicOr(key > Tk ? &gt[rel >> 5] : &eq[rel >> 5], 1u << (rel & 31));
     });
     __syncthreads();
+    SEL_STAMP(7);
     const int w0 = tid * W;
-    uint32_t gwr[8], ewr[8];
+    uint32_t gwr[kWordsPT], ewr[kWordsPT];
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < kWordsPT / 4; ++q) {
       uint4 a = make_uint4(0, 0, 0, 0), b = a;
       if (q * 4 < W) {
         a = reinterpret_cast<const uint4*>(gt)[(w0 >> 2) + q];
@@ -909,16 +937,17 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
     int cg = 0, ce = 0;
 #pragma unroll
-    for (int x = 0; x < 8; ++x) {
+    for (int x = 0; x < kWordsPT; ++x) {
       cg += __popc(gwr[x]);
       ce += __popc(ewr[x]);
     }
     int g_incl = cg, e_incl = ce, g_tot, e_tot;
     block_inclusive_sum2(g_incl, e_incl, scratch, g_tot, e_tot);
+    SEL_STAMP(8);
     int e_run = eq_seen + e_incl - ce;  // equal keys before this thread's words (all chunks)
     int pos = out_pos + (g_incl - cg) + (min(e_run, need_eq) - min(eq_seen, need_eq));
 #pragma unroll
-    for (int x = 0; x < 8; ++x) {
+    for (int x = 0; x < kWordsPT; ++x) {
       const uint32_t gw = gwr[x], ew = ewr[x];
       uint32_t both = gw | ew;
       uint32_t sel = gw;
@@ -943,6 +972,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     out_pos += g_tot + (min(eq_seen + e_tot, need_eq) - min(eq_seen, need_eq));
     eq_seen += e_tot;
     __syncthreads();
+    SEL_STAMP(9);
   }
   if (!do_diff) return;
 
@@ -968,6 +998,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     const int words = (int)((m + 31) >> 5);
     for (int i = tid; i < words; i += kSelThreads) eq[i] = 0;
     __syncthreads();
+    SEL_STAMP(10);
 #pragma unroll
     for (int u = 0; u < kDiffIpt; ++u) {
       const int s = tid * ipt + u;
@@ -980,6 +1011,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       }
     }
     __syncthreads();
+    SEL_STAMP(11);
     for (int i = tid; i < k; i += kSelThreads) {
       const int32_t t = new_s[i];
       matched[i] = (uint8_t)((eq[t >> 5] >> (t & 31)) & 1u);
@@ -1023,6 +1055,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
   }
   __syncthreads();
+  SEL_STAMP(12);
   // both ordered compactions in one sweep: rank of missing tokens and of evicted slots
   int n_missing, n_evict;
   {
@@ -1047,6 +1080,7 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
   }
   __syncthreads();
+  SEL_STAMP(13);
   const int n_pair = min(n_missing, n_evict);
   const int32_t* ev_list = reinterpret_cast<const int32_t*>(gt);
   for (int j = tid; j < n_pair; j += kSelThreads) {
@@ -1065,6 +1099,14 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     for (int s = tid; s < k; s += kSelThreads) df.evict[(int64_t)h * k + s] = evict_s[s];
   }
   if (tid == 0 && df.miss_count) df.miss_count[h] = n_pair;
+#ifdef LRQK_SEL_STAMPS
+  __syncthreads();
+  SEL_STAMP(14);
+  if (tid == 0 && df.evict && k >= 128) {
+    uint32_t* o = reinterpret_cast<uint32_t*>(df.evict + (int64_t)h * k + k - 64);
+    for (int i = 0; i < 16; ++i) o[i] = s_stamp[i] ? (uint32_t)(s_stamp[i] - s_stamp[0]) : 0u;
+  }
+#endif
 }
 
 // --------------------------------------------------------------------------- host side

@@ -191,14 +191,19 @@ class LightAttentionIndicesFactory:
         """lrqk_attention.py:1317-1383.  dst [b,Hq,<=k,d] must be the topk area of Kgpu or Vgpu
         (a narrow view); src [b,Hkv,seq,d] on the GPU, or the pinned [K|V] store with dst_mask."""
         b, H = hit_indices.shape[:2]
-        idx = hit_indices.reshape(b, H, -1).to(torch.int32).contiguous()
+        idx = hit_indices.reshape(b, H, -1).to(device=dst.device, dtype=torch.int32)
         count = idx.shape[2]
-        if src.is_cuda:
-            full = self.Kgpu if dst.data_ptr() == self.Kgpu.data_ptr() else self.Vgpu
-            assert dst.data_ptr() == full.data_ptr(), "dst must be the topk area of Kgpu or Vgpu"
-            ops.gather_rows(src.contiguous(), idx, full, count)
-            return dst
-        raise NotImplementedError("host-side fetch goes through decode(); use ops.fetch_rows for a custom path")
+        full = self.Kgpu if dst.data_ptr() == self.Kgpu.data_ptr() else self.Vgpu
+        assert dst.data_ptr() == full.data_ptr(), "dst must be the topk area of Kgpu or Vgpu"
+        if not src.is_cuda:
+            # host source (:1351-1381): every listed row, or with dst_mask only the slots it marks; the
+            # kernel reads the pinned rows through their device mapping and skips negative ids
+            if not (src.is_pinned() and src.is_contiguous()):
+                raise ValueError("a host source must be contiguous pinned memory")
+            if dst_mask is not None:
+                idx = torch.where(dst_mask.reshape(b, H, -1).to(dst.device), idx, torch.full_like(idx, -1))
+        ops.gather_rows(src if not src.is_cuda else src.contiguous(), idx.contiguous(), full, count)
+        return dst if count >= self.attn_topk else dst.narrow(2, 0, count)
 
     # ------------------------------------------------------------------ prefill
     @torch.inference_mode()

@@ -241,13 +241,16 @@ def fetch_rows_staged(ws: Workspace, kv_store: torch.Tensor, k_act: torch.Tensor
 
 
 def gather_rows(src: torch.Tensor, idx: torch.Tensor, dst: torch.Tensor, count: int):
-    """dst[b,h,j,:] = src[b,h//g,idx[b,h,j],:] for j < count.  src [b,Hkv,l,d], dst [b,Hq,n,d]."""
-    _need_cuda(src, idx, dst)
+    """dst[b,h,j,:] = src[b,h//g,idx[b,h,j],:] for j < count; slots whose id is negative keep their
+    contents.  src [b,Hkv,l,d] on the GPU or in pinned host memory, dst [b,Hq,n,d]."""
+    _need_cuda(idx, dst)
+    if not src.is_cuda and not src.is_pinned():
+        raise ValueError("a host source must be pinned memory")
     b, hkv, l, d = src.shape
     _, hq, n, _ = dst.shape
     assert src.is_contiguous() and dst.is_contiguous() and idx.is_contiguous() and idx.dtype == torch.int32
     check(_lib.load().lrqk_gather_rows(src.data_ptr(), l, idx.data_ptr(), idx.shape[2], count, dst.data_ptr(), n, b, hq,
-                                       hkv, d, _dt(src), _stream(src)))
+                                       hkv, d, _dt(src), _stream(dst)))
 
 
 def append_token(k_new, v_new, k_act, v_act, slot: int, active_idx: Optional[torch.Tensor], token: int):

@@ -555,6 +555,38 @@ def test_independent_runs_agree(lrqk, oracle):
     assert worst_attn < 1e-3, worst_attn
 
 
+def test_fetch_by_hit_host_source(lrqk):
+    """fetch_by_hit with a pinned host source (lrqk_attention.py:1351-1381): all listed rows without a
+    mask, only the marked slots with one (the others keep their contents); against take_along_dim."""
+    _say("fetch_by_hit, host source")
+    gen = torch.Generator().manual_seed(5)
+    b, hq, hkv, d, k, L, seq = 2, 8, 2, 64, 32, 4, 300
+    g = hq // hkv
+    for dtype in (torch.float32, torch.bfloat16):
+        eng = lrqk.LightAttentionIndicesFactory(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=4,
+                                                device=torch.device(DEV), dtype=dtype)
+        eng.Kgpu = torch.randn((b, hq, k + L, d), generator=gen).to(DEV, dtype)
+        eng.Vgpu = torch.randn((b, hq, k + L, d), generator=gen).to(DEV, dtype)
+        src = torch.randn((b, hkv, seq, d), generator=gen).to(dtype).pin_memory()
+        hit = torch.stack([torch.stack([torch.randperm(seq, generator=gen)[:k] for _ in range(hq)]) for _ in range(b)])
+        want = torch.take_along_dim(src.unsqueeze(2).expand(b, hkv, g, seq, d), hit.view(b, hkv, g, k, 1), dim=3)
+        want = want.reshape(b, hq, k, d)
+        before = eng.Kgpu.clone()
+        out = eng.fetch_by_hit(eng.Kgpu_topk_area, src, hit.unsqueeze(-1).to(DEV))
+        assert out.shape == (b, hq, k, d) and torch.equal(eng.Kgpu[:, :, :k].cpu(), want)
+        assert torch.equal(eng.Kgpu[:, :, k:], before[:, :, k:])             # the ring is not touched
+        mask = torch.rand((b, hq, k), generator=gen) < 0.3
+        before = eng.Vgpu.clone()
+        eng.fetch_by_hit(eng.Vgpu_topk_area, src, hit.unsqueeze(-1).to(DEV), dst_mask=mask.to(DEV))
+        expect = torch.where(mask[..., None], want, before[:, :, :k].cpu())
+        assert torch.equal(eng.Vgpu[:, :, :k].cpu(), expect) and torch.equal(eng.Vgpu[:, :, k:], before[:, :, k:])
+        # fewer ids than slots: only the leading slots are written and returned
+        out = eng.fetch_by_hit(eng.Kgpu_topk_area, src, hit[:, :, :5].unsqueeze(-1).to(DEV))
+        assert out.shape == (b, hq, 5, d) and torch.equal(out.cpu(), want[:, :, :5])
+        with pytest.raises(ValueError):
+            eng.fetch_by_hit(eng.Kgpu_topk_area, src.clone(), hit.unsqueeze(-1).to(DEV))     # pageable memory
+
+
 def test_cache_front_door(lrqk, oracle):
     """DynamicLRQKCache: pending -> collecting -> decoding, error behaviour, sequence length."""
     _say("cache front door")
