@@ -17,6 +17,7 @@
 // last-arriving workgroup continues was measured slower: the device-scope fence it needs
 // costs ~15 us per workgroup because each XCD has its own L2.)
 #include <algorithm>
+#include <stdlib.h>
 
 #include "common.hpp"
 #include "ctx.hpp"
@@ -140,7 +141,8 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
                                                                 int d, int lpr_log2, float* __restrict__ part, int S,
                                                                 GramAppend ap, const T* __restrict__ b_q,
                                                                 const T* __restrict__ b_k, const T* __restrict__ k_new,
-                                                                int hq, int hkv, float* __restrict__ pre) {
+                                                                int hq, int hkv, float* __restrict__ pre,
+                                                                float* __restrict__ kq_out) {
   constexpr int VEC = Vec16<T>::N;
   extern __shared__ __align__(16) float gram_dyn[];  // used by the extra workgroup only
   __shared__ float w_all[kGramWaves][kGramChunk];
@@ -228,6 +230,8 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
       a0[g] = ok ? a0[g] : 0.0f;
     }
     __syncthreads();  // w_s of this chunk is complete (every wave runs the same number of chunks)
+    // K q of the wave's rows for the attention that ends the step (it then reads only V)
+    if (kq_out && lane < kGramChunk && c0 + lane < w1) kq_out[(int64_t)h * n + c0 + lane] = w_s[lane];
 #pragma unroll
     for (int g = 0; g < kGramChunk / 2; ++g) {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[g], a0[g], acc, 0, 0, 0);
@@ -257,6 +261,191 @@ __global__ __launch_bounds__(kGramThreads) void als_gram_kernel(const T* __restr
     float v = 0.0f;
 #pragma unroll
     for (int wv = 0; wv < kGramWaves; ++wv) v += red[wv][e];
+    pout[e] = v;
+  }
+}
+
+// The same pass for bf16 storage with d = 128 and r a multiple of 8, built for throughput when many heads are
+// stepped together: the active A_K rows come in as 16-byte pieces (two loads per lane and chunk instead of
+// sixteen 2-byte ones) and reach the operand layout of the bf16 matrix cores through a wave-private LDS tile
+// (bf16 x bf16 products are exact in fp32, so A^T A is the same sum as on the fp32 pipe, at a sixteenth of its
+// cost); a wave walks its rows chunk by chunk with the next chunk's K and A rows and the ids of the chunk after
+// it already requested, and no workgroup barrier inside the loop; all LDS is one static block shared by the
+// roles, so the launch is bounded by registers (4 workgroups per CU), not by the extra workgroups' B tile.
+typedef __bf16 gram_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 gram_bf16x2 __attribute__((ext_vector_type(2)));
+constexpr int kGramSmemFloats = 32 * (128 + 1) + 2 * 128;  // the extra workgroups' need at d = 128 (>= 4 * kGramNe)
+static_assert(kGramSmemFloats >= kGramWaves * kGramNe, "the cross-wave reduction fits the shared block");
+
+__device__ __forceinline__ void gram_wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ __launch_bounds__(kGramThreads, 4) void als_gram_bf16_kernel(
+    const bf16_t* __restrict__ a_k, int64_t head_stride, int64_t a_rows, const int32_t* __restrict__ active_idx,
+    int64_t idx_stride, bf16_t* k_prev, int kprev_slots, int n, const bf16_t* __restrict__ q, int r,
+    float* __restrict__ part, int S, GramAppend ap, const bf16_t* __restrict__ b_q, const bf16_t* __restrict__ b_k,
+    const bf16_t* __restrict__ k_new, int hq, int hkv, float* __restrict__ pre, float* __restrict__ kq_out) {
+  constexpr int d = 128, VEC = 8, lpr_log2 = 4, lpr = 16, gpw = kWave / lpr;  // 16 lanes per K row, 4 rows per load
+  constexpr int KL = kGramChunk / gpw;                                          // K loads per lane and chunk
+  __shared__ __align__(16) float gsm[kGramSmemFloats];
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int h = blockIdx.y, s = blockIdx.x;
+  if (s >= S) {
+    als_bgram_body<bf16_t>(b_q, b_k, q, k_new, h, hq, hkv, r, d, lpr_log2, pre + (int64_t)h * kPreNe, gsm, s - S);
+    return;
+  }
+  // wave-private: the chunk's A rows as bf16 [32][32] (64-byte rows), and its 32 products K q
+  uint16_t* At = reinterpret_cast<uint16_t*>(gsm) + wave * (kGramChunk * 32);
+  float* w_s = gsm + kGramWaves * (kGramChunk * 32 / 2) + wave * kGramChunk;
+
+  const int sub = lane & (lpr - 1), grp = lane >> lpr_log2;
+  const int arow = lane >> 2, aq = lane & 3;  // A loads: tokens arow and arow + 16 of the chunk, piece aq of the row
+  const int lpa = r >> 3;
+  const int aqc = min(aq, lpa - 1);
+  const int rows_per_split = (n + S - 1) / S;
+  const int s0 = s * rows_per_split;
+  const int s1 = min(n, s0 + rows_per_split);
+  const int rows_per_wave = (rows_per_split + kGramWaves - 1) / kGramWaves;
+  const int w0 = s0 + wave * rows_per_wave;
+  const int w1 = min(s1, w0 + rows_per_wave);
+  const int n_chunks = (rows_per_wave + kGramChunk - 1) / kGramChunk;
+  const bf16_t* A = a_k + (int64_t)h * head_stride;
+  const bf16_t* Kp = k_prev + (int64_t)h * kprev_slots * d;
+  const int col = lane & 31, khalf = lane >> 5;
+  const bf16_t* knew_h = Kp;
+  if (ap.slot >= 0) {
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    knew_h = (const bf16_t*)ap.k_new + ((int64_t)bb * ap.hkv + kvh) * d;
+  }
+  uint32_t qw[4];  // this lane's eight elements of q, as stored
+  {
+    Vec16<bf16_t> qv;
+    qv.load(q + (int64_t)h * d + sub * VEC);
+    qw[0] = qv.raw.x;
+    qw[1] = qv.raw.y;
+    qw[2] = qv.raw.z;
+    qw[3] = qv.raw.w;
+  }
+  // every load is unconditional: indices are clamped into range and the results masked afterwards
+  auto load_ids = [&](int c0, int32_t (&tok)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = min(c0 + arow + 16 * j, n - 1);
+      const int32_t id = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      tok[j] = t == ap.slot ? ap.token : id;
+    }
+  };
+  auto load_a = [&](const int32_t (&tok)[2], uint4 (&av)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t sr = min(max((int64_t)tok[j], (int64_t)0), a_rows - 1);
+      av[j] = *reinterpret_cast<const uint4*>(A + sr * r + aqc * 8);
+    }
+  };
+  auto load_k = [&](int c0, Vec16<bf16_t> (&kv)[KL]) {
+#pragma unroll
+    for (int u = 0; u < KL; ++u) {
+      const int row = min(c0 + u * gpw + grp, n - 1);
+      kv[u].load((row == ap.slot ? knew_h : Kp + (int64_t)row * d) + sub * VEC);
+    }
+  };
+
+  v16f acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  float racc = 0.0f;
+  int32_t tok_cur[2], tok_nxt[2];
+  uint4 a_cur[2];
+  Vec16<bf16_t> kv[KL];
+  load_ids(w0, tok_cur);
+  load_k(w0, kv);
+  load_ids(w0 + kGramChunk, tok_nxt);
+  load_a(tok_cur, a_cur);
+
+  for (int ch = 0; ch < n_chunks; ++ch) {
+    const int c0 = w0 + ch * kGramChunk;
+    // K q of the chunk's rows: products of bf16 pairs summed in fp32 (q stays in its storage form)
+#pragma unroll
+    for (int u = 0; u < KL; ++u) {
+      const int row = u * gpw + grp;
+      const uint32_t kw[4] = {kv[u].raw.x, kv[u].raw.y, kv[u].raw.z, kv[u].raw.w};
+      float wv = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        wv = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(gram_bf16x2, kw[e]), __builtin_bit_cast(gram_bf16x2, qw[e]),
+                                             wv, false);
+      wv = group_sum(wv, lpr);
+      if (sub == 0) w_s[row] = (c0 + row < w1) ? wv : 0.0f;
+    }
+    // the next chunk's rows and the ids of the one after it (wave-uniform conditions)
+    uint4 a_nxt[2] = {a_cur[0], a_cur[1]};
+    int32_t tok_nn[2] = {0, 0};
+    if (ch + 1 < n_chunks) {
+      load_k(c0 + kGramChunk, kv);
+      load_a(tok_nxt, a_nxt);
+    }
+    if (ch + 2 < n_chunks) load_ids(c0 + 2 * kGramChunk, tok_nn);
+    // this chunk's A rows into the tile (rows that do not count, and columns >= r, as zeros)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bool ok = (c0 + arow + 16 * j < w1) && tok_cur[j] >= 0 && (int64_t)tok_cur[j] < a_rows && aq < lpa;
+      const uint4 v = ok ? a_cur[j] : make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4*>(At + (arow + 16 * j) * 32 + aq * 8) = v;
+    }
+    gram_wave_sync();
+    if (kq_out && lane < kGramChunk && c0 + lane < w1) kq_out[(int64_t)h * n + c0 + lane] = w_s[lane];
+    // lane (col, khalf) takes tokens 16 mm + 8 khalf .. + 7 of its column: the k elements of one bf16 MFMA (both
+    // operands are the same registers, so their order is immaterial)
+#pragma unroll
+    for (int mm = 0; mm < kGramChunk / 16; ++mm) {
+      const int t0 = 16 * mm + 8 * khalf;
+      uint32_t e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = At[(t0 + j) * 32 + col];
+      const float4 wa = *reinterpret_cast<const float4*>(w_s + t0);
+      const float4 wb = *reinterpret_cast<const float4*>(w_s + t0 + 4);
+      const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) racc = fmaf(wv[j], __uint_as_float(e[j] << 16), racc);
+      const gram_bf16x8 op = __builtin_bit_cast(
+          gram_bf16x8, make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)));
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(op, op, acc, 0, 0, 0);
+    }
+    gram_wave_sync();  // the tile and w_s are rewritten by the next chunk
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      a_cur[j] = a_nxt[j];
+      tok_cur[j] = tok_nxt[j];
+      tok_nxt[j] = tok_nn[j];
+    }
+  }
+  racc += __shfl_xor(racc, 32, kWave);
+  if (ap.slot >= w0 && ap.slot < w1 && lane < lpr) {  // this wave owns the new token's slot
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    const int64_t so = ((int64_t)bb * ap.hkv + kvh) * d + lane * VEC;
+    const int64_t dof = ((int64_t)h * kprev_slots + ap.slot) * d + lane * VEC;
+    Vec16<bf16_t> kx, vx;
+    kx.load((const bf16_t*)ap.k_new + so);
+    vx.load((const bf16_t*)ap.v_new + so);
+    *reinterpret_cast<decltype(kx.raw)*>(k_prev + dof) = kx.raw;
+    *reinterpret_cast<decltype(vx.raw)*>((bf16_t*)ap.v_act + dof) = vx.raw;
+    if (lane == 0) ap.idx_out[(int64_t)h * idx_stride + ap.slot] = ap.token;
+  }
+  // ---- cross-wave reduction through the same block of LDS
+  __syncthreads();
+  float* red = gsm;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[wave * kGramNe + mfma_row(lane, v) * 32 + col] = acc[v];
+  if (lane < 32) red[wave * kGramNe + 32 * 32 + col] = racc;
+  __syncthreads();
+  float* pout = part + ((int64_t)h * S + s) * kGramNe;
+  for (int e = tid; e < kGramNe; e += kGramThreads) {
+    float v = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kGramWaves; ++wv) v += red[wv * kGramNe + e];
     pout[e] = v;
   }
 }
@@ -415,6 +604,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                            float tol, void* q_hat, void* k_hat, int64_t append_row, GramAppend ap, bool defer_finish,
                            hipStream_t st) {
   constexpr int VEC = Vec16<T>::N;
+  ctx->kq_valid = false;
   const int bh = b * hq;
   const int lpr = d / VEC;
   int lpr_log2 = 0;
@@ -427,6 +617,12 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   int S = (n + kGramWaves * kGramChunk - 1) / (kGramWaves * kGramChunk);
   if (S < 1) S = 1;
   if (S > 32) S = 32;
+  // bf16, d = 128, r in {8, 16, 24, 32}, 16-byte aligned rows: the pipelined pass on the bf16 matrix cores
+  const bool fast_bf16 = sizeof(T) == 2 && d == 128 && r % 8 == 0 && ((uintptr_t)a_k % 16 == 0) &&
+                         (head_stride * sizeof(T)) % 16 == 0 && !getenv("LRQK_GRAM_OLD");
+  // (the pipelined pass: two chunks per wave measured best at 1, 4 and 8 sequences of the Llama-3-8B shape)
+  if (fast_bf16) S = std::min(32, std::max(1, (n + 2 * kGramWaves * kGramChunk - 1) / (2 * kGramWaves * kGramChunk)));
+  if (const char* e = getenv("LRQK_GRAM_S")) S = atoi(e);
   int rc = ctx->als_part.ensure((size_t)bh * S * kGramNe * sizeof(float));
   if (rc) return rc;
   if ((rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float)))) return rc;
@@ -448,10 +644,32 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   }
   if ((rc = ctx->als_pre.ensure((size_t)bh * kPreNe * sizeof(float)))) return rc;
   float* pre = (float*)ctx->als_pre.p;
-  hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S + 2, (unsigned)bh), dim3(kGramThreads), smem_gram, st,
-                     (const T*)a_k, head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n, (const T*)q,
-                     r, d, lpr_log2, part, S, ap, (const T*)b_q, (const T*)b_k, (const T*)k_new, hq, hkv, pre);
+  // With the ring append folded in, the pass sees every slot as the attention of this step will (except the
+  // slots that the misses replace): it leaves K q per slot for that attention.
+  float* kq_out = nullptr;
+  if (defer_finish && ap.slot >= 0 && n == kprev_slots) {
+    if ((rc = ctx->als_kq.ensure((size_t)bh * n * sizeof(float)))) return rc;
+    kq_out = (float*)ctx->als_kq.p;
+  }
+  if (fast_bf16) {
+    hipLaunchKernelGGL(als_gram_bf16_kernel, dim3((unsigned)S + 2, (unsigned)bh), dim3(kGramThreads), 0, st,
+                       (const bf16_t*)a_k, head_stride, a_rows, active_idx, idx_stride, (bf16_t*)k_prev, kprev_slots, n,
+                       (const bf16_t*)q, r, part, S, ap, (const bf16_t*)b_q, (const bf16_t*)b_k, (const bf16_t*)k_new,
+                       hq, hkv, pre, kq_out);
+  } else {
+    hipLaunchKernelGGL((als_gram_kernel<T>), dim3((unsigned)S + 2, (unsigned)bh), dim3(kGramThreads), smem_gram, st,
+                       (const T*)a_k, head_stride, a_rows, active_idx, idx_stride, (T*)k_prev, kprev_slots, n,
+                       (const T*)q, r, d, lpr_log2, part, S, ap, (const T*)b_q, (const T*)b_k, (const T*)k_new, hq, hkv,
+                       pre, kq_out);
+  }
   LRQK_HIP_CHECK(hipGetLastError());
+  if (kq_out) {
+    ctx->kq_valid = true;
+    ctx->kq_k_act = k_prev;
+    ctx->kq_q = q;
+    ctx->kq_bh = bh;
+    ctx->kq_n = n;
+  }
 #define LRQK_SOLVE_CASE(KS)                                                                                     \
   hipLaunchKernelGGL((als_solve_kernel<KS>), dim3((unsigned)bh), dim3(kSolveThreads), smem_solve, st, (const float*)pre, \
                      (const float*)part, S, r, max_iter, iter_out, deltas)

@@ -9,6 +9,7 @@
 // the others meanwhile run the attention over the slots that stay resident; the combine
 // kernel then adds the freshly fetched slots of its head before merging.
 #include <math.h>
+#include <stdlib.h>
 
 #include <mutex>
 
@@ -87,6 +88,48 @@ __device__ __forceinline__ void attn_scan(const float* qf, const T* __restrict__
   }
 }
 
+// The same pass when the products K q of the rows are already known (`w`, one float per slot, unscaled):
+// only the V rows are read.
+template <typename T, int NW, int U, typename RowOf>
+__device__ __forceinline__ void attn_scan_w(const float* __restrict__ w, float scale_log2e, const T* __restrict__ Vh,
+                                            int d, int lpr_log2, int begin, int end, RowOf row_of,
+                                            AttnAcc<Vec16<T>::N>& st) {
+  constexpr int VEC = Vec16<T>::N;
+  const int lane = lane_id(), wave = wave_id();
+  const int lpr = 1 << lpr_log2;
+  const int sub = lane & (lpr - 1);
+  const int grp = lane >> lpr_log2;
+  const int gpw = kWave >> lpr_log2;
+  const int rows_per_iter = gpw * NW;
+  for (int base = begin; base < end; base += U * rows_per_iter) {
+    Vec16<T> vv[U];
+    float wl[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = base + u * rows_per_iter + wave * gpw + grp;
+      bool valid;
+      const int rr = row_of(min(i, end - 1), valid);
+      ok[u] = valid && i < end;
+      wl[u] = w[rr];
+      vv[u].load(Vh + (int64_t)rr * d + sub * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float vf[VEC];
+      vv[u].unpack(vf);
+      const float sc = ok[u] ? wl[u] * scale_log2e : -INFINITY;
+      const float m_new = fmaxf(st.m, sc);
+      const float alpha = (m_new == -INFINITY) ? 0.0f : exp2f(st.m - m_new);
+      const float p = (m_new == -INFINITY) ? 0.0f : exp2f(sc - m_new);
+      st.l = st.l * alpha + p;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) st.acc[e] = st.acc[e] * alpha + p * vf[e];
+      st.m = m_new;
+    }
+  }
+}
+
 // Merges the lane groups of a wave, then the waves of the workgroup; afterwards threads c < d + 2
 // hold element c of the workgroup's (m, l, acc[d]) triple in the return value.
 // red: [NW][2 + 256] floats of LDS.
@@ -154,7 +197,7 @@ __device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const
                                                   const T* __restrict__ V, int n_slots, int n_valid, int d,
                                                   int lpr_log2, float scale_log2e, float* __restrict__ part, int S,
                                                   int stride_s, const uint8_t* __restrict__ skip, int k_skip, int h,
-                                                  int s) {
+                                                  int s, const float* __restrict__ w = nullptr) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float red[kAttnWaves][2 + 256];
   const int rows_per_split = (n_valid + S - 1) / S;
@@ -166,7 +209,15 @@ __device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const
   const T* Vh = V + (int64_t)h * n_slots * d;
   AttnAcc<VEC> st;
   st.init();
-  if (skip) {
+  if (skip && w) {
+    // (decode step) the factor update's first kernel left K q of every slot, as the slots were before this
+    // step's misses; the slots that are being replaced are skipped here anyway
+    const uint8_t* sk = skip + (int64_t)h * k_skip;
+    attn_scan_w<T, kAttnWaves, U>(w + (int64_t)h * n_slots, scale_log2e, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
+      valid = sk[min(i, k_skip - 1)] == 0 || i >= k_skip;
+      return i;
+    }, st);
+  } else if (skip) {
     const uint8_t* sk = skip + (int64_t)h * k_skip;
     attn_scan<T, kAttnWaves, U>(qf, Kh, Vh, d, lpr_log2, r0, r1, [&](int i, bool& valid) {
       valid = sk[min(i, k_skip - 1)] == 0 || i >= k_skip;
@@ -397,7 +448,8 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
     const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
     int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
     int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
-    FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic, const int32_t* __restrict__ miss_new) {
+    FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic, const int32_t* __restrict__ miss_new,
+    const float* __restrict__ kq) {
   const int h = blockIdx.y;
   if (with_finish && (int)blockIdx.x >= n_fetch + S) {
     if ((int)blockIdx.x == n_fetch + S)
@@ -414,7 +466,7 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
   }
   // (eight row groups in flight per wave: the launch has few attention workgroups)
   attn_partial_body<T, 8>(q, K, V, n_slots, n_slots, d, lpr_log2, scale_log2e, part, S, S + n_fetch, evict, k, h,
-                          (int)blockIdx.x - n_fetch);
+                          (int)blockIdx.x - n_fetch, kq);
 }
 
 // One workgroup per head merges its S partial (max, sum, acc) triples (S <= kCombMaxS).
@@ -601,7 +653,9 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   if ((int64_t)(S + want_fetch + 2) * bh > slots) S = (n_slots + 255) / 256;
   if (S > 64) S = 64;
   const int room = slots / bh - S - 2;
-  const int n_fetch = std::min(want_fetch, std::max(room, 8));
+  int n_fetch = std::min(want_fetch, std::max(room, 8));
+  if (const char* e = getenv("LRQK_FA_S")) S = atoi(e);
+  if (const char* e = getenv("LRQK_FA_NF")) n_fetch = atoi(e);
   if ((rc = ctx->attn_part.ensure((size_t)bh * (S + n_fetch) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   static_assert(kAttnThreads == kFinThreads, "the finish stage rides in an attention-sized workgroup");
@@ -615,10 +669,15 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
     }
   }
   const int index_role = with_finish && ctx->fin.qa != nullptr && ctx->fin.append_row >= 0 ? 1 : 0;
+  // K q of every slot, left by this step's Gram pass over the same buffers and query (else the role reads K)
+  const float* kq = nullptr;
+  if (ctx->kq_valid && ctx->kq_k_act == k_act && ctx->kq_q == q && ctx->kq_bh == bh && ctx->kq_n == n_slots)
+    kq = (const float*)ctx->als_kq.p;
+  ctx->kq_valid = false;
   hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish + index_role), (unsigned)bh),
                      dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
-                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new);
+                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new, kq);
   LRQK_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
                      (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);

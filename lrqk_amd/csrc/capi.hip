@@ -48,6 +48,7 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->attn_part.release();
   ctx->als_part.release();
   ctx->als_pre.release();
+  ctx->als_kq.release();
   ctx->als_iter.release();
   ctx->prefill_ws.release();
   ctx->new_idx.release();
@@ -78,6 +79,7 @@ extern "C" int lrqk_ctx_reserve(lrqk_ctx* ctx, int bh, int64_t max_tokens, int t
   if ((rc = ctx->keys.ensure((size_t)bh * key_stride * 4))) return rc;
   if ((rc = ctx->attn_part.ensure((size_t)bh * 64 * (d + 2) * sizeof(float)))) return rc;
   if ((rc = ctx->als_part.ensure((size_t)bh * 32 * (32 * 32 + 32) * sizeof(float)))) return rc;
+  if ((rc = ctx->als_kq.ensure((size_t)bh * n_active * sizeof(float)))) return rc;
   if ((rc = ctx->als_iter.ensure((size_t)bh * LRQK_MAX_DECODE_ITERS * (2 * r + 1) * sizeof(float)))) return rc;
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
   if ((rc = ctx->misc.ensure((size_t)bh * (topk * 5 + 16)))) return rc;

@@ -50,6 +50,11 @@ struct lrqk_ctx {
   lrqk::DevBuf cand_cnt;    // per-chunk counts / thresholds
   lrqk::DevBuf attn_part;   // f32 [bh][S][d+2]
   lrqk::DevBuf als_part;    // f32 [bh][S][32*32 + 32]
+  lrqk::DevBuf als_kq;      // f32 [bh][n]: K q of every active slot, left by the step's Gram pass for its attention
+  bool kq_valid = false;    //   set by that pass, consumed by the fetch + attention launch of the same step
+  const void* kq_k_act = nullptr;
+  const void* kq_q = nullptr;
+  int kq_bh = 0, kq_n = 0;
   lrqk::DevBuf als_pre;     // f32 [bh][4*1024 + 65]: what the solve needs from B_Q, B_K, q, k (formed beside the Gram pass)
   lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators

@@ -20,7 +20,7 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   const int bh = b * hq;
   const int n = topk + lite;
   int rc;
-  ctx->fin_pending = ctx->qhat_pending = false;  // nothing survives a call that failed half-way
+  ctx->fin_pending = ctx->qhat_pending = ctx->kq_valid = false;  // nothing survives a call that failed half-way
   ctx->sidx_rows_hint = token;                   // rows [0, token) of A_K exist before this step
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
   // misc: miss_slots i32 [bh][topk] | miss_count i32 [bh] | miss_old i32 [bh][topk] | miss_new i32 [bh][topk] |
