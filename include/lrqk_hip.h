@@ -94,7 +94,9 @@ int lrqk_diff(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t 
 /* py:1235-1273 + py:1275-1315 in one pass -- lrqk_score_select followed by lrqk_diff, with the
  * diff done by the select kernel while the selection is still on chip (m > topk required).
  * new_idx: [bh][topk] receives the ascending selection; hit / evict / miss_slots / miss_count
- * as in lrqk_diff (evict may be NULL). */
+ * as in lrqk_diff (evict may be NULL).  new_idx may be NULL: the caller then only gets what
+ * changes (hit, evict, miss_slots, miss_count), and the selection is never put in order -- the
+ * form lrqk_decode_step uses. */
 int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh,
                            int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit,
                            int64_t hit_stride, uint8_t* evict, int32_t* miss_slots, int32_t* miss_count,

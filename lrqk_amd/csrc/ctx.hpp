@@ -104,7 +104,8 @@ namespace lrqk {
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
-                      int32_t* miss_old = nullptr, const VictimView* vic = nullptr, int32_t* miss_new = nullptr);
+                      int32_t* miss_old = nullptr, const VictimView* vic = nullptr, int32_t* miss_new = nullptr,
+                      bool want_new_idx = true);
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
 // into its first kernel.
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,

@@ -159,6 +159,7 @@ struct SelState {
   uint32_t* t_used;
   float* q_cur;
   int* cand_count;
+  int* level;        // slack of the carried bound per head (see bound_rank): level | calm calls << 8
   int* stats;
   int* rescored;     // per workgroup of the last index scan: rows whose bound passed (rescored exactly)
   int rescored_cap;
@@ -172,6 +173,7 @@ __global__ void init_select_state_kernel(SelState st, int bh) {
     st.t_used[i] = 0xffffffffu;
     st.q_cur[i] = 0.0f;
     st.cand_count[i] = 0;
+    st.level[i] = 0;
   }
   if (i < 3) st.stats[i] = 0;
 }
@@ -675,12 +677,6 @@ __device__ __forceinline__ void find_digits(const uint32_t* hist_a, const uint32
   rem_b = s_res[3];
 }
 
-#ifdef LRQK_SEL_STAMPS
-#define SEL_STAMP(i) do { if (threadIdx.x == 0) s_stamp[i] = wall_clock64(); } while (0)
-#else
-#define SEL_STAMP(i) do { } while (0)
-#endif
-
 struct DiffArgs {
   int32_t* hit;        // [bh][hit_stride] resident token ids, nullptr = no diff
   int64_t hit_stride;
@@ -698,27 +694,41 @@ struct DiffArgs {
 // mode: 0 = use the candidate list if valid, else compute the head's keys from A_K;
 //       1 = keys[] already holds the head's keys (caller-provided scores).
 // Dynamic LDS: gt | eq bitmaps (2 * kChunkWords words), then, with a diff, 10*k bytes.
+// LDS blocks of the selector (declared by the kernels, so that the two bodies below share them)
+struct SelLds {
+  uint32_t* dyn;     // dynamic LDS
+  uint32_t* hist;    // [kBins]
+  uint32_t* hist_b;  // [kBins], directly behind hist
+  int* scratch;      // [2 * kSelWaves]
+  uint32_t* wred;    // [2 * kSelWaves]
+  int* s_res;        // [8]
+  int* s_n;          // [1]
+};
+#define LRQK_SEL_LDS(L)                                           \
+  extern __shared__ __align__(16) uint32_t dyn_lds[];             \
+  __shared__ __align__(16) uint32_t hist2_lds[2 * kBins];         \
+  __shared__ int scratch_lds[2 * kSelWaves];                      \
+  __shared__ uint32_t wred_lds[2 * kSelWaves];                    \
+  __shared__ int s_res_lds[8];                                    \
+  __shared__ int s_n_lds;                                         \
+  SelLds L{dyn_lds, hist2_lds, hist2_lds + kBins, scratch_lds, wred_lds, s_res_lds, &s_n_lds};
+
+// n_list: the length of the head's candidate list if the caller has read it already (and every thread of the
+// workgroup with it), else -1.
 template <typename T, int R>
-__global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uint2* __restrict__ cand_all, int cand_cap,
-                                                             SelState st, uint32_t* __restrict__ keys_all,
-                                                             int64_t key_stride,
-                                                             const T* __restrict__ a_k, int64_t head_stride,
-                                                             const T* __restrict__ q_hat, int64_t m, int r, int round_bf16,
-                                                             int k, int32_t* __restrict__ out_all, int64_t out_stride,
-                                                             DiffArgs df) {
-  extern __shared__ __align__(16) uint32_t dyn[];
-  __shared__ uint32_t hist[kBins];
-  __shared__ uint32_t hist_b[kBins];
-  __shared__ int scratch[2 * kSelWaves];
-  __shared__ uint32_t wred[2 * kSelWaves];
-  __shared__ int s_res[4];
-  __shared__ int s_n;
-#ifdef LRQK_SEL_STAMPS
-  __shared__ uint64_t s_stamp[16];
-  if (threadIdx.x < 16) s_stamp[threadIdx.x] = 0;
-  __syncthreads();
-#endif
-  SEL_STAMP(0);
+__device__ __forceinline__ void select_generic(const SelLds& L, int mode, const uint2* __restrict__ cand_all, int cand_cap,
+                                               SelState st, uint32_t* __restrict__ keys_all, int64_t key_stride,
+                                               const T* __restrict__ a_k, int64_t head_stride,
+                                               const T* __restrict__ q_hat, int64_t m, int r, int round_bf16, int k,
+                                               int32_t* __restrict__ out_all, int64_t out_stride, DiffArgs df,
+                                               int n_list, int bound_rank_k = 0) {
+  uint32_t* const dyn = L.dyn;
+  uint32_t* const hist = L.hist;
+  uint32_t* const hist_b = L.hist_b;
+  int* const scratch = L.scratch;
+  uint32_t* const wred = L.wred;
+  int* const s_res = L.s_res;
+  int& s_n = *L.s_n;
   uint32_t* gt = dyn;
   uint32_t* eq = dyn + kChunkWords;
   const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
@@ -741,13 +751,10 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   int64_t N = m;
   uint32_t lo = 0;
   if (mode == 0) {
-    if (tid == 0) {
-      s_n = st.cand_count[h];
-      st.cand_count[h] = 0;  // re-arm for the next call
-    }
+    if (tid == 0 && n_list < 0) s_n = st.cand_count[h];
     __syncthreads();
-    SEL_STAMP(1);
-    const int n = s_n;
+    if (tid == 0) st.cand_count[h] = 0;  // re-arm for the next call (every thread has read the count by now)
+    const int n = n_list < 0 ? s_n : n_list;
     fast = n >= k && n <= cand_cap;
     if (fast) {
       N = n;
@@ -830,7 +837,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   }
   if (tid == 0) s_res[0] = s_res[1] = s_res[2] = s_res[3] = 0;
   __syncthreads();
-  SEL_STAMP(2);
   vmax = 0u;
   vor = 0u;
 #pragma unroll
@@ -843,14 +849,13 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
   const int nbits = range ? (32 - __clz((int)(range >> tz))) : 0;  // significant bits of (key - lo) >> tz
   const int s1 = max(nbits - 12, 0), s2 = max(s1 - 12, 0);
 
-  const int k2 = (int)min(((int64_t)kBoundRankNum * k) / kBoundRankDen, N);  // rank that defines the next t_low
+  // rank that defines the next t_low
+  const int k2 = (int)min(bound_rank_k > 0 ? (int64_t)bound_rank_k : ((int64_t)kBoundRankNum * k) / kBoundRankDen, N);
   // ---- pass 1 (both ranks share it)
   for_each([&](uint32_t key, int64_t) { atomicAdd(&hist[((key - lo) >> tz) >> s1], 1u); });
   __syncthreads();
-  SEL_STAMP(3);
   int D1, need1, E1, needE;
   find_digits(hist, hist, k, k2, scratch, s_res, D1, need1, E1, needE);
-  SEL_STAMP(4);
   uint32_t offT = (uint32_t)D1 << s1, offE = (uint32_t)E1 << s1;
   int need_eq = need1;
   if (s1 > 0) {
@@ -890,7 +895,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       need_eq = need3;
     }
   }
-  SEL_STAMP(5);
   const uint32_t Tk = lo + (offT << tz);
   if (tid == 0) {
     st.t_low[h] = lo + (offE << tz);  // rank >= 1.5k (rounded down to the resolved bits)
@@ -916,13 +920,11 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       }
     }
     __syncthreads();
-    SEL_STAMP(6);
     for_each([&](uint32_t key, int64_t idx) {
       const int64_t rel = idx - c0;
       if (key >= Tk && rel >= 0 && rel < span) atomicOr(key > Tk ? &gt[rel >> 5] : &eq[rel >> 5], 1u << (rel & 31));
     });
     __syncthreads();
-    SEL_STAMP(7);
     const int w0 = tid * W;
     uint32_t gwr[kWordsPT], ewr[kWordsPT];
 #pragma unroll
@@ -943,7 +945,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
     int g_incl = cg, e_incl = ce, g_tot, e_tot;
     block_inclusive_sum2(g_incl, e_incl, scratch, g_tot, e_tot);
-    SEL_STAMP(8);
     int e_run = eq_seen + e_incl - ce;  // equal keys before this thread's words (all chunks)
     int pos = out_pos + (g_incl - cg) + (min(e_run, need_eq) - min(eq_seen, need_eq));
 #pragma unroll
@@ -972,7 +973,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     out_pos += g_tot + (min(eq_seen + e_tot, need_eq) - min(eq_seen, need_eq));
     eq_seen += e_tot;
     __syncthreads();
-    SEL_STAMP(9);
   }
   if (!do_diff) return;
 
@@ -998,7 +998,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     const int words = (int)((m + 31) >> 5);
     for (int i = tid; i < words; i += kSelThreads) eq[i] = 0;
     __syncthreads();
-    SEL_STAMP(10);
 #pragma unroll
     for (int u = 0; u < kDiffIpt; ++u) {
       const int s = tid * ipt + u;
@@ -1011,7 +1010,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
       }
     }
     __syncthreads();
-    SEL_STAMP(11);
     for (int i = tid; i < k; i += kSelThreads) {
       const int32_t t = new_s[i];
       matched[i] = (uint8_t)((eq[t >> 5] >> (t & 31)) & 1u);
@@ -1055,7 +1053,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
   }
   __syncthreads();
-  SEL_STAMP(12);
   // both ordered compactions in one sweep: rank of missing tokens and of evicted slots
   int n_missing, n_evict;
   {
@@ -1080,7 +1077,6 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     }
   }
   __syncthreads();
-  SEL_STAMP(13);
   const int n_pair = min(n_missing, n_evict);
   const int32_t* ev_list = reinterpret_cast<const int32_t*>(gt);
   for (int j = tid; j < n_pair; j += kSelThreads) {
@@ -1099,14 +1095,390 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uin
     for (int s = tid; s < k; s += kSelThreads) df.evict[(int64_t)h * k + s] = evict_s[s];
   }
   if (tid == 0 && df.miss_count) df.miss_count[h] = n_pair;
-#ifdef LRQK_SEL_STAMPS
-  __syncthreads();
-  SEL_STAMP(14);
-  if (tid == 0 && df.evict && k >= 128) {
-    uint32_t* o = reinterpret_cast<uint32_t*>(df.evict + (int64_t)h * k + k - 64);
-    for (int i = 0; i < 16; ++i) o[i] = s_stamp[i] ? (uint32_t)(s_stamp[i] - s_stamp[0]) : 0u;
+}
+
+template <typename T, int R>
+__global__ __launch_bounds__(kSelThreads) void select_kernel(int mode, const uint2* __restrict__ cand_all, int cand_cap,
+                                                             SelState st, uint32_t* __restrict__ keys_all,
+                                                             int64_t key_stride, const T* __restrict__ a_k,
+                                                             int64_t head_stride, const T* __restrict__ q_hat, int64_t m,
+                                                             int r, int round_bf16, int k, int32_t* __restrict__ out_all,
+                                                             int64_t out_stride, DiffArgs df) {
+  LRQK_SEL_LDS(L);
+  select_generic<T, R>(L, mode, cand_all, cand_cap, st, keys_all, key_stride, a_k, head_stride, q_hat, m, r, round_bf16, k,
+                       out_all, out_stride, df, -1);
+}
+
+// --------------------------------------------------------------------------- select + diff of the decode step
+// The decode step does not need the ascending list of the selected tokens, only what changes: which slots lose
+// their token and which tokens come in (row-major pairing: the j-th freed slot takes the j-th smallest new
+// token).  With a usable candidate list (k <= n <= 16384 entries, all token ids below 262144) that is done
+// without ever ordering the selection: the candidates stay in registers; three bitmaps over the token ids
+// (selected, tied at the threshold, resident) turn every membership question into one bit test; the only
+// ordered quantities are the ranks of the tied candidates (to take the lowest ids among them) and of the
+// incoming tokens, both a prefix count over bitmap words; workgroup scans take one barrier (wave scans by lane
+// moves, the wave totals rescanned by every wave).  Anything else (no list, overflow, longer contexts) goes
+// through select_generic in the same launch.
+
+// Exclusive scan of two counters in thread order; one barrier.  slot: 2 * kSelWaves ints; consecutive calls must
+// be separated by a barrier.
+__device__ __forceinline__ void step_scan2(int a, int b, int* slot, int& ex_a, int& ex_b, int& tot_a, int& tot_b) {
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+  const int ia = wave_inclusive_sum(a), ib = wave_inclusive_sum(b);
+  if (lane == kWave - 1) {
+    slot[wave] = ia;
+    slot[kSelWaves + wave] = ib;
   }
-#endif
+  __syncthreads();
+  const int ta = lane < kSelWaves ? slot[lane] : 0;
+  const int tb = lane < kSelWaves ? slot[kSelWaves + lane] : 0;
+  const int sa = wave_inclusive_sum(ta), sb = wave_inclusive_sum(tb);
+  const int base_a = wave ? __builtin_amdgcn_readlane(sa, wave - 1) : 0;
+  const int base_b = wave ? __builtin_amdgcn_readlane(sb, wave - 1) : 0;
+  tot_a = __builtin_amdgcn_readlane(sa, kSelWaves - 1);
+  tot_b = __builtin_amdgcn_readlane(sb, kSelWaves - 1);
+  ex_a = base_a + ia - a;
+  ex_b = base_b + ib - b;
+}
+
+// Like find_digits, with the one-barrier scan; cnt_a: number of elements in the digit found for need_a.
+// s_res: 5 ints.  Two barriers.
+__device__ __forceinline__ void step_find_digits(const uint32_t* hist_a, const uint32_t* hist_b, int need_a, int need_b,
+                                                 int* slot, int* s_res, int& dig_a, int& rem_a, int& dig_b, int& rem_b,
+                                                 int& cnt_a) {
+  const int tid = threadIdx.x;
+  int ca[kBinsPT], cb[kBinsPT], la = 0, lb = 0;
+#pragma unroll
+  for (int x = 0; x < kBinsPT; ++x) {
+    ca[x] = (int)hist_a[tid * kBinsPT + x];
+    cb[x] = (int)hist_b[tid * kBinsPT + x];
+    la += ca[x];
+    lb += cb[x];
+  }
+  int ea, eb, ta, tb;
+  step_scan2(la, lb, slot, ea, eb, ta, tb);
+  const int above_a = ta - ea - la, above_b = tb - eb - lb;  // elements in bins above this thread's bins
+  if (above_a < need_a && need_a <= above_a + la) {
+    int c = above_a;
+#pragma unroll
+    for (int x = kBinsPT - 1; x >= 0; --x) {
+      if (c < need_a && c + ca[x] >= need_a) {
+        s_res[0] = tid * kBinsPT + x;
+        s_res[1] = need_a - c;
+        s_res[4] = ca[x];
+      }
+      c += ca[x];
+    }
+  }
+  if (above_b < need_b && need_b <= above_b + lb) {
+    int c = above_b;
+#pragma unroll
+    for (int x = kBinsPT - 1; x >= 0; --x) {
+      if (c < need_b && c + cb[x] >= need_b) {
+        s_res[2] = tid * kBinsPT + x;
+        s_res[3] = need_b - c;
+      }
+      c += cb[x];
+    }
+  }
+  __syncthreads();
+  dig_a = s_res[0];
+  rem_a = s_res[1];
+  dig_b = s_res[2];
+  rem_b = s_res[3];
+  cnt_a = s_res[4];
+}
+
+// Dynamic LDS of the step's select: three bitmaps of `words4` words, word prefixes (u16), incoming tokens,
+// outgoing tokens (i32 [k] each), freed slots (u16 [k]).
+static inline size_t step_select_words4(int64_t m) { return (size_t)(((m + 31) >> 5) + 3) & ~(size_t)3; }
+static inline size_t step_select_smem(int64_t m, int k) {
+  return step_select_words4(m) * (3 * 4 + 2) + (size_t)k * (4 + 4 + 2) + 16;
+}
+
+template <int CPT>
+__device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* __restrict__ cand, int N, uint32_t lo,
+                                                 SelState st, int h, int64_t m, int k, int k2, const DiffArgs& df) {
+  const int tid = threadIdx.x;
+  const int words = (int)((m + 31) >> 5);
+  const int words4 = (words + 3) & ~3;
+  uint32_t* bmS = L.dyn;              // selected tokens
+  uint32_t* bmE = bmS + words4;       // candidates tied at the threshold
+  uint32_t* bmH = bmE + words4;       // resident tokens
+  uint16_t* wpre = reinterpret_cast<uint16_t*>(bmH + words4);  // [words4] marked tokens in the words before
+  int32_t* miss_s = reinterpret_cast<int32_t*>(wpre + words4);  // [k] incoming tokens, ascending
+  int32_t* ev_old = miss_s + k;                                 // [k] tokens of the freed slots
+  uint16_t* ev_slot = reinterpret_cast<uint16_t*>(ev_old + k);  // [k] freed slots, ascending
+  uint32_t* hist = L.hist;
+  uint32_t* hist_b = L.hist_b;
+  uint32_t* bmM = L.hist;             // incoming tokens (takes the place of the two histograms, 2 * kBins words)
+  int* s_res = L.s_res;
+  int32_t* hit = df.hit + (int64_t)h * df.hit_stride;
+
+  // ---- requests first: the candidates and the resident ids (contiguous per thread, to keep slot order)
+  uint2 c[CPT];
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) c[u] = cand[min(tid + u * kSelThreads, N - 1)];
+  constexpr int kIpt = kFusedDiffMaxK / kSelThreads;
+  const int ipt = (k + kSelThreads - 1) / kSelThreads;
+  int32_t hv[kIpt];
+#pragma unroll
+  for (int u = 0; u < kIpt; ++u) hv[u] = hit[min(tid * ipt + u, k - 1)];
+  // ---- meanwhile: clear the bitmaps and the first histogram
+  {
+    uint4* z = reinterpret_cast<uint4*>(bmS);
+    for (int i = tid; i < 3 * words4 / 4; i += kSelThreads) z[i] = make_uint4(0, 0, 0, 0);
+    for (int i = tid; i < kBins; i += kSelThreads) hist[i] = 0;
+    if (tid < 8) s_res[tid] = 0;
+    if (tid < 2) L.wred[tid] = 0;
+  }
+  __syncthreads();
+  // ---- resident bitmap; range of the keys
+#pragma unroll
+  for (int u = 0; u < kIpt; ++u) {
+    const int32_t v = hv[u];
+    if (u < ipt && tid * ipt + u < k && v >= 0 && v < m) atomicOr(&bmH[v >> 5], 1u << (v & 31));
+  }
+  uint32_t vmax = 0u, vor = 0u;
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    if (tid + u * kSelThreads < N) {
+      vmax = max(vmax, c[u].x);
+      vor |= c[u].x - lo;
+    }
+  }
+  vmax = wave_reduce_u32(vmax, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+  vor = wave_reduce_u32(vor, [](uint32_t a, uint32_t b) { return a | b; });
+  if (lane_id() == 0) {
+    atomicMax(&L.wred[0], vmax);
+    atomicOr(&L.wred[1], vor);
+  }
+  __syncthreads();
+  vmax = L.wred[0];
+  vor = L.wred[1];
+  const uint32_t range = vmax - lo;
+  const int tz = vor ? (__ffs((int)vor) - 1) : 0;
+  const int nbits = range ? (32 - __clz((int)(range >> tz))) : 0;
+  const int s1 = max(nbits - 12, 0), s2 = max(s1 - 12, 0);
+  // ---- radix select of the k-th and k2-th largest keys (one pass for bf16-rounded scores)
+#pragma unroll
+  for (int u = 0; u < CPT; ++u)
+    if (tid + u * kSelThreads < N) atomicAdd(&hist[((c[u].x - lo) >> tz) >> s1], 1u);
+  __syncthreads();
+  int D1, need1, E1, needE, cntT;
+  step_find_digits(hist, hist, k, k2, L.scratch, s_res, D1, need1, E1, needE, cntT);
+  uint32_t offT = (uint32_t)D1 << s1, offE = (uint32_t)E1 << s1;
+  int need_eq = need1;
+  if (s1 > 0) {
+    for (int i = tid; i < 2 * kBins; i += kSelThreads) hist[i] = 0;
+    __syncthreads();
+    const uint32_t m2 = (1u << (s1 - s2)) - 1u;
+#pragma unroll
+    for (int u = 0; u < CPT; ++u) {
+      if (tid + u * kSelThreads < N) {
+        const uint32_t o = (c[u].x - lo) >> tz;
+        const uint32_t top = o >> s1;
+        if (top == (uint32_t)D1) atomicAdd(&hist[(o >> s2) & m2], 1u);
+        if (top == (uint32_t)E1) atomicAdd(&hist_b[(o >> s2) & m2], 1u);
+      }
+    }
+    __syncthreads();
+    int D2, need2, E2, needE2;
+    step_find_digits(hist, hist_b, need1, needE, L.scratch, s_res, D2, need2, E2, needE2, cntT);
+    offT |= (uint32_t)D2 << s2;
+    offE |= (uint32_t)E2 << s2;
+    need_eq = need2;
+    if (s2 > 0) {
+      for (int i = tid; i < kBins; i += kSelThreads) hist[i] = 0;
+      __syncthreads();
+      const uint32_t m3 = (1u << s2) - 1u;
+      const uint32_t pre = offT >> s2;
+#pragma unroll
+      for (int u = 0; u < CPT; ++u) {
+        if (tid + u * kSelThreads < N) {
+          const uint32_t o = (c[u].x - lo) >> tz;
+          if ((o >> s2) == pre) atomicAdd(&hist[o & m3], 1u);
+        }
+      }
+      __syncthreads();
+      int D3, need3, dd, dr;
+      step_find_digits(hist, hist, need2, need2, L.scratch, s_res, D3, need3, dd, dr, cntT);
+      offT |= (uint32_t)D3;
+      need_eq = need3;
+    }
+  }
+  const uint32_t Tk = lo + (offT << tz);
+  if (tid == 0) {
+    st.t_low[h] = lo + (offE << tz);
+    st.q_norm[h] = st.q_cur[h];
+  }
+  const bool all_eq = need_eq >= cntT;  // every candidate tied at the threshold is selected: no order needed
+  // ---- classify (the histograms are dead: their block becomes the bitmap of the incoming tokens)
+  for (int i = tid; i < words4; i += kSelThreads) bmM[i] = 0;
+  uint32_t selmask = 0u, eqmask = 0u;
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    if (tid + u * kSelThreads < N) {
+      const uint32_t key = c[u].x, idx = c[u].y;
+      if (key > Tk || (all_eq && key == Tk)) {
+        selmask |= 1u << u;
+        atomicOr(&bmS[idx >> 5], 1u << (idx & 31));
+      } else if (key == Tk) {
+        eqmask |= 1u << u;
+        atomicOr(&bmE[idx >> 5], 1u << (idx & 31));
+      }
+    }
+  }
+  __syncthreads();
+  const int wpt = (words4 + kSelThreads - 1) / kSelThreads;  // bitmap words per thread (<= kWordsPT)
+  const int w0 = tid * wpt;
+  if (!all_eq) {
+    // the need_eq lowest token ids among the tied candidates: rank = marked tokens before it
+    int cnt = 0;
+    for (int x = 0; x < wpt; ++x) cnt += (w0 + x < words4) ? __popc(bmE[w0 + x]) : 0;
+    int ex, exb, tot, totb;
+    step_scan2(cnt, 0, L.scratch, ex, exb, tot, totb);
+    for (int x = 0; x < wpt; ++x) {
+      if (w0 + x < words4) {
+        wpre[w0 + x] = (uint16_t)ex;
+        ex += __popc(bmE[w0 + x]);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < CPT; ++u) {
+      if ((eqmask >> u) & 1u) {
+        const uint32_t idx = c[u].y;
+        const int rank = (int)wpre[idx >> 5] + __popc(bmE[idx >> 5] & ((1u << (idx & 31)) - 1u));
+        if (rank < need_eq) {
+          selmask |= 1u << u;
+          atomicOr(&bmS[idx >> 5], 1u << (idx & 31));
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- diff: slots whose token left the selection; selected tokens that are not resident
+  bool ev[kIpt];
+  int n_ev = 0;
+#pragma unroll
+  for (int u = 0; u < kIpt; ++u) {
+    const int32_t v = hv[u];
+    const bool live = u < ipt && tid * ipt + u < k;
+    const bool in_range = v >= 0 && v < m;
+    const bool found = in_range && ((bmS[in_range ? (v >> 5) : 0] >> (v & 31)) & 1u);
+    ev[u] = live && !found;
+    n_ev += ev[u] ? 1 : 0;
+  }
+  uint32_t missmask = 0u;
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    if ((selmask >> u) & 1u) {
+      const uint32_t idx = c[u].y;
+      if (!((bmH[idx >> 5] >> (idx & 31)) & 1u)) {
+        missmask |= 1u << u;
+        atomicOr(&bmM[idx >> 5], 1u << (idx & 31));
+      }
+    }
+  }
+  __syncthreads();
+  int cnt_m = 0;
+  for (int x = 0; x < wpt; ++x) cnt_m += (w0 + x < words4) ? __popc(bmM[w0 + x]) : 0;
+  int ex_ev, ex_m, n_evict, n_missing;
+  step_scan2(n_ev, cnt_m, L.scratch, ex_ev, ex_m, n_evict, n_missing);
+#pragma unroll
+  for (int u = 0; u < kIpt; ++u) {
+    if (ev[u]) {
+      ev_slot[ex_ev] = (uint16_t)(tid * ipt + u);
+      ev_old[ex_ev] = hv[u];
+      ++ex_ev;
+    }
+  }
+  for (int x = 0; x < wpt; ++x) {
+    if (w0 + x < words4) {
+      wpre[w0 + x] = (uint16_t)ex_m;
+      ex_m += __popc(bmM[w0 + x]);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    if ((missmask >> u) & 1u) {
+      const uint32_t idx = c[u].y;
+      miss_s[(int)wpre[idx >> 5] + __popc(bmM[idx >> 5] & ((1u << (idx & 31)) - 1u))] = (int32_t)idx;
+    }
+  }
+  __syncthreads();
+  const int n_pair = min(n_missing, n_evict);
+  for (int j = tid; j < n_pair; j += kSelThreads) {
+    const int s = ev_slot[j];
+    const int32_t t_new = miss_s[j];
+    if (df.miss_old) df.miss_old[(int64_t)h * k + j] = ev_old[j];
+    if (df.miss_new) df.miss_new[(int64_t)h * k + j] = t_new;
+    hit[s] = t_new;
+    if (df.miss_slots) df.miss_slots[(int64_t)h * k + j] = s;
+  }
+  if (df.evict) {
+#pragma unroll
+    for (int u = 0; u < kIpt; ++u)
+      if (u < ipt && tid * ipt + u < k) df.evict[(int64_t)h * k + tid * ipt + u] = ev[u] ? 1 : 0;
+  }
+  if (tid == 0) {
+    if (df.vic_ptr) {
+      const int base = df.vic_ptr[h];
+      df.vic_base[h] = base;
+      df.vic_ptr[h] = (base + min(n_pair, df.vic_nv)) % df.vic_nv;
+    }
+    if (df.miss_count) df.miss_count[h] = n_pair;
+    st.cand_count[h] = 0;  // re-arm for the next call
+  }
+}
+
+// Rank of the key that the next scan's bound is taken from: 1.5 k, doubled (twice at most) for a head
+// whose list was unusable lately -- a head whose proxy query jumps from step to step needs more slack, and
+// only that head pays for it with more rows to rescore.  state: level in the low byte, calm calls above it.
+__device__ __forceinline__ int bound_rank(int k, int level, int64_t n) {
+  return (int)min((((int64_t)kBoundRankNum * k) / kBoundRankDen) << level, n);
+}
+constexpr int kCalmCalls = 32;  // usable lists in a row before a head's slack is halved again
+
+template <typename T, int R>
+__global__ __launch_bounds__(kSelThreads) void select_step_kernel(const uint2* __restrict__ cand_all, int cand_cap,
+                                                                  SelState st, uint32_t* __restrict__ keys_all,
+                                                                  int64_t key_stride, const T* __restrict__ a_k,
+                                                                  int64_t head_stride, const T* __restrict__ q_hat,
+                                                                  int64_t m, int r, int round_bf16, int k,
+                                                                  int32_t* __restrict__ out_all, int64_t out_stride,
+                                                                  DiffArgs df) {
+  LRQK_SEL_LDS(L);
+  const int h = blockIdx.x;
+  const int n = __builtin_amdgcn_readfirstlane(st.cand_count[h]);
+  const int lvl = __builtin_amdgcn_readfirstlane(st.level[h]);
+  const bool fast = n >= k && n <= cand_cap && n <= 16 * kSelThreads;
+  int level = lvl & 0xff, calm = lvl >> 8;
+  if (!fast) {
+    level = 2;
+    calm = 0;
+  } else if (level > 0 && ++calm >= kCalmCalls) {
+    --level;
+    calm = 0;
+  }
+  if (fast) {
+    if (threadIdx.x == 0) atomicAdd(&st.stats[0], 1);
+    const uint2* cand = cand_all + (int64_t)h * cand_cap;
+    const uint32_t lo = st.t_used[h];
+    const int k2 = bound_rank(k, level, n);
+    if (n <= 8 * kSelThreads)
+      select_step_fast<8>(L, cand, n, lo, st, h, m, k, k2, df);
+    else
+      select_step_fast<16>(L, cand, n, lo, st, h, m, k, k2, df);
+  } else {
+    select_generic<T, R>(L, 0, cand_all, cand_cap, st, keys_all, key_stride, a_k, head_stride, q_hat, m, r, round_bf16, k,
+                         out_all, out_stride, df, n, bound_rank(k, level, m));
+  }
+  // (both bodies hold barriers, so every thread has read the old value by now)
+  if (threadIdx.x == 0) st.level[h] = level | (calm << 8);
 }
 
 // --------------------------------------------------------------------------- host side
@@ -1152,22 +1524,23 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
   sb->key_stride = (m + 63) & ~(int64_t)63;
   if ((rc = ctx->keys.ensure((size_t)bh * sb->key_stride * 4))) return rc;
   sb->keys = (uint32_t*)ctx->keys.p;
-  sb->cand_cap = 4 * topk < 4096 ? 4096 : 4 * topk;
+  sb->cand_cap = 8 * topk < 4096 ? 4096 : 8 * topk;  // (the register-resident paths take up to 8192 and 16384 entries)
   if ((rc = ctx->cand.ensure((size_t)bh * sb->cand_cap * sizeof(uint2)))) return rc;
   sb->cand = (uint2*)ctx->cand.p;
-  // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | cand_count i32 [bh] |
+  // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | cand_count i32 [bh] | level i32 [bh] |
   // stats i32 [3]: served from the list, rescans because the list was too short, because it overflowed
   void* before = ctx->cand_cnt.p;
   constexpr int kRescSlots = 8192;  // workgroups of one index scan (never more than the GPU holds at a time)
-  if ((rc = ctx->cand_cnt.ensure((size_t)(5 * bh + 3 + bh + kRescSlots) * 4))) return rc;
+  if ((rc = ctx->cand_cnt.ensure((size_t)(6 * bh + 3 + bh + kRescSlots) * 4))) return rc;
   uint32_t* base = (uint32_t*)ctx->cand_cnt.p;
   sb->st.t_low = base;
   sb->st.q_norm = (float*)(base + bh);
   sb->st.t_used = base + 2 * bh;
   sb->st.q_cur = (float*)(base + 3 * bh);
   sb->st.cand_count = (int*)(base + 4 * bh);
-  sb->st.stats = (int*)(base + 5 * bh);
-  sb->st.rescored = (int*)(base + 5 * bh + 3);
+  sb->st.level = (int*)(base + 5 * bh);
+  sb->st.stats = (int*)(base + 6 * bh);
+  sb->st.rescored = (int*)(base + 6 * bh + 3);
   sb->st.rescored_cap = bh + kRescSlots;
   if (before != ctx->cand_cnt.p || ctx->sel_bh != bh) {
     hipLaunchKernelGGL(init_select_state_kernel, dim3((unsigned)((bh + 255) / 256)), dim3(256), 0, st, sb->st, bh);
@@ -1180,10 +1553,24 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
 template <typename T, int R>
 static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void* a_k, int64_t head_stride,
                                 const void* q_hat, int bh, int64_t m, int r, int round_bf16, int topk, int32_t* out_idx,
-                                int64_t out_stride, const DiffArgs& df, hipStream_t st) {
-  const size_t smem = select_smem(topk, df.hit != nullptr);
+                                int64_t out_stride, const DiffArgs& df, hipStream_t st, bool want_out = true) {
+  size_t smem = select_smem(topk, df.hit != nullptr);
+  // the decode step's select + diff (no ascending output): as long as its bitmaps fit the LDS beside the
+  // generic path's blocks
+  constexpr size_t kLdsStatic = (size_t)2 * kBins * 4 + 1024;
+  const bool step_path = !want_out && df.hit != nullptr && !df.replace_all && m <= kChunkBits && topk <= kFusedDiffMaxK &&
+                         std::max(smem, step_select_smem(m, topk)) + kLdsStatic <= (size_t)160 * 1024;
+  if (step_path) {
+    smem = std::max(smem, step_select_smem(m, topk));
+    static size_t step_allowed = 0;
+    if (smem > step_allowed) {
+      LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_step_kernel<T, R>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+      step_allowed = smem;
+    }
+  }
   static size_t smem_allowed = 0;
-  if (smem > smem_allowed) {
+  if (!step_path && smem > smem_allowed) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_kernel<T, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem));
     smem_allowed = smem;
@@ -1246,9 +1633,14 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
     LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used + 1], st));
     ++ctx->tev_used;
   }
-  hipLaunchKernelGGL((select_kernel<T, R>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, 0, sb.cand, sb.cand_cap,
-                     sb.st, sb.keys, sb.key_stride, (const T*)a_k, head_stride, (const T*)q_hat, m, r, round_bf16, topk,
-                     out_idx, out_stride, df);
+  if (step_path)
+    hipLaunchKernelGGL((select_step_kernel<T, R>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, sb.cand, sb.cand_cap,
+                       sb.st, sb.keys, sb.key_stride, (const T*)a_k, head_stride, (const T*)q_hat, m, r, round_bf16, topk,
+                       out_idx, out_stride, df);
+  else
+    hipLaunchKernelGGL((select_kernel<T, R>), dim3((unsigned)bh), dim3(kSelThreads), smem, st, 0, sb.cand, sb.cand_cap,
+                       sb.st, sb.keys, sb.key_stride, (const T*)a_k, head_stride, (const T*)q_hat, m, r, round_bf16, topk,
+                       out_idx, out_stride, df);
   LRQK_HIP_CHECK(hipGetLastError());
   return LRQK_OK;
 }
@@ -1256,11 +1648,12 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
 template <typename T>
 static int dispatch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void* a_k, int64_t head_stride,
                                   const void* q_hat, int bh, int64_t m, int r, int round_bf16, int topk,
-                                  int32_t* out_idx, int64_t out_stride, const DiffArgs& df, hipStream_t st) {
+                                  int32_t* out_idx, int64_t out_stride, const DiffArgs& df, hipStream_t st,
+                                  bool want_out = true) {
   const bool vec_ok = ((uintptr_t)a_k % 16 == 0) && ((head_stride * sizeof(T)) % 16 == 0);
 #define LRQK_FS_CASE(RR)                                                                                            \
   return launch_filter_select<T, RR>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, out_idx, out_stride, \
-                                     df, st)
+                                     df, st, want_out)
   if (vec_ok && r == 64) LRQK_FS_CASE(64);
   if (vec_ok && r == 32) LRQK_FS_CASE(32);
   if (vec_ok && r == 16) LRQK_FS_CASE(16);
@@ -1294,7 +1687,7 @@ static int arange_result(int bh, int64_t m, int32_t* out_idx, int64_t out_stride
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,
                       int topk, int dtype, int round_bf16, int32_t* new_idx, int32_t* hit, int64_t hit_stride,
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
-                      int32_t* miss_old, const VictimView* vic, int32_t* miss_new) {
+                      int32_t* miss_old, const VictimView* vic, int32_t* miss_new, bool want_new_idx) {
   int rc = check_select_args(ctx, bh, m, topk, new_idx, topk);
   if (rc) return rc;
   if (m <= topk || topk > kFusedDiffMaxK) {
@@ -1306,10 +1699,11 @@ int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
   DiffArgs df{hit, hit_stride, evict, miss_slots, miss_count, replace_all, miss_old, miss_new,
               vic && vic->nv > 0 ? vic->ptr : nullptr, vic && vic->nv > 0 ? vic->base : nullptr, vic ? vic->nv : 0};
   if (dtype == LRQK_F32)
-    rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, new_idx, topk, df, st);
+    rc = dispatch_filter_select<float>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, 0, topk, new_idx, topk, df, st,
+                                       want_new_idx);
   else
     rc = dispatch_filter_select<bf16_t>(ctx, sb, a_k, head_stride, q_hat, bh, m, r, round_bf16, topk, new_idx, topk, df,
-                                        st);
+                                        st, want_new_idx);
   return rc ? rc : 1;
 }
 
@@ -1357,14 +1751,20 @@ extern "C" int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t he
                                       int64_t m, int r, int topk, int dtype, int round_bf16, int32_t* new_idx,
                                       int32_t* hit, int64_t hit_stride, uint8_t* evict, int32_t* miss_slots,
                                       int32_t* miss_count, void* stream) {
-  LRQK_REQUIRE(a_k && q_hat && new_idx && hit && miss_slots && miss_count, LRQK_EINVAL, "null pointer");
+  LRQK_REQUIRE(ctx && a_k && q_hat && hit && miss_slots && miss_count, LRQK_EINVAL, "null pointer");
+  const bool want_new = new_idx != nullptr;
+  if (!want_new) {  // the caller only wants what changes: the selection is never put in order
+    int rce = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t));
+    if (rce) return rce;
+    new_idx = (int32_t*)ctx->new_idx.p;
+  }
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_EINVAL, "r=%d", r);
   LRQK_REQUIRE(m > topk, LRQK_EINVAL, "m=%lld must exceed topk=%d (no diff happens in the prefix branch)",
                (long long)m, topk);
   LRQK_REQUIRE(head_stride >= m * r && hit_stride >= topk, LRQK_EINVAL, "stride too small");
   int rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_bf16, new_idx, hit, hit_stride,
-                             evict, miss_slots, miss_count, 0, (hipStream_t)stream);
+                             evict, miss_slots, miss_count, 0, (hipStream_t)stream, nullptr, nullptr, nullptr, want_new);
   if (rc < 0) return rc;
   if (rc == 0) return lrqk_diff(new_idx, topk, hit, hit_stride, bh, topk, evict, miss_slots, miss_count, stream);
   return LRQK_OK;
@@ -1404,7 +1804,7 @@ extern "C" int lrqk_scan_stats(lrqk_ctx* ctx, int64_t* rows_scanned, int64_t* ro
   *rows_scanned = *rows_rescored = 0;
   if (!ctx->cand_cnt.p || ctx->sel_bh <= 0 || ctx->scan_wgs <= 0) return LRQK_OK;
   std::vector<int> v((size_t)ctx->scan_wgs);
-  LRQK_HIP_CHECK(hipMemcpy(v.data(), (int*)ctx->cand_cnt.p + 5 * ctx->sel_bh + 3, v.size() * sizeof(int),
+  LRQK_HIP_CHECK(hipMemcpy(v.data(), (int*)ctx->cand_cnt.p + 6 * ctx->sel_bh + 3, v.size() * sizeof(int),
                            hipMemcpyDeviceToHost));
   int64_t t = 0;
   for (int x : v) t += x;
@@ -1417,7 +1817,7 @@ extern "C" int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads
   LRQK_REQUIRE(ctx && fast_heads && full_heads, LRQK_EINVAL, "null pointer");
   *fast_heads = *full_heads = 0;
   if (!ctx->cand_cnt.p || ctx->sel_bh <= 0) return LRQK_OK;
-  int* stats = (int*)ctx->cand_cnt.p + 5 * ctx->sel_bh;
+  int* stats = (int*)ctx->cand_cnt.p + 6 * ctx->sel_bh;
   int v[3];
   LRQK_HIP_CHECK(hipMemcpy(v, stats, sizeof(v), hipMemcpyDeviceToHost));
   *fast_heads = v[0];

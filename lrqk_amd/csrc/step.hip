@@ -57,7 +57,8 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   }
   const VictimView* vic = fused_tail && ctx->vic.nv > 0 && !ctx->vic_dirty ? &ctx->vic : nullptr;
   rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_scores, new_idx, active_idx, n, ev,
-                         miss_slots, mcount, no_hit_miss, (hipStream_t)stream, miss_old, vic, miss_new);
+                         miss_slots, mcount, no_hit_miss, (hipStream_t)stream, miss_old, vic, miss_new,
+                         /*want_new_idx=*/false);
   const bool fused_diff = rc == 1;  // the select kernel also wrote miss_old / miss_new
   const bool vic_active = vic != nullptr && fused_diff;
   if (rc < 0) return rc;

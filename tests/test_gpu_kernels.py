@@ -313,6 +313,69 @@ def test_score_select_diff_fused(ops, oracle, m, cap, k, H, dtype):
         q = (q.float() + 0.05 * torch.randn(q.shape, generator=g)).to(dtype)
 
 
+@pytest.mark.parametrize("m,k,H,dtype,r,index,ties", [(40000, 512, 3, torch.bfloat16, 16, False, False),
+                                                       (131500, 2048, 4, torch.bfloat16, 32, True, False),
+                                                       (131500, 2048, 2, torch.bfloat16, 32, True, True),
+                                                       (262144, 2048, 2, torch.bfloat16, 16, True, False),
+                                                       (131500, 2048, 2, torch.bfloat16, 32, False, False),
+                                                       (30000, 4096, 2, torch.float32, 16, True, False),
+                                                       (9000, 1024, 2, torch.float32, 8, False, True)])
+def test_score_select_diff_unordered(ops, oracle, m, k, H, dtype, r, index, ties):
+    """The decode step's form of the fused select + diff (no ascending list; lrqk_score_select_diff with
+    new_idx = NULL) against the oracle's two stages, over several rounds on one workspace (the first has no
+    carried bound and rescans; later ones take the candidate list, also a list of more than 8192 entries
+    when the query shrinks).  `ties`: scores take a handful of values, so the threshold cuts through a large
+    class of equal scores and the lowest token ids of that class must win."""
+    _say("score_select_diff unordered", m, k, H, dtype, r, index, ties)
+    ws = ops.Workspace()
+    ws.score_index(index)
+    g = torch.Generator().manual_seed(m + k + r)
+    if ties:
+        A = torch.zeros((1, H, m, r))
+        A[..., 0] = torch.randint(0, 40 if m > 100000 else 5, (1, H, m), generator=g).float()
+        q = torch.zeros((1, H, 1, r))
+        q[..., 0] = 1.0
+        A, q = A.to(dtype), q.to(dtype)
+    else:
+        A = torch.randn((1, H, m, r), generator=g).to(dtype)
+        q = torch.randn((1, H, 1, r), generator=g).to(dtype)
+    hit = torch.stack([torch.randperm(m, generator=g)[:k] for _ in range(H)]).view(1, H, k).to(torch.int32)
+    Ad = A.to(DEV)
+    hit_d = hit.to(DEV).contiguous()
+    now = hit.long().unsqueeze(-1)
+    turn = not index and m > 100000
+    if turn:
+        # rows three times as long along the first coordinate: a query of the same length that turns towards it
+        # spreads the scores 1.5 times as wide, and the plain scan's bound (which follows |q| only) lets ~10 k
+        # rows through -- a list beyond the 8192 entries of the usual register budget
+        A[..., 0] *= 3.0
+        q[..., 0] = 0.0
+        q = q / q.float().norm(dim=-1, keepdim=True)
+        Ad = A.to(DEV)
+    scales = [1.0, 1.0, 1.0, 0.45, 1.0, 2.5, 1.0]
+    for rnd, sc in enumerate(scales):
+        if turn and rnd in (3, 5):
+            qf = q.float()
+            qf[..., 0] = 0.4 if rnd == 3 else 0.0
+            q = (qf / qf.norm(dim=-1, keepdim=True)).to(dtype)
+        elif not ties:
+            q = ((q.float() + 0.05 * torch.randn(q.shape, generator=g)) * sc).to(dtype)
+        exp_new = oracle.compute_hit_indices(q, A, k, True)
+        exp_upd, exp_ev = oracle.only_indices_in_cpu(now, exp_new)
+        new, evict, slots, count = ops.score_select_diff(ws, Ad, q.to(DEV), m, k, hit_d, want_new=False)
+        assert new is None
+        assert torch.equal(hit_d.cpu().long(), exp_upd[..., 0]), rnd
+        assert torch.equal(evict.cpu().bool(), exp_ev), rnd
+        assert torch.equal(count.cpu().long(), exp_ev.sum(-1)), rnd
+        for h in range(H):
+            c = int(count[0, h])
+            assert slots[0, h, :c].cpu().tolist() == exp_ev[0, h].nonzero().view(-1).tolist()
+        now = exp_upd
+    fast, full = ws.select_stats()
+    _say("   heads served from the list:", fast, "rescanned:", full)
+    assert fast > 0
+
+
 def test_score_select_many_chunks(ops, ws, oracle):
     """More candidates than one bitmap chunk covers (262144): the ordered output runs chunk by chunk."""
     _say("score_select many chunks")
