@@ -13,6 +13,7 @@
 // dimensions that are a multiple of the 16-byte vector, and a generic VALU version for
 // every other shape.  Both write the same partial-sum layout.
 #include <algorithm>
+#include <stdlib.h>
 
 #include "common.hpp"
 #include "ctx.hpp"
@@ -536,7 +537,9 @@ __device__ __forceinline__ bf16x8 pf_bf16x8(uint32_t a, uint32_t b, uint32_t c, 
   return __builtin_bit_cast(bf16x8, make_uint4(a, b, c, d));
 }
 
-template <int NB, int NW>
+// GRAMS = false: only A <- X Mt^T (the last pass of the iteration on Gram matrices, which needs neither the sums
+// over the new rows nor their change): the old rows are not read and nothing is reduced.
+template <int NB, int NW, bool GRAMS = true>
 __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* __restrict__ X, int xh, int hq,
                                                                   int64_t l, int r, int d,
                                                                   const float* __restrict__ Mt, float* __restrict__ A,
@@ -636,10 +639,12 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
 
     floatx16 c;
     float old[16];
+    if constexpr (GRAMS) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
-      old[v] = Ah[rr * r + min(col, r - 1)];
+      for (int v = 0; v < 16; ++v) {
+        const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
+        old[v] = Ah[rr * r + min(col, r - 1)];
+      }
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) c[v] = 0.0f;
@@ -660,14 +665,20 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       for (int v = 0; v < 16; ++v) {
         const int row = pf_mfma_row(lane, v);
         if (row < rows && col < r) {
-          const float df = old[v] - c[v];
-          dsum = fmaf(df, df, dsum);
+          if constexpr (GRAMS) {
+            const float df = old[v] - c[v];
+            dsum = fmaf(df, df, dsum);
+          }
           Ah[(t0 + row) * r + col] = c[v];
         }
       }
     } else {
 #pragma unroll
       for (int v = 0; v < 16; ++v) c[v] = (pf_mfma_row(lane, v) < rows && col < r) ? old[v] : 0.0f;
+    }
+    if constexpr (!GRAMS) {
+      pf_wave_sync();  // this wave's reads of the tile precede its next staging writes
+      continue;
     }
     // the three pieces of C, eight rows (one k block) at a time
     bf16x8 cp[3][2];
@@ -735,6 +746,7 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
     }
     pf_wave_sync();  // this wave's reads of the tile precede its next staging writes
   }
+  if constexpr (!GRAMS) return;
   __syncthreads();  // every wave is done with its tile (and with Mt): the LDS is reused below
 
   // reduce the waves' tiles through LDS, one 32 x 32 block at a time (tile nb of G_AX: columns 32 nb + n)
@@ -1016,6 +1028,27 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
                      (float*)nullptr, (const int*)nullptr, S);
   LRQK_HIP_CHECK(hipGetLastError());
+  if constexpr (sizeof(T) == 2) {
+    // bf16 rows of 128 elements: every iteration on the d x d Gram matrices (fp64), then one pass per side
+    // that applies the last Mq, Mk
+    if (mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE")) {
+      float *mt_q = nullptr, *mt_k = nullptr;
+      if ((rc = prefill_gram_domain(ctx, q, k, partQ, partK, S, b_q, b_k, b, hq, hkv, l, r, iters, tol, flags, &mt_q,
+                                    &mt_k, st)))
+        return rc;
+      if (iters > 0) {
+        PfPassFn<T> lean = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, false>;
+        if (smem_pass > 48 * 1024)
+          LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)lean, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
+        hipLaunchKernelGGL(lean, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)mt_q, a_q, partQ, deltas,
+                           (const int*)nullptr, S);
+        hipLaunchKernelGGL(lean, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)mt_k, a_k, partK,
+                           deltas + (size_t)bh * S, (const int*)nullptr, S);
+        LRQK_HIP_CHECK(hipGetLastError());
+      }
+      return LRQK_OK;
+    }
+  }
   for (int it = 0; it < iters; ++it) {
     float* dq = deltas + ((size_t)it * 2 + 0) * bh * S;
     float* dk = deltas + ((size_t)it * 2 + 1) * bh * S;

@@ -51,6 +51,7 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->als_kq.release();
   ctx->als_iter.release();
   ctx->prefill_ws.release();
+  ctx->prefill_gd.release();
   ctx->new_idx.release();
   ctx->misc.release();
   ctx->stage_dev.release();

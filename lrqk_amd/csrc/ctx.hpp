@@ -58,6 +58,7 @@ struct lrqk_ctx {
   lrqk::DevBuf als_pre;     // f32 [bh][4*1024 + 65]: what the solve needs from B_Q, B_K, q, k (formed beside the Gram pass)
   lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
+  lrqk::DevBuf prefill_gd;  // prefill ALS on Gram matrices: X^T X sums, fp64 state
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
   lrqk::DevBuf misc;        // evict mask, miss lists, counters of the fused step
   // finish stage of the factor update deferred into later launches of the decode step
@@ -106,6 +107,10 @@ int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
                       uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, int replace_all, hipStream_t st,
                       int32_t* miss_old = nullptr, const VictimView* vic = nullptr, int32_t* miss_new = nullptr,
                       bool want_new_idx = true);
+// Prefill iterations on Gram matrices (bf16 input, d = 128, r <= 32); see als_prefill_gram.hip.
+int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float* partQ, const float* partK, int S,
+                        float* b_q, float* b_k, int b, int hq, int hkv, int64_t l, int r, int iters, float tol, int* flags,
+                        float** mt_q, float** mt_k, hipStream_t st);
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
 // into its first kernel.
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
