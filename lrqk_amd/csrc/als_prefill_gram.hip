@@ -152,20 +152,33 @@ __device__ __forceinline__ void gd_solve(double (&x)[32], int col, double* __res
         for (int i = 0; i < 32; ++i) mine[i] = x[i];
       }
       __syncthreads();
-      // inverse of the pivot block [[a, b], [b', c]] (rows q, q + 1 of the two columns)
-      const double a = pv[q], bb = pv[32 + q], b2 = pv[q + 1], c = pv[32 + q + 1];
-      const double det = fma(a, c, -bb * b2);
-      double inv = __builtin_amdgcn_rcp(det);
-      inv = fma(fma(-det, inv, 1.0), inv, inv);
-      inv = fma(fma(-det, inv, 1.0), inv, inv);
-      const double xa = (c * x[q] - bb * x[q + 1]) * inv;
-      const double xb = (a * x[q + 1] - b2 * x[q]) * inv;
+      if (col >= 0) {  // (wave-uniform but for the last wave of a group: idle threads stay off the LDS)
+        // the two columns as 16-byte reads
+        double c0[32], c1[32];
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        if (i != q && i != q + 1) x[i] = fma(-pv[i], xa, fma(-pv[32 + i], xb, x[i]));
+        for (int i = 0; i < 32; i += 2) {
+          const double2 u0 = *reinterpret_cast<const double2*>(pv + i);
+          const double2 u1 = *reinterpret_cast<const double2*>(pv + 32 + i);
+          c0[i] = u0.x;
+          c0[i + 1] = u0.y;
+          c1[i] = u1.x;
+          c1[i + 1] = u1.y;
+        }
+        // inverse of the pivot block [[a, b], [b', c]] (rows q, q + 1 of the two columns)
+        const double a = c0[q], bb = c1[q], b2 = c0[q + 1], c = c1[q + 1];
+        const double det = fma(a, c, -bb * b2);
+        double inv = __builtin_amdgcn_rcp(det);
+        inv = fma(fma(-det, inv, 1.0), inv, inv);
+        inv = fma(fma(-det, inv, 1.0), inv, inv);
+        const double xa = (c * x[q] - bb * x[q + 1]) * inv;
+        const double xb = (a * x[q + 1] - b2 * x[q]) * inv;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+          if (i != q && i != q + 1) x[i] = fma(-c0[i], xa, fma(-c1[i], xb, x[i]));
+        }
+        x[q] = xa;
+        x[q + 1] = xb;
       }
-      x[q] = xa;
-      x[q + 1] = xb;
     }
     // rotate by four: the next pivot rows move to positions 0..3
     const double t0 = x[0], t1 = x[1], t2 = x[2], t3 = x[3];
@@ -509,9 +522,9 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
                         float** mt_q, float** mt_k, hipStream_t st) {
   const int bh = b * hq, bkv = b * hkv;
   const int d = kGdD;
-  // splits of the long axis for the X^T X sums: about one workgroup per CU
-  int Sx = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 256 / bh), (l + 511) / 512));
-  int Sxk = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 256 / bkv), (l + 511) / 512));
+  // splits of the long axis for the X^T X sums: about two workgroups per CU (measured: 89 us against 103 with one)
+  int Sx = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 512 / bh), (l + 511) / 512));
+  int Sxk = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 512 / bkv), (l + 511) / 512));
   int rc = ctx->prefill_gd.ensure(gramdom_bytes(bh, bkv, Sx, Sxk, iters));
   if (rc) return rc;
   const size_t dd = (size_t)d * d;
