@@ -29,10 +29,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 # HBM bytes per launch of the proxy-score kernel read from hardware counters (rocprofv3 --pmc FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB device copy: x2.000 and x1.000), per
-# workload at its default context.  The summary of those runs is kept under profiles/.
+# workload at its default context (the scaling factors come from this library's own probe kernels of known size in
+# the same runs).  The summary of those runs is kept under profiles/.
 # Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
 # 8-bit copy (36 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
-MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (84032.6 * 2.000 + 837.7 * 1.000) * 1024,
+MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (83860.8 * 2.000 + 867.4 * 1.000) * 1024,
                           ("llama8b_128k_bf16", False): (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
 
 
@@ -170,7 +171,26 @@ def prefill_als(a):
     # HBM bytes: every pass reads X once; apply passes read and write A (fp32), Gram passes read A
     bytes_ = bh * ((2 + 2 * iters) * l * d * e + 2 * l * r * 4 + iters * 2 * 2 * l * r * 4)
     tf = flops / (ms * 1e-3) / 1e12
-    if e == 2 and d <= 128:
+    bkv = w.batch * w.num_kv_heads
+    if e == 2 and d == 128 and r <= 32 and not os.environ.get("LRQK_PREFILL_ROWWISE"):
+        # bf16 rows of 128 elements: the iterations run on d x d Gram matrices (fp64, 32 small independent problems),
+        # and the long axis is read three times whatever the iteration count: initial Grams of the given factors,
+        # X^T X, and the final A = X M.  HBM bytes: 3 x (Q + K, K once per kv head) + the initial factors read
+        # + the final factors written (fp32).
+        bytes_g = 3.0 * (bh + bkv) * l * d * e + 4.0 * bh * l * r * 4
+        gbs = bytes_g / (ms * 1e-3) / 1e9
+        # executed bf16 MFMAs of 32x32x16 per 32 rows: 48 per side (initial Grams, three-piece operands),
+        # 32 per input head (X^T X), 24 per side (apply)
+        exec_flops = (l / 32.0) * (bh * 2 * (48 + 24) + (bh + bkv) * 32) * 2.0 * 32 * 32 * 16
+        roof = {"bound": "hbm", "kernel": "pf_pass_bf16_kernel + pf_xtx_kernel (three readings of the long axis); "
+                                          "pf_gramdom_kernel (fp64 d x d algebra per head, latency-bound) between them",
+                "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                "traffic": None, "hbm_bytes_per_call": round(bytes_g),
+                "algorithmic_flops_per_call": round(flops), "algorithmic_equiv_tflops": round(tf, 2),
+                "executed_bf16_mfma_tflops": round(exec_flops / (ms * 1e-3) / 1e12, 1),
+                "executed_bf16_mfma_frac": round(exec_flops / (ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
+                "readings_of_the_long_axis": 3, "row_by_row_formulation_readings": 1 + iters}
+    elif e == 2 and d <= 128:
         # bf16 input: the passes run on the bf16 matrix cores (fp32 operands as three bf16 pieces), where the
         # arithmetic is far from any limit; what bounds them is the stream over X and A
         gbs = bytes_ / (ms * 1e-3) / 1e9
