@@ -622,7 +622,6 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                          (head_stride * sizeof(T)) % 16 == 0 && !getenv("LRQK_GRAM_OLD");
   // (the pipelined pass: two chunks per wave measured best at 1, 4 and 8 sequences of the Llama-3-8B shape)
   if (fast_bf16) S = std::min(32, std::max(1, (n + 2 * kGramWaves * kGramChunk - 1) / (2 * kGramWaves * kGramChunk)));
-  if (const char* e = getenv("LRQK_GRAM_S")) S = atoi(e);
   int rc = ctx->als_part.ensure((size_t)bh * S * kGramNe * sizeof(float));
   if (rc) return rc;
   if ((rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float)))) return rc;
@@ -636,8 +635,9 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                 "the solve kernel's LDS fits the default dynamic limit");
   // the Gram launch carries two more workgroups per head, each with B_Q or B_K (fp32, padded rows) in LDS
   const size_t smem_gram = ((size_t)32 * (d + 1) + 2 * d) * sizeof(float);
-  static size_t gram_allowed = 48 * 1024;
-  if (smem_gram > gram_allowed) {
+  static std::atomic<size_t> gram_allowed_dev[kMaxDeviceSlots];
+  std::atomic<size_t>& gram_allowed = gram_allowed_dev[per_device_slot()];
+  if (smem_gram > std::max<size_t>(gram_allowed, 48 * 1024)) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_gram_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem_gram));
     gram_allowed = smem_gram;

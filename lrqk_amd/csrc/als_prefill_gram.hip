@@ -21,7 +21,6 @@
 // bf16 x bf16 products added in fp32 tile by tile and across tiles, then across splits in fp64.  Measured
 // against the fp64 restatement the results are closer than the same iteration in fp32 LAPACK.
 #include <algorithm>
-#include <stdlib.h>
 
 #include "common.hpp"
 #include "ctx.hpp"
@@ -285,7 +284,6 @@ struct GdArgs {
   int bh, hq, hkv, r;
   int64_t l;
   float tol;
-  int dbg;
 };
 
 // The state (G, C) of both sides from the first Gram passes: S partial sums of [G | C] packed as [r][r + d]
@@ -365,7 +363,7 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
 #pragma unroll
     for (int i = 0; i < 32; ++i) x[i] = t < 32 ? G[i * 32 + t] : C[i * d + c];
   }
-  if (!(a.dbg & 1)) gd_solve(x, t, piv + 128 * grp);
+  gd_solve(x, t, piv + 128 * grp);
   if (stage == 2) {
     if (t >= 32) {
       float* out = (grp ? a.b_k : a.b_q) + (int64_t)h * r * d;
@@ -386,7 +384,7 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   // ---- W1 = Gk + B_Q B_Q^T
   {
     double o[4];
-    if (!(a.dbg & 4)) gd_outer(BT, BT, o);
+    gd_outer(BT, BT, o);
     if (tid < 256) {
       const int i = tid >> 3, j0 = (tid & 7) * 4;
 #pragma unroll
@@ -402,7 +400,7 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   __syncthreads();
   {
     double o[4];
-    if (!(a.dbg & 4)) gd_outer(BT, BT, o);
+    gd_outer(BT, BT, o);
     if (tid < 256) {
       const int i = tid >> 3, j0 = (tid & 7) * 4;
 #pragma unroll
@@ -415,7 +413,7 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     for (int i = 0; i < 32; ++i) x[i] = t < 32 ? Gs[i * kGdLg + t] : Ck[i * d + c] + bcol[i];
   }
   __syncthreads();  // (W1 is read above from what the previous block wrote; B_K B_K^T is complete)
-  if (!(a.dbg & 1)) gd_solve(x, grp == 0 ? t : -1, piv);
+  gd_solve(x, grp == 0 ? t : -1, piv);
   double part_q = 0.0;  // sum of Cq (the old one) . Mq'^T over this thread's column
   if (grp == 0 && t >= 32) {
     float* mt = a.Mt_q + (int64_t)h * r * d;
@@ -432,10 +430,10 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   if (tid < 32) tr_old = tid < r ? Gq[tid * 32 + tid] : 0.0;
   __syncthreads();
   // ---- T = Mq'^T Sq, Gq' = Mq'^T T^T
-  if (!(a.dbg & 2)) gd_times_s(MT, Sq, TT);
+  gd_times_s(MT, Sq, TT);
   {
     double o[4];
-    if (!(a.dbg & 4)) gd_outer(MT, TT, o);
+    gd_outer(MT, TT, o);
     double tr_new = 0.0;
     if (tid < 256) {
       const int i = tid >> 3, j0 = (tid & 7) * 4;
@@ -463,7 +461,7 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
       x[i] = t < 32 ? Gs[2 * 32 * kGdLg + i * kGdLg + t] + Gs[32 * kGdLg + i * kGdLg + t] : TT[c * kGdLd + i] + bcol[i];
   }
   __syncthreads();
-  if (!(a.dbg & 1)) gd_solve(x, grp == 1 ? t : -1, piv + 128);
+  gd_solve(x, grp == 1 ? t : -1, piv + 128);
   double part_k = 0.0;
   if (grp == 1 && t >= 32) {
     float* mt = a.Mt_k + (int64_t)h * r * d;
@@ -480,10 +478,10 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   if (tid < 32) trk_old = tid < r ? Gk[tid * 32 + tid] : 0.0;
   __syncthreads();
   // ---- U = Mk'^T Sk, Gk' = Mk'^T U^T, Ck' = U
-  if (!(a.dbg & 2)) gd_times_s(MT, Sk, TT);
+  gd_times_s(MT, Sk, TT);
   {
     double o[4];
-    if (!(a.dbg & 4)) gd_outer(MT, TT, o);
+    gd_outer(MT, TT, o);
     double tr_new = 0.0;
     if (tid < 256) {
       const int i = tid >> 3, j0 = (tid & 7) * 4;
@@ -548,13 +546,14 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
                      (const float*)xk_part, Sxk, (int)dd, Sk);
   LRQK_HIP_CHECK(hipGetLastError());
   const size_t smem = ((size_t)3 * kGdD * kGdLd + 3 * 32 * kGdLg + 256 + 8) * sizeof(double);
-  static bool attr = false;
+  static std::atomic<bool> attr_dev[kMaxDeviceSlots];
+  std::atomic<bool>& attr = attr_dev[per_device_slot()];
   if (!attr) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)pf_gramdom_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem));
     attr = true;
   }
-  GdArgs a{partQ, partK, S, Sq, Sk, G, C, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol, getenv("LRQK_GD_DBG") ? atoi(getenv("LRQK_GD_DBG")) : 0};
+  GdArgs a{partQ, partK, S, Sq, Sk, G, C, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol};
   hipLaunchKernelGGL(pf_gramdom_init_kernel, dim3((unsigned)((32 * (32 + kGdD) + 255) / 256), (unsigned)bh, 2u), dim3(256), 0,
                      st, a);
   for (int it = 0; it < iters; ++it)

@@ -9,7 +9,6 @@
 // the others meanwhile run the attention over the slots that stay resident; the combine
 // kernel then adds the freshly fetched slots of its head before merging.
 #include <math.h>
-#include <stdlib.h>
 
 #include <mutex>
 
@@ -639,13 +638,16 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   // The launch should not hold more workgroups than the GPU does at a time (a second batch would only start when
   // the first has finished): 128 slots per attention workgroup if everything fits, else 256, and as many fetch
   // workgroups as still fit, between 8 and the number that a miss rate of 1/8 keeps busy.
-  static int slots = 0;
+  static std::atomic<int> slots_dev[kMaxDeviceSlots];
+  std::atomic<int>& slots_a = slots_dev[per_device_slot()];
+  int slots = slots_a;
   if (slots == 0) {
     int per_cu = 0, dev = 0, n_cu = 0;
     LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fetch_attn_partial_kernel<T>, kAttnThreads, 0));
     LRQK_HIP_CHECK(hipGetDevice(&dev));
     LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     slots = std::max(1, per_cu * n_cu);
+    slots_a = slots;
   }
   const int rpb = kAttnThreads / (2 * cpr);
   const int want_fetch = std::max(1, std::min(32, (k / 8 + rpb - 1) / rpb));
@@ -653,9 +655,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   if ((int64_t)(S + want_fetch + 2) * bh > slots) S = (n_slots + 255) / 256;
   if (S > 64) S = 64;
   const int room = slots / bh - S - 2;
-  int n_fetch = std::min(want_fetch, std::max(room, 8));
-  if (const char* e = getenv("LRQK_FA_S")) S = atoi(e);
-  if (const char* e = getenv("LRQK_FA_NF")) n_fetch = atoi(e);
+  const int n_fetch = std::min(want_fetch, std::max(room, 8));
   if ((rc = ctx->attn_part.ensure((size_t)bh * (S + n_fetch) * (d + 2) * sizeof(float)))) return rc;
   const float scale_log2e = (1.0f / sqrtf((float)d)) * 1.4426950408889634f;
   static_assert(kAttnThreads == kFinThreads, "the finish stage rides in an attention-sized workgroup");

@@ -1,5 +1,6 @@
 // Library-owned device workspace.
 #pragma once
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
@@ -100,6 +101,15 @@ struct lrqk_ctx {
 };
 
 namespace lrqk {
+// Launch set-up that is remembered between calls (function attributes raised so far, occupancy figures) belongs to
+// a device: one slot per device ordinal, atomics because callers may come from several host threads (the set-up
+// itself is idempotent, so a duplicate is harmless).
+constexpr int kMaxDeviceSlots = 64;
+inline int per_device_slot() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  return dev >= 0 && dev < kMaxDeviceSlots ? dev : 0;
+}
 // Proxy-score scan + top-k with the hit/miss diff fused into the select kernel when the
 // sizes allow.  Returns 1 if the diff ran, 0 if the caller still has to, negative on error.
 int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const void* q_hat, int bh, int64_t m, int r,

@@ -195,7 +195,8 @@ extern "C" int lrqk_diff(const int32_t* new_idx, int64_t new_stride, int32_t* hi
   LRQK_REQUIRE(k > 0 && k <= LRQK_MAX_TOPK, LRQK_ELIMIT, "k=%d not in 1..%d", k, LRQK_MAX_TOPK);
   LRQK_REQUIRE(new_stride >= k && hit_stride >= k, LRQK_EINVAL, "stride smaller than k");
   const size_t smem = (size_t)k * 10;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set_dev[kMaxDeviceSlots];
+  std::atomic<bool>& attr_set = attr_set_dev[per_device_slot()];
   if (smem > 48 * 1024 && !attr_set) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)diff_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        LRQK_MAX_TOPK * 10));

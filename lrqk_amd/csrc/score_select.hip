@@ -1562,14 +1562,16 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
                          std::max(smem, step_select_smem(m, topk)) + kLdsStatic <= (size_t)160 * 1024;
   if (step_path) {
     smem = std::max(smem, step_select_smem(m, topk));
-    static size_t step_allowed = 0;
+    static std::atomic<size_t> step_allowed_dev[kMaxDeviceSlots];
+    std::atomic<size_t>& step_allowed = step_allowed_dev[per_device_slot()];
     if (smem > step_allowed) {
       LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_step_kernel<T, R>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
       step_allowed = smem;
     }
   }
-  static size_t smem_allowed = 0;
+  static std::atomic<size_t> smem_allowed_dev[kMaxDeviceSlots];
+  std::atomic<size_t>& smem_allowed = smem_allowed_dev[per_device_slot()];
   if (!step_path && smem > smem_allowed) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_kernel<T, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem));
@@ -1578,7 +1580,8 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
   const bool timed = ctx->tev && ctx->tev_used < ctx->tev_pairs && (ctx->tev_seen++ % ctx->tev_every) == 0;
   if (timed) LRQK_HIP_CHECK(hipEventRecord(ctx->tev[2 * ctx->tev_used], st));
   constexpr size_t filt_smem = (size_t)kFiltRows * kFiltTiles * sizeof(uint2);
-  static bool filt_attr = false;
+  static std::atomic<bool> filt_attr_dev[kMaxDeviceSlots];
+  std::atomic<bool>& filt_attr = filt_attr_dev[per_device_slot()];
   if (!filt_attr && filt_smem > 48 * 1024) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)score_filter_kernel<T, R>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)filt_smem));
@@ -1604,13 +1607,16 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
     if (ri < 0) return ri;
     if (ri == 1) {
       // no more workgroups than the GPU holds at a time: beyond that a workgroup takes more tiles
-      static int slots = 0;
+      static std::atomic<int> slots_dev[kMaxDeviceSlots];
+      std::atomic<int>& slots_a = slots_dev[per_device_slot()];
+      int slots = slots_a;
       if (slots == 0) {
         int per_cu = 0, dev = 0, n_cu = 0;
         LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, score_prefilter_kernel<T, R>, kFiltThreads, 0));
         LRQK_HIP_CHECK(hipGetDevice(&dev));
         LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
         slots = std::max(1, per_cu * n_cu);
+        slots_a = slots;
       }
       const int64_t tiles = (m + kFiltRows - 1) / kFiltRows;
       const int64_t wgs = std::max<int64_t>(1, std::min<int64_t>((tiles + kFiltTiles - 1) / kFiltTiles, slots / bh));
@@ -1785,7 +1791,8 @@ extern "C" int lrqk_select_from_scores(lrqk_ctx* ctx, const float* scores, int b
                      sb.key_stride);
   LRQK_HIP_CHECK(hipGetLastError());
   const size_t smem = select_smem(topk, false);
-  static bool attr_done = false;
+  static std::atomic<bool> attr_done_dev[kMaxDeviceSlots];
+  std::atomic<bool>& attr_done = attr_done_dev[per_device_slot()];
   if (!attr_done) {
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)select_kernel<float, 0>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem));
