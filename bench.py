@@ -70,6 +70,10 @@ def parse():
     p.add_argument("--seqs", type=int, default=0,
                    help="decode mode: sequences stepped together (the batch of the layer-step; 0 = the workload's "
                         "own, 1 for the 128K configuration); value stays the time of one layer-step of the whole batch")
+    p.add_argument("--context-scale", type=float, default=0.0,
+                   help="decoder mode: length of a fixed direction added to every token embedding (in embedding "
+                        "lengths); > 0 makes successive queries correlated, as a trained model's are (random weights and "
+                        "random ids alone give unrelated queries and a hit rate of k / l)")
     p.add_argument("--settle", type=int, default=512,
                    help="decode mode: further untimed steps before the warm-up steps.  The first process on a box "
                         "enqueues its first few hundred steps several times slower than later ones (cold host-side "
@@ -226,7 +230,7 @@ def decoder(a):
     cfg = DecoderConfig(layers=a.layers)
     dev = torch.device("cuda:0")
     t0 = time.perf_counter()
-    model = LlamaShapeDecoder(cfg, torch.bfloat16, dev, seed=a.seed)
+    model = LlamaShapeDecoder(cfg, torch.bfloat16, dev, seed=a.seed, context_scale=a.context_scale)
     model.progress = lambda msg: print(msg, file=sys.stderr, flush=True)
     g = torch.Generator(device=dev).manual_seed(a.seed + 1)
     ids = torch.randint(0, cfg.vocab, (a.batch, a.prompt), generator=g, device=dev)
@@ -241,17 +245,60 @@ def decoder(a):
         m_, s_, _ = cache.lwattn[li].miss_stats()
         miss += m_
         sel += s_
+    # a few more positions with an event pair around every layer's cache path (update + attention): the share of
+    # a decoded position that the path takes, the rest being the projections, MLP and lm_head
+    model.path_events = []
+    tok = toks[:, -1]
+    pos = a.prompt + a.new_tokens - 1
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    extra = 8
+    for _ in range(extra):
+        tok = model.forward(tok[:, None], pos, cache).argmax(-1)
+        pos += 1
+    torch.cuda.synchronize()
+    t_extra = (time.perf_counter() - t0) / extra
+    path_us = sum(e0.elapsed_time(e1) for e0, e1 in model.path_events) * 1e3 / len(model.path_events)
+    model.path_events = None
+    cpu = None
+    if a.cpu_steps > 0:
+        # the oracle's cache path (factor update, scan, select, diff, gather, attention) of ONE layer at this batch
+        # and context, continued from layer 0's state with stand-in q, k, v; everything else a decoded position
+        # needs (projections, MLP, lm_head, the other layers) is not in this figure
+        import types
+        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        eng0 = cache.lwattn[0]
+        wl = types.SimpleNamespace(lite_tokens=64, num_active_tokens=2048, groups=cfg.heads // cfg.kv_heads, r=32,
+                                   max_iter=(2, 2), tol=(1e-2, 1e-2))
+        o, orc = oracle_from_engine(eng0, wl, threads)
+        gq = torch.Generator().manual_seed(a.seed + 7)
+        qkv = [(torch.randn((a.batch, cfg.heads, 1, cfg.head_dim), generator=gq).bfloat16(),
+                torch.randn((a.batch, cfg.kv_heads, 1, cfg.head_dim), generator=gq).bfloat16(),
+                torch.randn((a.batch, cfg.kv_heads, 1, cfg.head_dim), generator=gq).bfloat16()) for _ in range(2)]
+        Ko, Vo = o.decode(*qkv[0])          # untimed warm-up step
+        t0 = time.perf_counter()
+        Ko, Vo = o.decode(*qkv[1])
+        orc.attention(qkv[1][0], Ko, Vo, torch.float32)
+        cpu_s = time.perf_counter() - t0
+        cpu = {"value": round(cpu_s * 1e6, 1), "unit": "us/layer-step (cache path only)", "cores": threads, "kind": "port",
+               "sample": f"one decode step of layer 0's cache path at batch {a.batch} continued from the GPU state "
+                         f"(stand-in q, k, v); compare with cache_path_us_per_layer_step"}
     out = {"metric": "lrqk_decoder_tokens_per_s", "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1,
            "steps": n_dec, "warmup": 0, "ms_per_step": round(t_decode / n_dec * 1e3, 3), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
            "config": {"workload": f"llama3_8b_shape_decoder@{a.prompt}", "layers": cfg.layers, "batch": a.batch,
                       "prompt_tokens": a.prompt, "new_tokens": a.new_tokens, "r": 32, "k": 2048, "lite": 64,
+                      "context_scale": a.context_scale,
                       "max_iter": [2, 2]},
            "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3), "setup_s": round(setup_s, 2),
            "reference_style_tokens_per_s": round(a.batch * len(steps) / max(sum(steps), 1e-9), 2),
            "us_per_layer_step": round(t_decode / n_dec / cfg.layers * 1e6, 1),
            "last_step_hit_rate": round(1.0 - miss / max(sel, 1), 4),
-           "roofline": None, "cpu_baseline": None}
+           "context_scale": a.context_scale,
+           "cache_path_us_per_layer_step": round(path_us, 1),
+           "other_us_per_layer_step": round(t_extra / cfg.layers * 1e6 - path_us, 1),
+           "roofline": None, "cpu_baseline": cpu}
     print(json.dumps(out))
 
 

@@ -49,9 +49,15 @@ def _rms(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
 
 class LlamaShapeDecoder:
     def __init__(self, cfg: DecoderConfig = LLAMA3_8B, dtype=torch.bfloat16, device="cuda:0", seed: int = 0,
-                 mlp_chunk: int = 16384):
+                 mlp_chunk: int = 16384, context_scale: float = 0.0):
+        """``context_scale`` > 0 adds a fixed direction of that length (in units of an embedding's length) to every
+        token embedding.  With random weights and random ids the hidden states of successive positions are
+        unrelated, so every decode step selects a fresh set of tokens; a shared component makes successive
+        queries (and all keys) correlated, as the residual stream of a trained model does, and the selection then
+        drifts slowly from step to step -- the regime the cache is built for."""
         self.cfg, self.dtype, self.device = cfg, dtype, torch.device(device)
         self.mlp_chunk = mlp_chunk
+        self.context_scale = context_scale
         g = torch.Generator(device=self.device).manual_seed(seed)
 
         def w(*shape, std=0.02):
@@ -59,6 +65,8 @@ class LlamaShapeDecoder:
 
         c = cfg
         self.embed = w(c.vocab, c.hidden)
+        ctx = torch.randn((c.hidden,), generator=g, device=self.device, dtype=torch.float32)
+        self.context = (ctx / ctx.norm() * (0.02 * math.sqrt(c.hidden)) * context_scale).to(dtype)
         self.lm_head = w(c.hidden, c.vocab)
         self.final_norm = torch.ones(c.hidden, dtype=dtype, device=self.device)
         self.layers = []
@@ -74,6 +82,7 @@ class LlamaShapeDecoder:
         self.ws = ops.Workspace()
         self.dense: Optional[List[Tuple[torch.Tensor, torch.Tensor]]] = None
         self.progress = None   # optional callable(str), called once per layer while the prompt is processed
+        self.path_events = None  # a list: decode steps append an event pair around each layer's cache path
 
     # ------------------------------------------------------------------ pieces
     def _rope(self, x: torch.Tensor, pos0: int) -> torch.Tensor:
@@ -105,6 +114,8 @@ class LlamaShapeDecoder:
         c = self.cfg
         b, s = ids.shape
         x = self.embed[ids]
+        if self.context_scale:
+            x = x + self.context
         if cache is None and self.dense is None:
             self.dense = [None] * c.layers
         for li, L in enumerate(self.layers):
@@ -127,11 +138,18 @@ class LlamaShapeDecoder:
                 eng = cache.lwattn[li]
                 eng.attn_in_step = True
                 eng.last_attn = None
+                if self.path_events is not None:
+                    e0 = torch.cuda.Event(enable_timing=True)
+                    e0.record()
                 K, V = cache.update(q, k, v, li)
                 if eng.last_attn is not None:
                     o = eng.last_attn
                 else:   # prefix / edge branches return a view of the first n slots of the persistent buffers
                     o = ops.attention(self.ws, q, eng.Kgpu, eng.Vgpu, n_valid=K.shape[2])
+                if self.path_events is not None:
+                    e1 = torch.cuda.Event(enable_timing=True)
+                    e1.record()
+                    self.path_events.append((e0, e1))
             x = x + o.transpose(1, 2).reshape(b, s, c.heads * c.head_dim) @ L["wo"]
             x = x + self._mlp(L, _rms(x, L["n2"], c.rms_eps))
             if s > 1 and self.progress is not None:
