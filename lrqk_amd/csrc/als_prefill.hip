@@ -539,7 +539,9 @@ __device__ __forceinline__ bf16x8 pf_bf16x8(uint32_t a, uint32_t b, uint32_t c, 
 
 // GRAMS = false: only A <- X Mt^T (the last pass of the iteration on Gram matrices, which needs neither the sums
 // over the new rows nor their change): the old rows are not read and nothing is reduced.
-template <int NB, int NW, bool GRAMS = true>
+// GIVEN = true: only the sums over the given rows of A (Mt must be null); the rows of A are requested one tile
+// ahead, like the rows of X.
+template <int NB, int NW, bool GRAMS = true, bool GIVEN = false>
 __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* __restrict__ X, int xh, int hq,
                                                                   int64_t l, int r, int d,
                                                                   const float* __restrict__ Mt, float* __restrict__ A,
@@ -547,7 +549,9 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
                                                                   float* __restrict__ delta_part,
                                                                   const int* __restrict__ done_flag, int S) {
   if (done_flag && *done_flag) return;
-  constexpr int LDB = 32 * NB + 8;  // row stride of a bf16 tile (elements)
+  // row stride of a bf16 tile (elements): 16-byte operand reads want rows 4 banks apart, the transposing reads of
+  // the GIVEN form 8 banks
+  constexpr int LDB = 32 * NB + (GIVEN ? 16 : 8);
   constexpr int KB = 2 * NB;        // 16-column blocks of X
   constexpr int VEC = 8;
   constexpr int NL = 32 * 32 * NB / (kWave * VEC);
@@ -563,7 +567,7 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
   const int64_t xhead = (int64_t)b * xh + head / (hq / xh);
   const bf16_t* Xh = X + xhead * l * d;
   float* Ah = A + (int64_t)h * l * r;
-  const bool apply = Mt != nullptr;
+  const bool apply = !GIVEN && Mt != nullptr;
   const bool full_rows = d == 32 * NB;
 
   if (apply) {
@@ -617,7 +621,20 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       pre[i] = *reinterpret_cast<const uint4*>(Xh + base + (e < nvalid ? e : 0));
     }
   };
-  if (r0 + (int64_t)wave * 32 < r1) issue(r0 + (int64_t)wave * 32);
+  float old_next[GIVEN ? 16 : 1];
+  auto issue_old = [&](int64_t t0) {
+    if constexpr (GIVEN) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
+        old_next[v] = Ah[rr * r + min(col, r - 1)];
+      }
+    }
+  };
+  if (r0 + (int64_t)wave * 32 < r1) {
+    issue(r0 + (int64_t)wave * 32);
+    issue_old(r0 + (int64_t)wave * 32);
+  }
   __syncthreads();  // Mt staged, tiles cleared
 
   for (int64_t t0 = r0 + (int64_t)wave * 32; t0 < r1; t0 += 32 * NW) {
@@ -635,11 +652,17 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       }
     }
     pf_wave_sync();
-    if (t0 + 32 * NW < r1) issue(t0 + 32 * NW);
-
     floatx16 c;
     float old[16];
-    if constexpr (GRAMS) {
+    if constexpr (GIVEN) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) old[v] = old_next[v];
+    }
+    if (t0 + 32 * NW < r1) {
+      issue(t0 + 32 * NW);
+      issue_old(t0 + 32 * NW);
+    }
+    if constexpr (GRAMS && !GIVEN) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int64_t rr = min(t0 + pf_mfma_row(lane, v), l - 1);
@@ -722,18 +745,34 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
     // xb[kb] = this lane's eight rows of k block kb, column 32 nb + col -- then its Gram products
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      floatx16 xa;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) xa[v] = 0.0f;
-      xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb), ident[0], xa, 0, 0, 0);
-      xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb + 1), ident[1], xa, 0, 0, 0);
       bf16x8 xb[2];
+      if constexpr (GIVEN) {
+        // the transposing LDS read hands a lane four successive rows of its column (within 16 lanes, lane s points
+        // at row s / 4, columns 4 (s % 4) .. + 3, and lane t receives column t of the four rows): rows
+        // 16 kb + 4 half .. + 3 and the same + 8, the order of the accumulator layout
+        typedef short v4s __attribute__((ext_vector_type(4)));
+        typedef v4s __attribute__((address_space(3))) * lds_v4s;
+        const int s16 = lane & 15;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-        xb[kb] = pf_bf16x8(pf_pack2(__float_as_uint(xa[8 * kb + 0]), __float_as_uint(xa[8 * kb + 1])),
-                           pf_pack2(__float_as_uint(xa[8 * kb + 2]), __float_as_uint(xa[8 * kb + 3])),
-                           pf_pack2(__float_as_uint(xa[8 * kb + 4]), __float_as_uint(xa[8 * kb + 5])),
-                           pf_pack2(__float_as_uint(xa[8 * kb + 6]), __float_as_uint(xa[8 * kb + 7])));
+        for (int kb = 0; kb < 2; ++kb) {
+          const uint16_t* p = &x_s[(16 * kb + 4 * half + (s16 >> 2)) * LDB + 32 * nb + (col & 16) + 4 * (s16 & 3)];
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)p);
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(p + 8 * LDB));
+          xb[kb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      } else {
+        floatx16 xa;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) xa[v] = 0.0f;
+        xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb), ident[0], xa, 0, 0, 0);
+        xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb + 1), ident[1], xa, 0, 0, 0);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+          xb[kb] = pf_bf16x8(pf_pack2(__float_as_uint(xa[8 * kb + 0]), __float_as_uint(xa[8 * kb + 1])),
+                             pf_pack2(__float_as_uint(xa[8 * kb + 2]), __float_as_uint(xa[8 * kb + 3])),
+                             pf_pack2(__float_as_uint(xa[8 * kb + 4]), __float_as_uint(xa[8 * kb + 5])),
+                             pf_pack2(__float_as_uint(xa[8 * kb + 6]), __float_as_uint(xa[8 * kb + 7])));
+      }
       floatx16 t;
 #pragma unroll
       for (int v = 0; v < 16; ++v) t[v] = 0.0f;
@@ -1008,7 +1047,7 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
     if constexpr (sizeof(T) == 2) {
       if (nb <= 4) {  // bf16 input: the pass on the bf16 matrix cores (three-piece split, fp32 accuracy)
         pass = nb == 1 ? pf_pass_bf16_kernel<1, 8> : nb == 2 ? pf_pass_bf16_kernel<2, 8> : pf_pass_bf16_kernel<4, 8>;
-        smem_pass = std::max((size_t)(8 + 3) * 32 * (32 * nb + 8) * sizeof(uint16_t), (size_t)8 * 1024 * sizeof(float));
+        smem_pass = std::max((size_t)(8 + 3) * 32 * (32 * nb + 16) * sizeof(uint16_t), (size_t)8 * 1024 * sizeof(float));
       }
     }
   }
@@ -1023,9 +1062,17 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   const dim3 grid((unsigned)S, (unsigned)bh), blk((unsigned)pass_threads), sblk(small32 ? kPfSmallThreads : kPfThreads);
   const T* Q = (const T*)q;
   const T* K = (const T*)k;
-  hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
+  PfPassFn<T> first = pass;  // the sums over the given initial factors
+  if constexpr (sizeof(T) == 2) {
+    if (mfma && d == 128) {
+      first = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, true, true>;
+      if (smem_pass > 48 * 1024)
+        LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)first, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
+    }
+  }
+  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
                      (float*)nullptr, (const int*)nullptr, S);
-  hipLaunchKernelGGL(pass, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
+  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
                      (float*)nullptr, (const int*)nullptr, S);
   LRQK_HIP_CHECK(hipGetLastError());
   if constexpr (sizeof(T) == 2) {
