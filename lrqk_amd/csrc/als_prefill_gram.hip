@@ -121,103 +121,203 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
   }
 }
 
-// S64[x][e] = sum over splits of part[x][s][e], in fp64
-__global__ __launch_bounds__(256) void pf_xtx_reduce_kernel(const float* __restrict__ part, int S, int n,
-                                                            double* __restrict__ out) {
-  const int x = blockIdx.y;
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= n) return;
-  double v = 0.0;
-  for (int s = 0; s < S; ++s) v += (double)part[((int64_t)x * S + s) * n + e];
-  out[(int64_t)x * n + e] = v;
-}
-
 // ----------------------------------------------------------------------------- d x d algebra, fp64
-constexpr int kGdThreads = 320;   // two groups of 32 + 128 threads: one column of [W | RHS] each
-constexpr int kGdGroup = 160;
+constexpr int kGdThreads = 256;   // four waves: 32 of the 128 right-hand columns each (one wave per SIMD: 512 registers)
 constexpr int kGdD = 128;
 constexpr int kGdLd = 34;         // doubles per row of a transposed r x d matrix in LDS ([d][34], 16-byte rows)
 constexpr int kGdLg = 33;         // doubles per row of an r x r matrix in LDS
 
-// Gauss-Jordan elimination of [W | RHS] (W 32 x 32 symmetric positive definite, rows/columns beyond r
-// the identity), one column per thread of a group, the column in registers, two pivots per step: the owners of
-// columns p, p + 1 publish them, every thread inverts the 2 x 2 pivot block itself (positive definite, no
-// pivoting needed) and applies the rank-two update to its column.  One barrier per step: the two LDS buffers
-// are used in turn, and a buffer is rewritten two steps later, when the barrier in between has every thread
-// past its reads.  The pivot rows of a step sit at fixed register positions (0..3 for the two steps of the loop
-// body, then the column is rotated by four), so every register index is static and the loop stays rolled.
-// piv: 128 doubles of LDS per group.  Every thread of the workgroup calls this; `col` is the thread's column in
-// its group (< 0: the thread only keeps the barriers).
-__device__ __forceinline__ void gd_solve(double (&x)[32], int col, double* __restrict__ piv) {
-  for (int pb = 0; pb < 32; pb += 4) {
-#pragma unroll
-    for (int q = 0; q < 4; q += 2) {
-      double* pv = piv + (q >> 1) * 64;  // [2][32]: columns p and p + 1
-      const int p = pb + q;
-      if (col == p || col == p + 1) {
-        double* mine = pv + (col - p) * 32;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) mine[i] = x[i];
-      }
-      __syncthreads();
-      if (col >= 0) {  // (wave-uniform but for the last wave of a group: idle threads stay off the LDS)
-        // the two columns as 16-byte reads
-        double c0[32], c1[32];
-#pragma unroll
-        for (int i = 0; i < 32; i += 2) {
-          const double2 u0 = *reinterpret_cast<const double2*>(pv + i);
-          const double2 u1 = *reinterpret_cast<const double2*>(pv + 32 + i);
-          c0[i] = u0.x;
-          c0[i + 1] = u0.y;
-          c1[i] = u1.x;
-          c1[i + 1] = u1.y;
-        }
-        // inverse of the pivot block [[a, b], [b', c]] (rows q, q + 1 of the two columns)
-        const double a = c0[q], bb = c1[q], b2 = c0[q + 1], c = c1[q + 1];
-        const double det = fma(a, c, -bb * b2);
-        double inv = __builtin_amdgcn_rcp(det);
-        inv = fma(fma(-det, inv, 1.0), inv, inv);
-        inv = fma(fma(-det, inv, 1.0), inv, inv);
-        const double xa = (c * x[q] - bb * x[q + 1]) * inv;
-        const double xb = (a * x[q + 1] - b2 * x[q]) * inv;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-          if (i != q && i != q + 1) x[i] = fma(-c0[i], xa, fma(-c1[i], xb, x[i]));
-        }
-        x[q] = xa;
-        x[q + 1] = xb;
-      }
-    }
-    // rotate by four: the next pivot rows move to positions 0..3
-    const double t0 = x[0], t1 = x[1], t2 = x[2], t3 = x[3];
-#pragma unroll
-    for (int i = 0; i < 28; ++i) x[i] = x[i + 4];
-    x[28] = t0;
-    x[29] = t1;
-    x[30] = t2;
-    x[31] = t3;
-  }
-  __syncthreads();
+// ---- two systems [W | RHS] (W 32 x 32 symmetric positive definite up to rounding, rows/columns beyond r the
+// identity; RHS 32 x 128) solved side by side by block Gauss-Jordan elimination on the fp64 matrix cores, four
+// pivots per step.  The matrices live in the accumulator layout of 16 x 16 tiles (element v of lane l = row
+// 16 rt + l / 16 + 4 v, column 16 u + l % 16 of tile (rt, u)): each of the four waves holds W itself (every wave
+// eliminates its own copy: no wave waits for another, the solve has no barrier) and 32 columns of RHS.
+// Step m, with P the pivot columns 4 m .. 4 m + 3 (32 x 4) and D its rows 4 m .. 4 m + 3:
+//     X <- X - ((P - E) D^-1) X[4 m .. 4 m + 3, :]        (E: the identity in the pivot rows)
+// which leaves D^-1 X[pivot rows] in the pivot rows and clears the pivot columns elsewhere.  The right-hand
+// operand, four rows of X, is element m % 4 of the lane's own tile in row tile m / 4: no data moves for it.  The
+// left operand needs P by rows: the lanes that hold the pivot columns put them into the wave's own LDS slot, the
+// two pivot blocks are inverted side by side in the two halves of the wave (by 2 x 2 blocks, no pivoting) and
+// handed round through the same slot.  The products on W come first (the next step waits for them only); those on
+// RHS run on the matrix cores while the next step's inverse is computed.
+typedef double gd_v4d __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void gd_wave_sync() {  // orders one wave's LDS writes and reads
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// out[i][j] (+)= sum over c < 128 of PT[c][i] * RT[c][j]   (two r x d matrices, stored transposed), by threads
-// 0..255: thread (i = tid / 8, j = 4 (tid % 8) .. + 3).  Rows/columns beyond r come out as what the zero
-// padding of PT, RT gives.
-__device__ __forceinline__ void gd_outer(const double* __restrict__ PT, const double* __restrict__ RT, double (&o)[4]) {
-  const int tid = threadIdx.x;
-  const int i = tid >> 3, j0 = (tid & 7) * 4;
-  o[0] = o[1] = o[2] = o[3] = 0.0;
-  if (tid < 256) {
-#pragma unroll 4
-    for (int c = 0; c < kGdD; ++c) {
-      const double p = PT[c * kGdLd + i];
-      const double2 ra = *reinterpret_cast<const double2*>(&RT[c * kGdLd + j0]);
-      const double2 rb = *reinterpret_cast<const double2*>(&RT[c * kGdLd + j0 + 2]);
-      o[0] = fma(p, ra.x, o[0]);
-      o[1] = fma(p, ra.y, o[1]);
-      o[2] = fma(p, rb.x, o[2]);
-      o[3] = fma(p, rb.y, o[3]);
+__device__ __forceinline__ double gd_rcp(double x) {
+  double inv = __builtin_amdgcn_rcp(x);
+  inv = fma(fma(-x, inv, 1.0), inv, inv);
+  return fma(fma(-x, inv, 1.0), inv, inv);
+}
+
+// R = D^-1 for a 4 x 4 matrix with positive definite symmetric part, by 2 x 2 blocks (no pivoting):
+// D = [[A, B], [C, E]], S = E - C A^-1 B, D^-1 = [[A^-1 + Y S^-1 Z, -Y S^-1], [-S^-1 Z, S^-1]], Y = A^-1 B, Z = C A^-1.
+// D is taken as it is, not as symmetric: the Gram sums it comes from are symmetric only up to their rounding, and
+// the elimination around it uses both triangles.
+__device__ __forceinline__ void gd_inv4(const double (&D)[4][4], double (&R)[4][4]) {
+  const double ia = gd_rcp(fma(D[0][0], D[1][1], -D[0][1] * D[1][0]));
+  const double a00 = D[1][1] * ia, a01 = -D[0][1] * ia, a10 = -D[1][0] * ia, a11 = D[0][0] * ia;  // A^-1
+  // Y = A^-1 B  (B = D[0..1][2..3]),  Z = C A^-1  (C = D[2..3][0..1])
+  const double y00 = fma(a00, D[0][2], a01 * D[1][2]), y01 = fma(a00, D[0][3], a01 * D[1][3]);
+  const double y10 = fma(a10, D[0][2], a11 * D[1][2]), y11 = fma(a10, D[0][3], a11 * D[1][3]);
+  const double z00 = fma(D[2][0], a00, D[2][1] * a10), z01 = fma(D[2][0], a01, D[2][1] * a11);
+  const double z10 = fma(D[3][0], a00, D[3][1] * a10), z11 = fma(D[3][0], a01, D[3][1] * a11);
+  // S = E - C Y
+  const double s00 = D[2][2] - fma(D[2][0], y00, D[2][1] * y10), s01 = D[2][3] - fma(D[2][0], y01, D[2][1] * y11);
+  const double s10 = D[3][2] - fma(D[3][0], y00, D[3][1] * y10), s11 = D[3][3] - fma(D[3][0], y01, D[3][1] * y11);
+  const double is = gd_rcp(fma(s00, s11, -s01 * s10));
+  const double t00 = s11 * is, t01 = -s01 * is, t10 = -s10 * is, t11 = s00 * is;  // S^-1
+  // U = Y S^-1 (upper right, negated), V = S^-1 Z (lower left, negated)
+  const double u00 = fma(y00, t00, y01 * t10), u01 = fma(y00, t01, y01 * t11);
+  const double u10 = fma(y10, t00, y11 * t10), u11 = fma(y10, t01, y11 * t11);
+  const double v00 = fma(t00, z00, t01 * z10), v01 = fma(t00, z01, t01 * z11);
+  const double v10 = fma(t10, z00, t11 * z10), v11 = fma(t10, z01, t11 * z11);
+  R[0][0] = a00 + fma(u00, z00, u01 * z10);
+  R[0][1] = a01 + fma(u00, z01, u01 * z11);
+  R[1][0] = a10 + fma(u10, z00, u11 * z10);
+  R[1][1] = a11 + fma(u10, z01, u11 * z11);
+  R[0][2] = -u00; R[0][3] = -u01; R[1][2] = -u10; R[1][3] = -u11;
+  R[2][0] = -v00; R[2][1] = -v01; R[3][0] = -v10; R[3][1] = -v11;
+  R[2][2] = t00; R[2][3] = t01; R[3][2] = t10; R[3][3] = t11;
+}
+
+struct GdSys {
+  gd_v4d w[2][2];  // W: [row tile][column tile]
+  gd_v4d x[2][2];  // this wave's columns of RHS: [row tile][column tile 2 wave + u]
+};
+constexpr int kGdSlot = 2 * 128 + 32;                    // per wave: P of both systems, the two inverses
+constexpr int kGdPivDoubles = (kGdThreads / 64) * kGdSlot;
+__device__ __forceinline__ void gd_solve_pair(GdSys (&s)[2], double* __restrict__ piv) {
+  const int lane = lane_id(), wave = wave_id();
+  const int li = lane & 15, lk = lane >> 4;
+  double* pb = piv + wave * kGdSlot;
+  double* xch = pb + 256;
+#pragma unroll
+  for (int m = 0; m < 8; ++m) {
+    const int tp = m >> 2, vp = m & 3;  // the pivots' tile (row tile of the pivot rows, column tile of W) and element
+    {
+      const int kk = li - 4 * vp;
+      if (kk >= 0 && kk < 4) {
+#pragma unroll
+        for (int sy = 0; sy < 2; ++sy)
+#pragma unroll
+          for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pb[sy * 128 + (16 * rt + lk + 4 * v) * 4 + kk] = s[sy].w[rt][tp][v];
+      }
     }
+    gd_wave_sync();
+    {
+      const int mine = lane >> 5;
+      const double* P = pb + mine * 128;
+      double D[4][4], R[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const double2 lo = *reinterpret_cast<const double2*>(&P[(4 * m + i) * 4]);
+        const double2 hi = *reinterpret_cast<const double2*>(&P[(4 * m + i) * 4 + 2]);
+        D[i][0] = lo.x; D[i][1] = lo.y; D[i][2] = hi.x; D[i][3] = hi.y;
+      }
+      gd_inv4(D, R);
+      if ((lane & 31) == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          *reinterpret_cast<double2*>(&xch[mine * 16 + i * 4]) = make_double2(R[i][0], R[i][1]);
+          *reinterpret_cast<double2*>(&xch[mine * 16 + i * 4 + 2]) = make_double2(R[i][2], R[i][3]);
+        }
+      }
+      gd_wave_sync();
+    }
+    double aop[2][2];
+#pragma unroll
+    for (int sy = 0; sy < 2; ++sy) {
+      const double* P = pb + sy * 128;
+      double ic[4];  // column l / 16 of the inverse
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ic[k] = xch[sy * 16 + k * 4 + lk];
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        const int row = 16 * rt + li;
+        const double2 lo = *reinterpret_cast<const double2*>(&P[row * 4]);
+        const double2 hi = *reinterpret_cast<const double2*>(&P[row * 4 + 2]);
+        const double m0 = lo.x - (row == 4 * m ? 1.0 : 0.0), m1 = lo.y - (row == 4 * m + 1 ? 1.0 : 0.0);
+        const double m2 = hi.x - (row == 4 * m + 2 ? 1.0 : 0.0), m3 = hi.y - (row == 4 * m + 3 ? 1.0 : 0.0);
+        aop[sy][rt] = -fma(m0, ic[0], fma(m1, ic[1], fma(m2, ic[2], m3 * ic[3])));
+      }
+    }
+    gd_wave_sync();  // (the reads of the slot precede the next step's writes)
+    // W: the column tiles from the pivots' on (those before hold finished unit columns: zero in the pivot rows)
+#pragma unroll
+    for (int sy = 0; sy < 2; ++sy)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (u < tp) continue;
+        const double bop = s[sy].w[tp][u][vp];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+          s[sy].w[rt][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(aop[sy][rt], bop, s[sy].w[rt][u], 0, 0, 0);
+      }
+#pragma unroll
+    for (int sy = 0; sy < 2; ++sy)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const double bop = s[sy].x[tp][u][vp];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+          s[sy].x[rt][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(aop[sy][rt], bop, s[sy].x[rt][u], 0, 0, 0);
+      }
+  }
+}
+
+// One system filled from fw(row, column of W) and fx(row, column of RHS) / its solution handed to g(row, column
+// of RHS, value).
+template <typename FW, typename FX>
+__device__ __forceinline__ void gd_fill(GdSys& t, FW&& fw, FX&& fx) {
+  const int lane = lane_id(), wave = wave_id();
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int i = 16 * rt + (lane >> 4) + 4 * v;
+        t.w[rt][u][v] = fw(i, 16 * u + (lane & 15));
+        t.x[rt][u][v] = fx(i, 16 * (2 * wave + u) + (lane & 15));
+      }
+}
+template <typename G>
+__device__ __forceinline__ void gd_drain(const gd_v4d (&x)[2][2], G&& g) {
+  const int lane = lane_id(), wave = wave_id();
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) g(16 * rt + (lane >> 4) + 4 * v, 16 * (2 * wave + u) + (lane & 15), x[rt][u][v]);
+}
+
+// out[i][j] = sum over c < 128 of PT[c][i] * RT[c][j]   (two r x d matrices, stored transposed) on the fp64 matrix
+// cores, by waves 0..3: wave w owns the 16 x 16 tile (w / 2, w % 2) and runs its 32 products of depth 4 in a row.
+// Element v of a thread is out[gd_outer_row(v)][gd_outer_col()].  Rows/columns beyond r come out as what the zero
+// padding of PT, RT gives.
+__device__ __forceinline__ int gd_outer_row(int v) { return 16 * (wave_id() >> 1) + (lane_id() >> 4) + 4 * v; }
+__device__ __forceinline__ int gd_outer_col() { return 16 * (wave_id() & 1) + (lane_id() & 15); }
+__device__ __forceinline__ void gd_outer(const double* __restrict__ PT, const double* __restrict__ RT, double (&o)[4]) {
+  o[0] = o[1] = o[2] = o[3] = 0.0;
+  if (threadIdx.x < 256) {
+    const int lane = lane_id(), wave = wave_id();
+    const int li = lane & 15, lk = lane >> 4;
+    const double* pa = PT + lk * kGdLd + 16 * (wave >> 1) + li;
+    const double* pb = RT + lk * kGdLd + 16 * (wave & 1) + li;
+    gd_v4d acc = gd_v4d{0.0, 0.0, 0.0, 0.0};
+#pragma unroll 8
+    for (int c = 0; c < kGdD; c += 4)
+      acc = __builtin_amdgcn_mfma_f64_16x16x4f64(pa[c * kGdLd], pb[c * kGdLd], acc, 0, 0, 0);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) o[v] = acc[v];
   }
 }
 
@@ -226,7 +326,6 @@ __device__ __forceinline__ void gd_outer(const double* __restrict__ PT, const do
 // LDS copy), B operand lane l = S[k0 + l / 16][c0 + l % 16] (16 independent loads per lane in flight), result
 // element v of lane l = row l / 16 + 4 v, column l % 16 of the tile.  Waves 0..3 take 32 columns each.
 // One barrier.
-typedef double gd_v4d __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void gd_times_s(const double* __restrict__ MT, const double* __restrict__ S,
                                            double* __restrict__ TT) {
   const int lane = lane_id(), wave = wave_id();
@@ -284,6 +383,7 @@ struct GdArgs {
   const double* Sk;     // [b * hkv][d][d]
   double* G;            // [2][bh][32][32]  (side 0: Q, 1: K), padded with the identity
   double* C;            // [2][bh][32][d]   zero rows beyond r
+  double* BqT;          // [bh][d][32]      B_Q of the state, transposed (written by an iteration for the next)
   double* delta;        // [iters][2][bh]   squared changes |A - A'|^2 per head
   int* flags;           // [iters + 1]
   float* Mt_q;          // [bh][r][d]  Mq^T, Mk^T for the final row-by-row pass
@@ -295,12 +395,35 @@ struct GdArgs {
   float tol;
 };
 
-// The state (G, C) of both sides from the first Gram passes: S partial sums of [G | C] packed as [r][r + d]
-// floats per head, added in fp64; G padded with the identity, C with zero rows.  grid (ceil(32 * 160 / 256), bh, 2).
-__global__ __launch_bounds__(256) void pf_gramdom_init_kernel(GdArgs a) {
-  const int h = blockIdx.y, side = blockIdx.z;
+// One launch for everything that only adds partial sums up, in fp64:
+//   blocks [0, nq)        Sq[x][e] = sum over the Sx splits of xq_part[x][s][e]   (nq = bh * d * d / 256)
+//   blocks [nq, nq + nk)  Sk likewise over the bkv distinct K heads
+//   the rest              the state (G, C) of both sides from the first Gram passes: S partial sums of [G | C]
+//                         packed as [r][r + d] floats per head; G padded with the identity, C with zero rows
+//                         (20 blocks per head and side).
+constexpr int kGdInitBlocks = (32 * (32 + kGdD) + 255) / 256;
+__global__ __launch_bounds__(256) void pf_gramdom_init_kernel(GdArgs a, const float* __restrict__ xq_part, int Sx,
+                                                              const float* __restrict__ xk_part, int Sxk, int bkv,
+                                                              double* __restrict__ Sq, double* __restrict__ Sk) {
+  constexpr int dd = kGdD * kGdD, per = dd / 256;
+  int blk = blockIdx.x;
+  const int nq = a.bh * per, nk = bkv * per;
+  if (blk < nq + nk) {
+    const bool k_side = blk >= nq;
+    if (k_side) blk -= nq;
+    const int x = blk / per, e = (blk % per) * 256 + threadIdx.x;
+    const int S = k_side ? Sxk : Sx;
+    const float* part = (k_side ? xk_part : xq_part) + (int64_t)x * S * dd + e;
+    double v = 0.0;
+#pragma unroll 4
+    for (int s = 0; s < S; ++s) v += (double)part[(int64_t)s * dd];
+    (k_side ? Sk : Sq)[(int64_t)x * dd + e] = v;
+    return;
+  }
+  blk -= nq + nk;
+  const int h = blk / (2 * kGdInitBlocks), side = (blk / kGdInitBlocks) & 1;
   const int r = a.r, d = kGdD;
-  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int e = (blk % kGdInitBlocks) * 256 + threadIdx.x;
   if (e >= 32 * (32 + d)) return;
   const int ne = r * (r + d);
   const float* part = (side ? a.partK : a.partQ) + (int64_t)h * a.S * ne;
@@ -325,14 +448,11 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   double* TT = MT + kGdD * kGdLd;           // [128][34]  T, later U
   double* BT = TT + kGdD * kGdLd;           // [128][34]  B_Q, later B_K
   double* Gs = BT + kGdD * kGdLd;           // [3][32][33]
-  double* piv = Gs + 3 * 32 * kGdLg;        // [2 groups][2][2][32]
-  double* red = piv + 256;                  // [8]
+  double* piv = Gs + 3 * 32 * kGdLg;        // [2 buffers][2 systems][32][4]
+  double* red = piv + kGdPivDoubles;        // [8]
   const int tid = threadIdx.x;
   const int h = blockIdx.x;
   const int r = a.r, d = kGdD, bh = a.bh;
-  const int grp = tid >= kGdGroup ? 1 : 0;     // 0: the Q side's system, 1: the K side's
-  const int t = tid - grp * kGdGroup;          // column of [W | RHS] within the group
-  const int c = t - 32;                        // RHS column (valid when t >= 32)
   const int b = h / a.hq, kvh = (h % a.hq) / (a.hq / a.hkv);
   const double* Sq = a.Sq + (int64_t)h * d * d;
   const double* Sk = a.Sk + ((int64_t)b * a.hkv + kvh) * d * d;
@@ -364,80 +484,74 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     if (done) return;
   }
 
-  // ---- B_Q = Gq^-1 Cq and B_K = Gk^-1 Ck, side by side
-  double x[32];
-  {
-    const double* G = grp ? Gk : Gq;
-    const double* C = grp ? Ck : Cq;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) x[i] = t < 32 ? G[i * 32 + t] : C[i * d + c];
-  }
-  gd_solve(x, t, piv + 128 * grp);
-  if (stage == 2) {
-    if (t >= 32) {
-      float* out = (grp ? a.b_k : a.b_q) + (int64_t)h * r * d;
-#pragma unroll
-      for (int i = 0; i < 32; ++i)
-        if (i < r) out[i * d + c] = (float)x[i];
+  // Of an iteration's r x r systems only two follow each other: B_K = Gk^-1 Ck does not depend on the Q side's
+  // step and is solved beside it, and the next iteration's B_Q = Gq'^-1 Cq' is solved beside the K side's step
+  // and handed over in `BqT`.  Iteration 0 (and the final stage) start from the state alone: B_Q and B_K side by side.
+  GdSys sy[2];
+  gd_v4d bk[2][2];  // B_K in the layout of the right-hand sides
+  double* BqT = a.BqT + (int64_t)h * 32 * d;  // [32][d]
+  const bool fresh = stage == 2 || it == 0;
+  if (fresh) {
+    gd_fill(sy[0], [&](int i, int j) { return Gq[i * 32 + j]; }, [&](int i, int cc) { return Cq[i * d + cc]; });
+    if (stage == 2)
+      gd_fill(sy[1], [&](int i, int j) { return Gk[i * 32 + j]; }, [&](int i, int cc) { return Ck[i * d + cc]; });
+    else
+      gd_fill(sy[1], [&](int i, int j) { return i == j ? 1.0 : 0.0; }, [&](int, int) { return 0.0; });
+    gd_solve_pair(sy, piv);
+    if (stage == 2) {
+      float* oq = a.b_q + (int64_t)h * r * d;
+      float* ok = a.b_k + (int64_t)h * r * d;
+      gd_drain(sy[0].x, [&](int i, int cc, double v) { if (i < r) oq[i * d + cc] = (float)v; });
+      gd_drain(sy[1].x, [&](int i, int cc, double v) { if (i < r) ok[i * d + cc] = (float)v; });
+      return;
     }
-    return;
-  }
-  double bcol[32];  // this thread's column of B_Q (group 0) or B_K (group 1)
-#pragma unroll
-  for (int i = 0; i < 32; ++i) bcol[i] = x[i];
-  if (grp == 0 && t >= 32) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i) BT[c * kGdLd + i] = bcol[i];
+    gd_drain(sy[0].x, [&](int i, int cc, double v) { BT[cc * kGdLd + i] = v; });
+  } else {
+    for (int e = tid; e < 32 * d; e += kGdThreads) BT[(e % d) * kGdLd + e / d] = BqT[e];
   }
   __syncthreads();
   // ---- W1 = Gk + B_Q B_Q^T
   {
     double o[4];
     gd_outer(BT, BT, o);
-    if (tid < 256) {
-      const int i = tid >> 3, j0 = (tid & 7) * 4;
+    const int j = gd_outer_col();
 #pragma unroll
-      for (int u = 0; u < 4; ++u) Gs[i * kGdLg + j0 + u] = Gk[i * 32 + j0 + u] + o[u];
-    }
+    for (int u = 0; u < 4; ++u) Gs[gd_outer_row(u) * kGdLg + j] = Gk[gd_outer_row(u) * 32 + j] + o[u];
   }
   __syncthreads();
-  // ---- B_K B_K^T (the B tile now holds B_K)
-  if (grp == 1 && t >= 32) {
+  // ---- Mq'^T = W1^-1 (Ck + B_Q) beside B_K = Gk^-1 Ck
+  gd_fill(sy[0], [&](int i, int j) { return Gs[i * kGdLg + j]; },
+          [&](int i, int cc) { return Ck[i * d + cc] + BT[cc * kGdLd + i]; });
+  gd_fill(sy[1], [&](int i, int j) { return Gk[i * 32 + j]; }, [&](int i, int cc) { return Ck[i * d + cc]; });
+  __syncthreads();  // (every read of B_Q precedes the rewriting of the B tile below)
+  gd_solve_pair(sy, piv);
 #pragma unroll
-    for (int i = 0; i < 32; ++i) BT[c * kGdLd + i] = bcol[i];
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) bk[rt][u] = sy[1].x[rt][u];
+  // ---- the B tile now holds B_K; Mq'^T goes to its tile and to the caller, with the sum of Cq (the old one) . Mq'^T
+  gd_drain(bk, [&](int i, int cc, double v) { BT[cc * kGdLd + i] = v; });
+  double part_q = 0.0;
+  {
+    float* mt = a.Mt_q + (int64_t)h * r * d;
+    gd_drain(sy[0].x, [&](int i, int cc, double v) {
+      MT[cc * kGdLd + i] = v;
+      part_q = fma(Cq[i * d + cc], v, part_q);
+      if (i < r) mt[i * d + cc] = (float)v;
+    });
   }
+  double tr_old = 0.0;
+  if (tid < 32) tr_old = tid < r ? Gq[tid * 32 + tid] : 0.0;
   __syncthreads();
   {
     double o[4];
     gd_outer(BT, BT, o);
     if (tid < 256) {
-      const int i = tid >> 3, j0 = (tid & 7) * 4;
+      const int j = gd_outer_col();
 #pragma unroll
-      for (int u = 0; u < 4; ++u) Gs[32 * kGdLg + i * kGdLg + j0 + u] = o[u];
+      for (int u = 0; u < 4; ++u) Gs[32 * kGdLg + gd_outer_row(u) * kGdLg + j] = o[u];
     }
   }
-  // ---- Mq'^T = W1^-1 (Ck + B_Q)   (group 0; group 1 keeps the barriers)
-  if (grp == 0) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i) x[i] = t < 32 ? Gs[i * kGdLg + t] : Ck[i * d + c] + bcol[i];
-  }
-  __syncthreads();  // (W1 is read above from what the previous block wrote; B_K B_K^T is complete)
-  gd_solve(x, grp == 0 ? t : -1, piv);
-  double part_q = 0.0;  // sum of Cq (the old one) . Mq'^T over this thread's column
-  if (grp == 0 && t >= 32) {
-    float* mt = a.Mt_q + (int64_t)h * r * d;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      MT[c * kGdLd + i] = x[i];
-      part_q = fma(Cq[i * d + c], x[i], part_q);
-    }
-#pragma unroll
-    for (int i = 0; i < 32; ++i)
-      if (i < r) mt[i * d + c] = (float)x[i];
-  }
-  double tr_old = 0.0;
-  if (tid < 32) tr_old = tid < r ? Gq[tid * 32 + tid] : 0.0;
-  __syncthreads();
   // ---- T = Mq'^T Sq, Gq' = Mq'^T T^T
   gd_times_s(MT, Sq, TT);
   {
@@ -445,10 +559,10 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     gd_outer(MT, TT, o);
     double tr_new = 0.0;
     if (tid < 256) {
-      const int i = tid >> 3, j0 = (tid & 7) * 4;
+      const int j = gd_outer_col();
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int j = j0 + u;
+        const int i = gd_outer_row(u);
         const double v = (i < r && j < r) ? o[u] : (i == j ? 1.0 : 0.0);
         Gs[2 * 32 * kGdLg + i * kGdLg + j] = v;
         Gq[i * 32 + j] = v;
@@ -463,25 +577,29 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
 #pragma unroll
     for (int i = 0; i < 32; ++i) Cq[i * d + tid] = TT[tid * kGdLd + i];
   }
-  // ---- Mk'^T = (Gq' + B_K B_K^T)^-1 (T + B_K)   (group 1)
-  if (grp == 1) {
+  // ---- Mk'^T = (Gq' + B_K B_K^T)^-1 (T + B_K) beside the next B_Q = Gq'^-1 T
+  {
+    const double* Gn = Gs + 2 * 32 * kGdLg;
+    const double* Gb = Gs + 32 * kGdLg;
+    gd_fill(sy[0], [&](int i, int j) { return Gn[i * kGdLg + j]; }, [&](int i, int cc) { return TT[cc * kGdLd + i]; });
+    gd_fill(sy[1], [&](int i, int j) { return Gn[i * kGdLg + j] + Gb[i * kGdLg + j]; },
+            [&](int i, int cc) { return TT[cc * kGdLd + i]; });
 #pragma unroll
-    for (int i = 0; i < 32; ++i)
-      x[i] = t < 32 ? Gs[2 * 32 * kGdLg + i * kGdLg + t] + Gs[32 * kGdLg + i * kGdLg + t] : TT[c * kGdLd + i] + bcol[i];
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) sy[1].x[rt][u] += bk[rt][u];
   }
   __syncthreads();
-  gd_solve(x, grp == 1 ? t : -1, piv + 128);
+  gd_solve_pair(sy, piv);
+  gd_drain(sy[0].x, [&](int i, int cc, double v) { BqT[i * d + cc] = v; });
   double part_k = 0.0;
-  if (grp == 1 && t >= 32) {
+  {
     float* mt = a.Mt_k + (int64_t)h * r * d;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      MT[c * kGdLd + i] = x[i];
-      part_k = fma(Ck[i * d + c], x[i], part_k);
-    }
-#pragma unroll
-    for (int i = 0; i < 32; ++i)
-      if (i < r) mt[i * d + c] = (float)x[i];
+    gd_drain(sy[1].x, [&](int i, int cc, double v) {
+      MT[cc * kGdLd + i] = v;
+      part_k = fma(Ck[i * d + cc], v, part_k);
+      if (i < r) mt[i * d + cc] = (float)v;
+    });
   }
   double trk_old = 0.0;
   if (tid < 32) trk_old = tid < r ? Gk[tid * 32 + tid] : 0.0;
@@ -493,10 +611,10 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     gd_outer(MT, TT, o);
     double tr_new = 0.0;
     if (tid < 256) {
-      const int i = tid >> 3, j0 = (tid & 7) * 4;
+      const int j = gd_outer_col();
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int j = j0 + u;
+        const int i = gd_outer_row(u);
         const double v = (i < r && j < r) ? o[u] : (i == j ? 1.0 : 0.0);
         Gk[i * 32 + j] = v;
         if (i == j && i < r) tr_new += v;
@@ -517,6 +635,7 @@ static size_t gramdom_bytes(int bh, int bkv, int Sx, int Sxk, int iters) {
   return ((size_t)bh * Sx + (size_t)bkv * Sxk) * dd * sizeof(float)      // X^T X partial sums
          + ((size_t)bh + bkv) * dd * sizeof(double)                       // Sq, Sk
          + (size_t)2 * bh * (1024 + 32 * kGdD) * sizeof(double)           // G, C
+         + (size_t)bh * 32 * kGdD * sizeof(double)                        // B_Q handed from iteration to iteration
          + (size_t)std::max(iters, 1) * 2 * bh * sizeof(double)           // squared changes
          + (size_t)2 * bh * 32 * kGdD * sizeof(float) + 256;              // Mq^T, Mk^T
 }
@@ -540,6 +659,7 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
   double* Sk = (double*)p;                  p += (size_t)bkv * dd * sizeof(double);
   double* G = (double*)p;                   p += (size_t)2 * bh * 1024 * sizeof(double);
   double* C = (double*)p;                   p += (size_t)2 * bh * 32 * d * sizeof(double);
+  double* BqT = (double*)p;                 p += (size_t)bh * 32 * d * sizeof(double);
   double* delta = (double*)p;               p += (size_t)std::max(iters, 1) * 2 * bh * sizeof(double);
   float* Mtq = (float*)p;                   p += (size_t)bh * 32 * d * sizeof(float);
   float* Mtk = (float*)p;                   p += (size_t)bh * 32 * d * sizeof(float);
@@ -549,12 +669,8 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
                      xq_part, Sx);
   hipLaunchKernelGGL(pf_xtx_kernel, dim3((unsigned)Sxk, (unsigned)bkv), dim3(kXtxThreads), 0, st, (const bf16_t*)k, l,
                      xk_part, Sxk);
-  hipLaunchKernelGGL(pf_xtx_reduce_kernel, dim3((unsigned)((dd + 255) / 256), (unsigned)bh), dim3(256), 0, st,
-                     (const float*)xq_part, Sx, (int)dd, Sq);
-  hipLaunchKernelGGL(pf_xtx_reduce_kernel, dim3((unsigned)((dd + 255) / 256), (unsigned)bkv), dim3(256), 0, st,
-                     (const float*)xk_part, Sxk, (int)dd, Sk);
   LRQK_HIP_CHECK(hipGetLastError());
-  const size_t smem = ((size_t)3 * kGdD * kGdLd + 3 * 32 * kGdLg + 256 + 8) * sizeof(double);
+  const size_t smem = ((size_t)3 * kGdD * kGdLd + 3 * 32 * kGdLg + kGdPivDoubles + 8) * sizeof(double);
   static std::atomic<bool> attr_dev[kMaxDeviceSlots];
   std::atomic<bool>& attr = attr_dev[per_device_slot()];
   if (!attr) {
@@ -562,9 +678,10 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
                                        (int)smem));
     attr = true;
   }
-  GdArgs a{partQ, partK, S, Sq, Sk, G, C, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol};
-  hipLaunchKernelGGL(pf_gramdom_init_kernel, dim3((unsigned)((32 * (32 + kGdD) + 255) / 256), (unsigned)bh, 2u), dim3(256), 0,
-                     st, a);
+  GdArgs a{partQ, partK, S, Sq, Sk, G, C, BqT, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol};
+  const unsigned init_blocks = (unsigned)(((size_t)bh + bkv) * (dd / 256) + (size_t)2 * bh * kGdInitBlocks);
+  hipLaunchKernelGGL(pf_gramdom_init_kernel, dim3(init_blocks), dim3(256), 0, st, a, (const float*)xq_part, Sx,
+                     (const float*)xk_part, Sxk, bkv, Sq, Sk);
   for (int it = 0; it < iters; ++it)
     hipLaunchKernelGGL(pf_gramdom_kernel, dim3((unsigned)bh), dim3(kGdThreads), smem, st, 0, it, a);
   hipLaunchKernelGGL(pf_gramdom_kernel, dim3((unsigned)bh), dim3(kGdThreads), smem, st, 2, iters, a);
