@@ -148,9 +148,11 @@ __device__ __forceinline__ void gd_wave_sync() {  // orders one wave's LDS write
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// 1 / x to ~1e-14: the hardware estimate (2^-23) and one Newton step.  The pivot blocks' inverses need no more
+// (their error enters the solution once, scaled by the condition number, far below the rounding of the fp32 sums
+// the systems are built from), and every operation here is on the solve's dependent chain.
 __device__ __forceinline__ double gd_rcp(double x) {
-  double inv = __builtin_amdgcn_rcp(x);
-  inv = fma(fma(-x, inv, 1.0), inv, inv);
+  const double inv = __builtin_amdgcn_rcp(x);
   return fma(fma(-x, inv, 1.0), inv, inv);
 }
 
@@ -461,6 +463,30 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   double* Cq = a.C + (int64_t)h * 32 * d;
   double* Ck = a.C + ((int64_t)bh + h) * 32 * d;
 
+  // ---- what an iteration reads of its state is requested before anything else: the handed-over B_Q and this
+  // wave's tiles of Ck and Cq (Cq is rewritten only at the end of the Q side's step, Ck at the end of the iteration)
+  const bool fresh = stage == 2 || it == 0;
+  constexpr int kBqPer = 32 * kGdD / kGdThreads;
+  double bq_pre[kBqPer];
+  gd_v4d ckt[2][2], cqt[2][2];
+  if (!fresh) {
+    const double* src = a.BqT + (int64_t)h * 32 * d;  // [32][d]
+#pragma unroll
+    for (int u = 0; u < kBqPer; ++u) bq_pre[u] = src[tid + u * kGdThreads];
+  }
+  if (stage == 0) {
+    const int lane = lane_id(), wave = wave_id();
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int e = (16 * rt + (lane >> 4) + 4 * v) * d + 16 * (2 * wave + u) + (lane & 15);
+          ckt[rt][u][v] = Ck[e];
+          cqt[rt][u][v] = Cq[e];
+        }
+  }
   if (stage == 0) {
     // ---- the stopping test of the previous iteration (batch-wide, as the reference takes it)
     int done = 0;
@@ -490,7 +516,6 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   GdSys sy[2];
   gd_v4d bk[2][2];  // B_K in the layout of the right-hand sides
   double* BqT = a.BqT + (int64_t)h * 32 * d;  // [32][d]
-  const bool fresh = stage == 2 || it == 0;
   if (fresh) {
     gd_fill(sy[0], [&](int i, int j) { return Gq[i * 32 + j]; }, [&](int i, int cc) { return Cq[i * d + cc]; });
     if (stage == 2)
@@ -507,7 +532,11 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     }
     gd_drain(sy[0].x, [&](int i, int cc, double v) { BT[cc * kGdLd + i] = v; });
   } else {
-    for (int e = tid; e < 32 * d; e += kGdThreads) BT[(e % d) * kGdLd + e / d] = BqT[e];
+#pragma unroll
+    for (int u = 0; u < kBqPer; ++u) {
+      const int e = tid + u * kGdThreads;
+      BT[(e % d) * kGdLd + e / d] = bq_pre[u];
+    }
   }
   __syncthreads();
   // ---- W1 = Gk + B_Q B_Q^T
@@ -520,9 +549,15 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
   }
   __syncthreads();
   // ---- Mq'^T = W1^-1 (Ck + B_Q) beside B_K = Gk^-1 Ck
-  gd_fill(sy[0], [&](int i, int j) { return Gs[i * kGdLg + j]; },
-          [&](int i, int cc) { return Ck[i * d + cc] + BT[cc * kGdLd + i]; });
-  gd_fill(sy[1], [&](int i, int j) { return Gk[i * 32 + j]; }, [&](int i, int cc) { return Ck[i * d + cc]; });
+  gd_fill(sy[0], [&](int i, int j) { return Gs[i * kGdLg + j]; }, [&](int i, int cc) { return BT[cc * kGdLd + i]; });
+  gd_fill(sy[1], [&](int i, int j) { return Gk[i * 32 + j]; }, [&](int, int) { return 0.0; });
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      sy[0].x[rt][u] += ckt[rt][u];
+      sy[1].x[rt][u] = ckt[rt][u];
+    }
   __syncthreads();  // (every read of B_Q precedes the rewriting of the B tile below)
   gd_solve_pair(sy, piv);
 #pragma unroll
@@ -536,9 +571,14 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     float* mt = a.Mt_q + (int64_t)h * r * d;
     gd_drain(sy[0].x, [&](int i, int cc, double v) {
       MT[cc * kGdLd + i] = v;
-      part_q = fma(Cq[i * d + cc], v, part_q);
       if (i < r) mt[i * d + cc] = (float)v;
     });
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part_q = fma(cqt[rt][u][v], sy[0].x[rt][u][v], part_q);
   }
   double tr_old = 0.0;
   if (tid < 32) tr_old = tid < r ? Gq[tid * 32 + tid] : 0.0;
@@ -597,9 +637,14 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
     float* mt = a.Mt_k + (int64_t)h * r * d;
     gd_drain(sy[1].x, [&](int i, int cc, double v) {
       MT[cc * kGdLd + i] = v;
-      part_k = fma(Ck[i * d + cc], v, part_k);
       if (i < r) mt[i * d + cc] = (float)v;
     });
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part_k = fma(ckt[rt][u][v], sy[1].x[rt][u][v], part_k);
   }
   double trk_old = 0.0;
   if (tid < 32) trk_old = tid < r ? Gk[tid * 32 + tid] : 0.0;
