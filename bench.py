@@ -183,9 +183,9 @@ def prefill_als(a):
         # + the final factors written (fp32).
         bytes_g = 3.0 * (bh + bkv) * l * d * e + 4.0 * bh * l * r * 4
         gbs = bytes_g / (ms * 1e-3) / 1e9
-        # executed bf16 MFMAs of 32x32x16 per 32 rows: 48 per side (initial Grams, three-piece operands),
+        # executed bf16 MFMAs of 32x32x16 per 32 rows: 40 per side (initial Grams, three-piece operands),
         # 32 per input head (X^T X), 24 per side (apply)
-        exec_flops = (l / 32.0) * (bh * 2 * (48 + 24) + (bh + bkv) * 32) * 2.0 * 32 * 32 * 16
+        exec_flops = (l / 32.0) * (bh * 2 * (40 + 24) + (bh + bkv) * 32) * 2.0 * 32 * 32 * 16
         roof = {"bound": "hbm", "kernel": "pf_pass_bf16_kernel + pf_xtx_kernel (three readings of the long axis); "
                                           "pf_gramdom_kernel (fp64 d x d algebra per head, latency-bound) between them",
                 "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
