@@ -660,7 +660,11 @@ def test_als_prefill_long_sums(ops, ws, oracle):
                           # bf16 input on the bf16 matrix cores: d = 96 (rows not a whole number of 32-column
                           # blocks), one block, a prompt shorter than one tile, a ragged last tile per split
                           (torch.bfloat16, 2, 1, 1000, 96, 24, 2, 0.0), (torch.bfloat16, 2, 2, 333, 32, 16, 2, 0.0),
-                          (torch.bfloat16, 2, 1, 37, 64, 8, 1, 0.0), (torch.bfloat16, 4, 1, 20011, 128, 32, 2, 0.0)])
+                          (torch.bfloat16, 2, 1, 37, 64, 8, 1, 0.0), (torch.bfloat16, 4, 1, 20011, 128, 32, 2, 0.0),
+                          # the iteration on Gram matrices (bf16 rows of 128): ranks below 32 (identity padding of the
+                          # r x r systems), one iteration, and the batch-wide stopping test after the first / a later one
+                          (torch.bfloat16, 4, 2, 2000, 128, 16, 3, 0.0), (torch.bfloat16, 2, 1, 1500, 128, 24, 1, 0.0),
+                          (torch.bfloat16, 2, 1, 1200, 128, 32, 6, 1e30), (torch.bfloat16, 4, 2, 1500, 128, 20, 6, 5e-2)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
