@@ -617,7 +617,7 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
     const int64_t base = (t0 < r1 ? t0 : r0) * d;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const int e = (i * kWave + lane) * VEC;
+      const int e = (((i + wave) % NL) * kWave + lane) * VEC;  // (the waves start at different KB of their tiles)
       pre[i] = *reinterpret_cast<const uint4*>(Xh + base + (e < nvalid ? e : 0));
     }
   };
@@ -643,7 +643,7 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       const int nvalid = rows * d;
 #pragma unroll
       for (int i = 0; i < NL; ++i) {
-        const int e = (i * kWave + lane) * VEC;
+        const int e = (((i + wave) % NL) * kWave + lane) * VEC;
         if (e < 32 * d) {
           const int row = full_rows ? e / (32 * NB) : e / d;
           const int c0 = full_rows ? e % (32 * NB) : e - row * d;
