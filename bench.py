@@ -434,8 +434,7 @@ def main():
     sel_short, sel_over = eng.ws.select_stats_detail()
     host_rows = eng.ws.victim_stats()
     rows_scanned, rows_rescored = eng.ws.scan_stats()
-    vic_on = eng.victim_rows_effective > 0 and a.fetch == "direct" \
-        and not a.no_attn and a.variant == "default"
+    vic_on = eng.victim_rows_effective > 0 and a.fetch == "direct" and a.variant == "default"
     grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
     m_last = eng.lite_indices[eng.lite_len] - 1
     n_timed = len(counts)

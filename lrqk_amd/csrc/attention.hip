@@ -654,6 +654,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   int S = (n_slots + 127) / 128;  // small launches: finer attention splits
   if ((int64_t)(S + want_fetch + 2) * bh > slots) S = (n_slots + 255) / 256;
   if (S > 64) S = 64;
+  if (!out) S = 0;  // fetch only (the caller runs its own attention): no attention workgroups, nothing to merge
   const int room = slots / bh - S - 2;
   const int n_fetch = std::min(want_fetch, std::max(room, 8));
   if ((rc = ctx->attn_part.ensure((size_t)bh * (S + n_fetch) * (d + 2) * sizeof(float)))) return rc;
@@ -671,7 +672,7 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   const int index_role = with_finish && ctx->fin.qa != nullptr && ctx->fin.append_row >= 0 ? 1 : 0;
   // K q of every slot, left by this step's Gram pass over the same buffers and query (else the role reads K)
   const float* kq = nullptr;
-  if (ctx->kq_valid && ctx->kq_k_act == k_act && ctx->kq_q == q && ctx->kq_bh == bh && ctx->kq_n == n_slots)
+  if (out && ctx->kq_valid && ctx->kq_k_act == k_act && ctx->kq_q == q && ctx->kq_bh == bh && ctx->kq_n == n_slots)
     kq = (const float*)ctx->als_kq.p;
   ctx->kq_valid = false;
   hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish + index_role), (unsigned)bh),
@@ -679,14 +680,18 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
                      scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new, kq);
   LRQK_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
-                     (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);
-  LRQK_HIP_CHECK(hipGetLastError());
+  if (out) {
+    hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
+                       (const float*)ctx->attn_part.p, S + n_fetch, d, (T*)out);
+    LRQK_HIP_CHECK(hipGetLastError());
+  }
   return LRQK_OK;
 }
 
 // Miss fetch overlapped with the attention over the slots that stay resident, then the
 // refetched slots and the merge.  Same result as lrqk_fetch_rows followed by lrqk_attention.
+// out = NULL: the fetch alone (with the victim cache and the roles that ride along), for a caller
+// that runs its own attention over the active set.
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,

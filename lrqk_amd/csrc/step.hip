@@ -37,8 +37,8 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   // the step ends with the fetch + attention launch it rides there, and the scan takes the proxy
   // query from the iterates directly.  Any path that cannot absorb it flushes it as its own launch.
   // (a [K|V] row must fit the lanes of one wave for the fetch role to form its attention term)
-  const bool fused_tail = attn_out != nullptr && !no_hit_miss && ctx->fetch_mode == 0 &&
-                          2 * (size_t)d * elem_size(dtype) / 16 <= (size_t)kWave;
+  // (without attn_out the same launch runs with its fetch, finish and index roles only)
+  const bool fused_tail = !no_hit_miss && ctx->fetch_mode == 0 && 2 * (size_t)d * elem_size(dtype) / 16 <= (size_t)kWave;
   const bool defer_finish = fused_tail;
   // ring append folded into the first kernel of the factor update; the flush of a full ring
   // (which reads the slot just written) follows it
