@@ -67,6 +67,10 @@ def parse():
     p.add_argument("--batch", type=int, default=4, help="decoder mode: sequences")
     p.add_argument("--prompt", type=int, default=65536, help="decoder mode: prompt tokens per sequence")
     p.add_argument("--new-tokens", type=int, default=128, help="decoder mode: tokens decoded per sequence")
+    p.add_argument("--max-iter", type=int, default=0,
+                   help="decode mode: iterations of the factor update per step and at the prompt instead of the workload's "
+                        "(the reference's throughput script runs 8, tps_estimate.py:20-29); with --tol")
+    p.add_argument("--tol", type=float, default=1e-8, help="stopping tolerance used with --max-iter")
     p.add_argument("--seqs", type=int, default=0,
                    help="decode mode: sequences stepped together (the batch of the layer-step; 0 = the workload's "
                         "own, 1 for the 128K configuration); value stays the time of one layer-step of the whole batch")
@@ -326,6 +330,9 @@ def main():
     if a.seqs > 0 and a.seqs != w.batch:
         import dataclasses
         w = dataclasses.replace(w, batch=a.seqs)
+    if a.max_iter > 0:
+        import dataclasses
+        w = dataclasses.replace(w, max_iter=(a.max_iter, a.max_iter), tol=(a.tol, a.tol))
     l = a.context or w.context
     t_setup = time.perf_counter()
     # synthetic prompt, drawn on the GPU (128K x 48 heads x 128 would take minutes on the host)

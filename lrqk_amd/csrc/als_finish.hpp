@@ -31,10 +31,12 @@ __device__ __forceinline__ int als_decide(float (&sacc)[MAXIT], int bh, int max_
   bool found = false;
 #pragma unroll
   for (int it = 0; it < MAXIT; ++it) {
-    const float tot = wave_sum(sacc[it]);
-    if (!found && it < max_iter && tot / (float)((int64_t)bh * r) < tol) {
-      chosen = it;
-      found = true;
+    if (it < max_iter) {  // (uniform: iterations that do not exist cost nothing)
+      const float tot = wave_sum(sacc[it]);
+      if (!found && tot / (float)((int64_t)bh * r) < tol) {
+        chosen = it;
+        found = true;
+      }
     }
   }
   return chosen;

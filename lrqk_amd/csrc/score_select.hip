@@ -205,7 +205,7 @@ constexpr int kFiltRPT = LRQK_FILT_RPT;  // rows per thread and tile
 constexpr int kFiltTiles = LRQK_FILT_TILES;  // tiles per workgroup: one global list reservation for all of them
 constexpr int kFiltRows = kFiltThreads * kFiltRPT;
 constexpr int kPreCap = 2048;   // exact hits a prefilter workgroup can hold
-constexpr int kFiltMaxIt = 4;  // most iterations of the factor update whose pending iterate the filter can pick itself
+constexpr int kFiltMaxIt = 8;  // most iterations of the factor update whose pending iterate the filter can pick itself
 
 // Proxy query taken straight from the iterates of the factor update whose finish stage has not
 // run yet (iter_out == nullptr: q_hat is read instead).  Workgroup 0 of every head writes the

@@ -456,24 +456,26 @@ def test_poster_operating_point(lrqk, oracle):
     assert n > 0 and len(eng.KVcpu) == 6000 + 16
 
 
-@pytest.mark.parametrize("r,k,L,l,dtype", [(32, 512, 16, 3000, torch.bfloat16), (8, 256, 8, 2000, torch.bfloat16),
-                                             (16, 128, 8, 1000, torch.float32)])
-def test_eight_iterations_tight_tolerance(lrqk, oracle, r, k, L, l, dtype):
+@pytest.mark.parametrize("r,k,L,l,dtype,iters", [(32, 512, 16, 3000, torch.bfloat16, 8), (8, 256, 8, 2000, torch.bfloat16, 8),
+                                                   (16, 128, 8, 1000, torch.float32, 8),
+                                                   (16, 256, 8, 1500, torch.bfloat16, 12)])
+def test_eight_iterations_tight_tolerance(lrqk, oracle, r, k, L, l, dtype, iters):
     """max_iter (8, 8) with tol 1e-8, the setting of the reference's accuracy configurations
-    (eval_configs_lrqk): more decode iterations than the scan can take over from the solve kernel, so the
-    step finishes the factor update in a launch of its own.  Also the smallest rank the reference sweeps (8)."""
-    _say("max_iter 8 / tol 1e-8 trace", r, k, L, l, dtype)
+    (eval_configs_lrqk): the most decode iterations whose iterate the scan picks itself.  With 12 the step
+    finishes the factor update in a launch of its own before the scan.  Also the smallest rank the reference
+    sweeps (8)."""
+    _say("max_iter %d / tol 1e-8 trace" % iters, r, k, L, l, dtype)
     _, _, n = _lockstep(lrqk, oracle, b=1, hq=8, hkv=2, d=64, l=l, r=r, k=k, L=L, steps=20, dtype=dtype,
-                        max_iter=(8, 8), tol=(1e-8, 1e-8), rho=2 * r, sigma=0.05, capacity=1024,
+                        max_iter=(iters, iters), tol=(1e-8, 1e-8), rho=2 * r, sigma=0.05, capacity=1024,
                         compare_factors=False,
-                        oracle_heads=(0, 5), tag=f"iter8_r{r}")
+                        oracle_heads=(0, 5), tag=f"iter{iters}_r{r}")
     assert n > 0
 
 
 def test_reference_style_caller(lrqk, oracle):
     """The step as a reference-style caller drives it (DynamicLRQKCache.update returns K, V and the caller
-    runs the attention, py:2284-2290, 2326): no attention inside the step, hence the separate fetch launch
-    and no victim cache.  Same lock-step comparison, ring flush included."""
+    runs the attention, py:2284-2290, 2326): no attention inside the step, whose last launch then runs with its
+    fetch (victim cache included), finish and index roles only.  Same lock-step comparison, ring flush included."""
     _say("reference-style caller trace (attention outside the step)")
     _, _, n = _lockstep(lrqk, oracle, b=2, hq=8, hkv=2, d=64, l=1500, r=16, k=256, L=8, steps=30,
                         dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-2, 1e-2), rho=32, sigma=0.05, capacity=512,
