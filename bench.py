@@ -71,6 +71,9 @@ def parse():
                    help="decode mode: iterations of the factor update per step and at the prompt instead of the workload's "
                         "(the reference's throughput script runs 8, tps_estimate.py:20-29); with --tol")
     p.add_argument("--tol", type=float, default=1e-8, help="stopping tolerance used with --max-iter")
+    p.add_argument("--rank", type=int, default=0, help="decode mode: r instead of the workload's")
+    p.add_argument("--topk", type=int, default=0, help="decode mode: active tokens k instead of the workload's")
+    p.add_argument("--lite", type=int, default=0, help="decode mode: recent-token window instead of the workload's")
     p.add_argument("--seqs", type=int, default=0,
                    help="decode mode: sequences stepped together (the batch of the layer-step; 0 = the workload's "
                         "own, 1 for the 128K configuration); value stays the time of one layer-step of the whole batch")
@@ -333,6 +336,10 @@ def main():
     if a.max_iter > 0:
         import dataclasses
         w = dataclasses.replace(w, max_iter=(a.max_iter, a.max_iter), tol=(a.tol, a.tol))
+    if a.rank or a.topk or a.lite:
+        import dataclasses
+        w = dataclasses.replace(w, r=a.rank or w.r, num_active_tokens=a.topk or w.num_active_tokens,
+                                lite_tokens=a.lite or w.lite_tokens)
     l = a.context or w.context
     t_setup = time.perf_counter()
     # synthetic prompt, drawn on the GPU (128K x 48 heads x 128 would take minutes on the host)
