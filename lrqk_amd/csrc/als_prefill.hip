@@ -1062,26 +1062,32 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   const dim3 grid((unsigned)S, (unsigned)bh), blk((unsigned)pass_threads), sblk(small32 ? kPfSmallThreads : kPfThreads);
   const T* Q = (const T*)q;
   const T* K = (const T*)k;
-  PfPassFn<T> first = pass;  // the sums over the given initial factors
-  if constexpr (sizeof(T) == 2) {
-    if (mfma && d == 128) {
-      first = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, true, true>;
-      if (smem_pass > 48 * 1024)
-        LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)first, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
+  // bf16 rows of 128 elements: every iteration on the d x d Gram matrices (fp64), then one pass per side that
+  // applies the last Mq, Mk; the Q side's sums over the given factors are formed together with Q^T Q (one
+  // reading of Q), the K side's by the pass below (A_K has a head per query head, K per kv head)
+  const bool gram_domain = sizeof(T) == 2 && mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
+  const bool fused_sums = gram_domain && !getenv("LRQK_PREFILL_SEPARATE_SUMS");  // (the Q side's, with Q^T Q)
+  {
+    PfPassFn<T> first = pass;  // the sums over the given initial factors
+    if constexpr (sizeof(T) == 2) {
+      if (mfma && d == 128) {
+        first = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, true, true>;
+        if (smem_pass > 48 * 1024)
+          LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)first, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
+      }
     }
+    if (!fused_sums)
+      hipLaunchKernelGGL(first, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
+                         (float*)nullptr, (const int*)nullptr, S);
+    hipLaunchKernelGGL(first, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
+                       (float*)nullptr, (const int*)nullptr, S);
+    LRQK_HIP_CHECK(hipGetLastError());
   }
-  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
-                     (float*)nullptr, (const int*)nullptr, S);
-  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
-                     (float*)nullptr, (const int*)nullptr, S);
-  LRQK_HIP_CHECK(hipGetLastError());
   if constexpr (sizeof(T) == 2) {
-    // bf16 rows of 128 elements: every iteration on the d x d Gram matrices (fp64), then one pass per side
-    // that applies the last Mq, Mk
-    if (mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE")) {
+    if (gram_domain) {
       float *mt_q = nullptr, *mt_k = nullptr;
-      if ((rc = prefill_gram_domain(ctx, q, k, partQ, partK, S, b_q, b_k, b, hq, hkv, l, r, iters, tol, flags, &mt_q,
-                                    &mt_k, st)))
+      if ((rc = prefill_gram_domain(ctx, q, k, fused_sums ? nullptr : partQ, partK, S, fused_sums ? a_q : nullptr, b_q,
+                                    b_k, b, hq, hkv, l, r, iters, tol, flags, &mt_q, &mt_k, st)))
         return rc;
       if (iters > 0) {
         PfPassFn<T> lean = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, false>;
@@ -1089,8 +1095,11 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
           LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)lean, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
         hipLaunchKernelGGL(lean, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)mt_q, a_q, partQ, deltas,
                            (const int*)nullptr, S);
-        hipLaunchKernelGGL(lean, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)mt_k, a_k, partK,
-                           deltas + (size_t)bh * S, (const int*)nullptr, S);
+        int rck = LRQK_OK;
+        if (getenv("LRQK_PREFILL_SEPARATE_SUMS") || !prefill_apply_shared(k, mt_k, a_k, b, hq, hkv, l, r, st, &rck))
+          hipLaunchKernelGGL(lean, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)mt_k, a_k, partK,
+                             deltas + (size_t)bh * S, (const int*)nullptr, S);
+        if (rck) return rck;
         LRQK_HIP_CHECK(hipGetLastError());
       }
       return LRQK_OK;

@@ -35,9 +35,9 @@ __device__ __forceinline__ int gd_mfma_row(int lane, int v) { return ((v >> 2) <
 // ----------------------------------------------------------------------------- X^T X
 // grid (S, x heads); 8 waves share the rows (128 per step, staged in LDS as they lie in memory); wave w owns
 // the output blocks (w / 2, 2 (w % 2)) and (w / 2, 2 (w % 2) + 1) of 32 x 32.  A lane's operand for column
-// block nb is eight rows of one column, read from the tile as eight 16-bit values; every 32-row tile is summed
-// in a fresh accumulator and added to the running total in fp32 (the matrix cores do not round to nearest
-// when they add to a large accumulator).
+// block nb is eight rows of one column, which the transposing LDS read delivers four at a time; every 32-row
+// tile is summed in a fresh accumulator and added to the running total in fp32 (the matrix cores do not round
+// to nearest when they add to a large accumulator).
 constexpr int kXtxWaves = 8, kXtxThreads = kXtxWaves * kWave, kXtxRows = 128, kXtxD = 128;
 constexpr int kXtxLd = kXtxD + 16;  // bf16 elements per staged row: 288 bytes, so four successive rows start 8 banks apart
 
@@ -119,6 +119,312 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
     out[i * kXtxD + 32 * nb2 + col] = acc0[v];
     out[i * kXtxD + 32 * (nb2 + 1) + col] = acc1[v];
   }
+}
+
+// ----------------------------------------------------------------------------- X^T X and the sums over given factors
+// One reading of X for both (the Q side, where every head has rows of its own): the workgroup stages 128 rows of X
+// per step as pf_xtx_kernel does and its waves form, besides their two blocks of X^T X, the sums (A^T A, A^T X)
+// over the given factors A (fp32, [head][l][r]).  Wave (a, ch) = (w / 2, w % 2) takes the 32-row group a of the
+// step and the column blocks 2 ch, 2 ch + 1 of A^T X; of A^T A it takes the products of k block ch (the two
+// waves' halves are added at the end).  The rows of A are read in the accumulator layout (element v of lane l: row
+// gd_mfma_row(l, v), column l % 32) and split into three bf16 pieces (8 + 8 + 8 mantissa bits, exact); taken
+// eight at a time these are an operand's k elements, and X's come out of LDS in the same order by the transposing
+// read.  Products per 32 rows as in the row-by-row pass: all piece pairs of A^T A except lo x lo, three pieces of
+// A times X; every 32-row group in a fresh accumulator.  part: [head][S][r][r + d] like the row-by-row pass
+// writes them; xtx_part: [head][S][d][d].
+// (Several heads that share their X -- the K side -- in one workgroup were tried and are slower: a wave then works
+// through its heads' row groups one after the other, and their rows of A in flight together do not fit the
+// registers.  Requesting the rows of A a step ahead also made this kernel slower: 142 against 126 us at 32 heads
+// x 32K rows.)
+__device__ __forceinline__ void gd_split3(float x, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+  hi = __float_as_uint(x) & 0xffff0000u;
+  const float r1 = x - __uint_as_float(hi);  // exact
+  mid = __float_as_uint(r1) & 0xffff0000u;
+  const float r2 = r1 - __uint_as_float(mid);  // exact, at most 8 significant bits
+  lo = __float_as_uint(r2) & 0xffff0000u;
+}
+__device__ __forceinline__ uint32_t gd_pack2(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
+
+__global__ __launch_bounds__(kXtxThreads) void pf_sums_kernel(const bf16_t* __restrict__ X, int64_t l,
+                                                              const float* __restrict__ A, int r,
+                                                              float* __restrict__ part, float* __restrict__ xtx_part,
+                                                              int S) {
+  // the tile of X; at the end the waves' sums pass through it
+  __shared__ __align__(16) uint16_t x_s[kXtxRows * kXtxLd];
+  static_assert(sizeof(x_s) >= kXtxWaves * 1024 * sizeof(float), "the reduction uses the tile's LDS");
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int col = lane & 31, half = lane >> 5;
+  const int xh = blockIdx.y, s = blockIdx.x;
+  const bf16_t* Xh = X + (int64_t)xh * l * kXtxD;
+  const int wa = wave >> 1, ch = wave & 1;
+  const int nb1 = wa, nb2 = 2 * ch;  // blocks of X^T X
+  const float* Ah = A + (int64_t)xh * l * r;
+  constexpr int NL = kXtxRows * kXtxD / (kXtxThreads * 8);
+  uint4 pre_a[NL];
+  auto issue = [&](int64_t t0, uint4 (&dst)[NL]) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int e = (i * kXtxThreads + tid) * 8;
+      const int64_t row = t0 + e / kXtxD;
+      dst[i] = *reinterpret_cast<const uint4*>(Xh + min(row, l - 1) * kXtxD + e % kXtxD);
+    }
+  };
+  gd_floatx16 acc0, acc1, gAA, gAX[2];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = gAA[v] = gAX[0][v] = gAX[1][v] = 0.0f;
+  typedef short gd_v4s __attribute__((ext_vector_type(4)));
+  typedef gd_v4s __attribute__((address_space(3))) * gd_lds_v4s;
+  auto operand = [&](int row0, int nb) {  // rows row0 + 8 half .. + 7 of column 32 nb + col
+    const int s16 = lane & 15;
+    const uint16_t* p = &x_s[(row0 + 8 * half + (s16 >> 2)) * kXtxLd + 32 * nb + (col & 16) + 4 * (s16 & 3)];
+    const gd_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)p);
+    const gd_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)(p + 4 * kXtxLd));
+    return __builtin_bit_cast(gd_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto operand_acc = [&](int row0, int nb) {  // rows row0 + 4 half .. + 3 and the same + 8: the accumulator's order
+    const int s16 = lane & 15;
+    const uint16_t* p = &x_s[(row0 + 4 * half + (s16 >> 2)) * kXtxLd + 32 * nb + (col & 16) + 4 * (s16 & 3)];
+    const gd_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)p);
+    const gd_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)(p + 8 * kXtxLd));
+    return __builtin_bit_cast(gd_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  const int64_t stride = (int64_t)S * kXtxRows;
+  float arow[16];  // this wave's rows of A of the step being multiplied, requested at the start of the step
+  auto step = [&](int64_t t0, uint4 (&cur)[NL]) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int e = (i * kXtxThreads + tid) * 8;
+      const int row = e / kXtxD;
+      *reinterpret_cast<uint4*>(&x_s[row * kXtxLd + e % kXtxD]) = t0 + row < l ? cur[i] : make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+    if (t0 + stride < l) issue(t0 + stride, cur);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {  // (consumed after the blocks of X^T X below)
+      const int64_t row = min(t0 + 32 * wa + gd_mfma_row(lane, v), l - 1);
+      arow[v] = Ah[row * r + min(col, r - 1)];
+    }
+    const int tiles = (int)min((int64_t)4, (l - t0 + 31) / 32);
+    for (int tile = 0; tile < tiles; ++tile) {
+      gd_floatx16 t0a, t1a;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) t0a[v] = t1a[v] = 0.0f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const int row0 = 32 * tile + 16 * kb;
+        const gd_bf16x8 a = operand(row0, nb1);
+        const gd_bf16x8 b0 = operand(row0, nb2), b1 = operand(row0, nb2 + 1);
+        t0a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, t0a, 0, 0, 0);
+        t1a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, t1a, 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        acc0[v] += t0a[v];
+        acc1[v] += t1a[v];
+      }
+    }
+    if (t0 + 32 * wa < l) {  // (wave-uniform)
+      // the three pieces of the group's rows of A, eight rows (one k block) at a time
+      gd_bf16x8 cp[3][2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        uint32_t pc[3][8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int v = 8 * kb + q;
+          const bool valid = t0 + 32 * wa + gd_mfma_row(lane, v) < l && col < r;
+          gd_split3(valid ? arow[v] : 0.0f, pc[0][q], pc[1][q], pc[2][q]);
+        }
+#pragma unroll
+        for (int pp = 0; pp < 3; ++pp)
+          cp[pp][kb] = __builtin_bit_cast(gd_bf16x8, make_uint4(gd_pack2(pc[pp][0], pc[pp][1]), gd_pack2(pc[pp][2], pc[pp][3]),
+                                                                gd_pack2(pc[pp][4], pc[pp][5]), gd_pack2(pc[pp][6], pc[pp][7])));
+      }
+      {
+        gd_floatx16 t;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) t[v] = 0.0f;
+        // k block ch of A^T A, smallest pieces first
+        const gd_bf16x8 c0 = ch ? cp[0][1] : cp[0][0], c1 = ch ? cp[1][1] : cp[1][0], c2 = ch ? cp[2][1] : cp[2][0];
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c1, c2, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c2, c1, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c0, c2, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c2, c0, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c1, c1, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c0, c1, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c1, c0, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(c0, c0, t, 0, 0, 0);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) gAA[v] += t[v];
+      }
+#pragma unroll
+      for (int nbi = 0; nbi < 2; ++nbi) {
+        gd_bf16x8 xb[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) xb[kb] = operand_acc(32 * wa + 16 * kb, 2 * ch + nbi);
+        gd_floatx16 t;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) t[v] = 0.0f;
+#pragma unroll
+        for (int pp = 2; pp >= 0; --pp)
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cp[pp][kb], xb[kb], t, 0, 0, 0);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) gAX[nbi][v] += t[v];
+      }
+    }
+    __syncthreads();
+  };
+  const int64_t first = (int64_t)s * kXtxRows;
+  if (first < l) issue(first, pre_a);
+  for (int64_t t0 = first; t0 < l; t0 += stride) step(t0, pre_a);
+  {
+    float* out = xtx_part + ((int64_t)xh * S + s) * kXtxD * kXtxD;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int i = 32 * nb1 + gd_mfma_row(lane, v);
+      out[i * kXtxD + 32 * nb2 + col] = acc0[v];
+      out[i * kXtxD + 32 * (nb2 + 1) + col] = acc1[v];
+    }
+  }
+  // the waves' sums: round 0 is A^T A (all waves), rounds 1, 2 the column blocks 2 ch + 0 / + 1 of A^T X (the waves
+  // with the same ch)
+  float* sm = reinterpret_cast<float*>(x_s);
+  const int ne = r * (r + kXtxD);
+  float* outp = part + ((int64_t)xh * S + s) * ne;
+#pragma unroll 1
+  for (int blk = 0; blk < 3; ++blk) {
+    float* mine = sm + wave * 1024;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      mine[gd_mfma_row(lane, v) * 32 + col] = blk == 0 ? gAA[v] : (blk == 1 ? gAX[0][v] : gAX[1][v]);
+    __syncthreads();
+    const int n_out = (blk == 0 ? 1 : 2) * 1024;
+    for (int o = tid; o < n_out; o += kXtxThreads) {
+      const int e = o & 1023, c_half = blk == 0 ? -1 : (o >> 10);
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kXtxWaves; ++w)
+        if (c_half < 0 || (w & 1) == c_half) v += sm[w * 1024 + e];
+      const int m = e >> 5, n = e & 31;
+      if (blk == 0) {
+        if (m < r && n < r) outp[m * (r + kXtxD) + n] = v;
+      } else {
+        const int cx = 32 * (2 * c_half + (blk - 1)) + n;
+        if (m < r) outp[m * (r + kXtxD) + r + cx] = v;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ----------------------------------------------------------------------------- A = X Mt^T for heads that share X
+// The K side's last pass: the NH query heads of a kv head take their rows of A_K from the same rows of K, so one
+// workgroup stages 128 rows of K per step (as pf_xtx_kernel does) and applies the NH heads' Mt to them: K is read
+// once per kv head instead of once per query head.  Mt (fp32) lies in LDS as three bf16 pieces per head, X as it
+// is; wave w takes head w / (8 / NH) and NH / 2 of the step's four 32-row groups; 24 products of 32x32x16 per
+// group (X times the three pieces), fp32 accuracy as in the row-by-row pass.  grid (S, kv heads); split s takes
+// the steps s, s + S, ...
+constexpr int kApLd = kXtxD + 8;  // bf16 elements per staged row: 16-byte operand reads want rows 4 banks apart
+template <int NH>
+__global__ __launch_bounds__(kXtxThreads) void pf_apply_shared_kernel(const bf16_t* __restrict__ X, int64_t l,
+                                                                      const float* __restrict__ Mt, int r,
+                                                                      float* __restrict__ A, int S) {
+  static_assert(NH == 2 || NH == 4, "query heads per kv head");
+  extern __shared__ __align__(16) uint16_t ap_s[];
+  uint16_t* x_s = ap_s;                          // [128][kApLd]
+  uint16_t* mt_s = ap_s + kXtxRows * kApLd;      // [NH][3][32][kApLd]
+  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+  const int col = lane & 31, half = lane >> 5;
+  const int xh = blockIdx.y, s = blockIdx.x;
+  const bf16_t* Xh = X + (int64_t)xh * l * kXtxD;
+  constexpr int WPH = kXtxWaves / NH, GPW = 4 / WPH;  // waves per head, row groups per wave and step
+  const int hl = wave / WPH, g0 = (wave % WPH) * GPW;
+  float* Ah = A + ((int64_t)xh * NH + hl) * l * r;
+  for (int e = tid; e < NH * 32 * kXtxD; e += kXtxThreads) {
+    const int hh = e / (32 * kXtxD), n = (e / kXtxD) % 32, k = e % kXtxD;
+    const float v = n < r ? Mt[(((int64_t)xh * NH + hh) * r + n) * kXtxD + k] : 0.0f;
+    uint32_t p0, p1, p2;
+    gd_split3(v, p0, p1, p2);
+    mt_s[((hh * 3 + 0) * 32 + n) * kApLd + k] = (uint16_t)(p0 >> 16);
+    mt_s[((hh * 3 + 1) * 32 + n) * kApLd + k] = (uint16_t)(p1 >> 16);
+    mt_s[((hh * 3 + 2) * 32 + n) * kApLd + k] = (uint16_t)(p2 >> 16);
+  }
+  constexpr int NL = kXtxRows * kXtxD / (kXtxThreads * 8);
+  static_assert(NL == 4, "four 16-byte loads per thread and step");
+  uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0, pre2 = pre0, pre3 = pre0;
+  auto issue = [&](int64_t t0) {
+    auto ld = [&](int i) {
+      const int e = (i * kXtxThreads + tid) * 8;
+      const int64_t row = t0 + e / kXtxD;
+      return *reinterpret_cast<const uint4*>(Xh + min(row, l - 1) * kXtxD + e % kXtxD);
+    };
+    pre0 = ld(0);
+    pre1 = ld(1);
+    pre2 = ld(2);
+    pre3 = ld(3);
+  };
+  auto stage = [&](int i, const uint4& v) {
+    const int e = (i * kXtxThreads + tid) * 8;
+    *reinterpret_cast<uint4*>(&x_s[(e / kXtxD) * kApLd + e % kXtxD]) = v;  // (rows beyond l are never stored from)
+  };
+  const int64_t stride = (int64_t)S * kXtxRows;
+  const int64_t first = (int64_t)s * kXtxRows;
+  if (first < l) issue(first);
+  for (int64_t t0 = first; t0 < l; t0 += stride) {
+    stage(0, pre0);
+    stage(1, pre1);
+    stage(2, pre2);
+    stage(3, pre3);
+    __syncthreads();  // (the first one also covers the staging of Mt)
+    if (t0 + stride < l) issue(t0 + stride);
+#pragma unroll
+    for (int j = 0; j < GPW; ++j) {
+      const int g = g0 + j;
+      if (t0 + 32 * g >= l) continue;  // (wave-uniform)
+      gd_floatx16 c;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) c[v] = 0.0f;
+#pragma unroll
+      for (int kb = 0; kb < kXtxD / 16; ++kb) {
+        const gd_bf16x8 xa = *reinterpret_cast<const gd_bf16x8*>(&x_s[(32 * g + col) * kApLd + kb * 16 + 8 * half]);
+#pragma unroll
+        for (int pp = 0; pp < 3; ++pp) {
+          const gd_bf16x8 m =
+              *reinterpret_cast<const gd_bf16x8*>(&mt_s[((hl * 3 + pp) * 32 + col) * kApLd + kb * 16 + 8 * half]);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, m, c, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t row = t0 + 32 * g + gd_mfma_row(lane, v);
+        if (row < l && col < r) Ah[row * r + col] = c[v];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// A_K = K Mk for all query heads, reading K once per kv head.  Returns false if this grouping of heads has no
+// kernel here (the caller then runs its row-by-row pass).
+bool prefill_apply_shared(const void* k, const float* mt_k, float* a_k, int b, int hq, int hkv, int64_t l, int r,
+                          hipStream_t st, int* rc_out) {
+  *rc_out = LRQK_OK;
+  const int nh = hq / hkv, bkv = b * hkv;
+  if (nh != 2 && nh != 4) return false;
+  const int S = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 256 / bkv), (l + kXtxRows - 1) / kXtxRows));
+  const size_t smem = (size_t)(kXtxRows + nh * 3 * 32) * kApLd * sizeof(uint16_t);
+  auto kern = nh == 2 ? pf_apply_shared_kernel<2> : pf_apply_shared_kernel<4>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) {
+    *rc_out = set_error(LRQK_EHIP, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+    return true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)S, (unsigned)bkv), dim3(kXtxThreads), smem, st, (const bf16_t*)k, l, mt_k, r,
+                     a_k, S);
+  e = hipGetLastError();
+  if (e != hipSuccess) *rc_out = set_error(LRQK_EHIP, "launch failed: %s", hipGetErrorString(e));
+  return true;
 }
 
 // ----------------------------------------------------------------------------- d x d algebra, fp64
@@ -380,7 +686,8 @@ struct GdArgs {
   // initial (G, C) of the two sides as the first Gram passes left them: S partial sums of [r][r + d] floats per head
   const float* partQ;
   const float* partK;
-  int S;
+  int S;                // splits of partQ
+  int S_k;              // splits of partK
   const double* Sq;     // [bh][d][d]
   const double* Sk;     // [b * hkv][d][d]
   double* G;            // [2][bh][32][32]  (side 0: Q, 1: K), padded with the identity
@@ -428,12 +735,13 @@ __global__ __launch_bounds__(256) void pf_gramdom_init_kernel(GdArgs a, const fl
   const int e = (blk % kGdInitBlocks) * 256 + threadIdx.x;
   if (e >= 32 * (32 + d)) return;
   const int ne = r * (r + d);
-  const float* part = (side ? a.partK : a.partQ) + (int64_t)h * a.S * ne;
+  const int Sn = side ? a.S_k : a.S;
+  const float* part = (side ? a.partK : a.partQ) + (int64_t)h * Sn * ne;
   const int i = e / (32 + d), j = e % (32 + d);
   double v = 0.0;
   if (i < r && (j >= 32 || j < r)) {
     const int src = i * (r + d) + (j < 32 ? j : r + (j - 32));
-    for (int s = 0; s < a.S; ++s) v += (double)part[(int64_t)s * ne + src];
+    for (int s = 0; s < Sn; ++s) v += (double)part[(int64_t)s * ne + src];
   } else if (j < 32) {
     v = i == j ? 1.0 : 0.0;
   }
@@ -675,9 +983,10 @@ __global__ __launch_bounds__(kGdThreads) void pf_gramdom_kernel(int stage, int i
 }
 
 // Workspace (bytes) of the Gram-domain iteration for bh heads over bkv distinct K heads.
-static size_t gramdom_bytes(int bh, int bkv, int Sx, int Sxk, int iters) {
+static size_t gramdom_bytes(int bh, int bkv, int Sx, int Sxk, int iters, size_t own_part_floats) {
   const size_t dd = (size_t)kGdD * kGdD;
   return ((size_t)bh * Sx + (size_t)bkv * Sxk) * dd * sizeof(float)      // X^T X partial sums
+         + own_part_floats * sizeof(float)                                // (G, C) partial sums of the fused kernel
          + ((size_t)bh + bkv) * dd * sizeof(double)                       // Sq, Sk
          + (size_t)2 * bh * (1024 + 32 * kGdD) * sizeof(double)           // G, C
          + (size_t)bh * 32 * kGdD * sizeof(double)                        // B_Q handed from iteration to iteration
@@ -687,16 +996,28 @@ static size_t gramdom_bytes(int bh, int bkv, int Sx, int Sxk, int iters) {
 
 // Runs all iterations on the Gram matrices.  On return Mt_q / Mt_k (device pointers written to *mt_q, *mt_k)
 // hold Mq^T, Mk^T of the last iteration that ran, and b_q, b_k the final B factors; the caller applies
-// A_Q = Q Mq, A_K = K Mk.  partQ / partK: the initial [G | C] partial sums (S splits).
+// A_Q = Q Mq, A_K = K Mk.  The initial [G | C] sums: partK (and partQ) with S splits from the row-by-row pass; with
+// a_q0 (the given A_Q, [bh][l][r]) the Q side's are formed here together with Q^T Q and partQ is not read.
 int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float* partQ, const float* partK, int S,
-                        float* b_q, float* b_k, int b, int hq, int hkv, int64_t l, int r, int iters, float tol, int* flags,
-                        float** mt_q, float** mt_k, hipStream_t st) {
+                        const float* a_q0, float* b_q, float* b_k, int b, int hq, int hkv, int64_t l, int r, int iters,
+                        float tol, int* flags, float** mt_q, float** mt_k, hipStream_t st) {
   const int bh = b * hq, bkv = b * hkv;
   const int d = kGdD;
-  // splits of the long axis for the X^T X sums: about two workgroups per CU (measured: 89 us against 103 with one)
+  const bool fused = a_q0 != nullptr;
+  LRQK_REQUIRE(partK && (fused || partQ), LRQK_EINVAL, "neither partial sums nor initial factors");
+  // splits of the long axis for the X^T X sums: about two workgroups per CU.  The fused kernel: one workgroup per
+  // CU (registers), at most 4096 rows per split (its fp32 sums), at least one step each.
   int Sx = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 512 / bh), (l + 511) / 512));
-  int Sxk = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 512 / bkv), (l + 511) / 512));
-  int rc = ctx->prefill_gd.ensure(gramdom_bytes(bh, bkv, Sx, Sxk, iters));
+  const int Sxk = (int)std::max<int64_t>(1, std::min<int64_t>(std::max(1, 512 / bkv), (l + 511) / 512));
+  int Spq = S;
+  if (fused) {
+    int64_t v = std::max<int64_t>(std::max(1, 256 / bh), (l + 4095) / 4096);
+    v = std::min<int64_t>(v, 64);
+    Sx = Spq = (int)std::max<int64_t>(1, std::min<int64_t>(v, (l + kXtxRows - 1) / kXtxRows));
+  }
+  const size_t ne = (size_t)r * (r + d);
+  const size_t own_part = fused ? (size_t)bh * Spq * ne : 0;
+  int rc = ctx->prefill_gd.ensure(gramdom_bytes(bh, bkv, Sx, Sxk, iters, own_part));
   if (rc) return rc;
   const size_t dd = (size_t)d * d;
   char* p = (char*)ctx->prefill_gd.p;
@@ -709,9 +1030,17 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
   float* Mtq = (float*)p;                   p += (size_t)bh * 32 * d * sizeof(float);
   float* Mtk = (float*)p;                   p += (size_t)bh * 32 * d * sizeof(float);
   float* xq_part = (float*)p;               p += (size_t)bh * Sx * dd * sizeof(float);
-  float* xk_part = (float*)p;
-  hipLaunchKernelGGL(pf_xtx_kernel, dim3((unsigned)Sx, (unsigned)bh), dim3(kXtxThreads), 0, st, (const bf16_t*)q, l,
-                     xq_part, Sx);
+  float* xk_part = (float*)p;               p += (size_t)bkv * Sxk * dd * sizeof(float);
+  if (fused) {
+    float* pq = (float*)p;
+    LRQK_REQUIRE((uintptr_t)q % 16 == 0, LRQK_EINVAL, "rows must be 16-byte aligned");
+    hipLaunchKernelGGL(pf_sums_kernel, dim3((unsigned)Spq, (unsigned)bh), dim3(kXtxThreads), 0, st, (const bf16_t*)q, l,
+                       a_q0, r, pq, xq_part, Spq);
+    partQ = pq;
+  } else {
+    hipLaunchKernelGGL(pf_xtx_kernel, dim3((unsigned)Sx, (unsigned)bh), dim3(kXtxThreads), 0, st, (const bf16_t*)q, l,
+                       xq_part, Sx);
+  }
   hipLaunchKernelGGL(pf_xtx_kernel, dim3((unsigned)Sxk, (unsigned)bkv), dim3(kXtxThreads), 0, st, (const bf16_t*)k, l,
                      xk_part, Sxk);
   LRQK_HIP_CHECK(hipGetLastError());
@@ -723,7 +1052,7 @@ int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float
                                        (int)smem));
     attr = true;
   }
-  GdArgs a{partQ, partK, S, Sq, Sk, G, C, BqT, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol};
+  GdArgs a{partQ, partK, Spq, S, Sq, Sk, G, C, BqT, delta, flags, Mtq, Mtk, b_q, b_k, bh, hq, hkv, r, l, tol};
   const unsigned init_blocks = (unsigned)(((size_t)bh + bkv) * (dd / 256) + (size_t)2 * bh * kGdInitBlocks);
   hipLaunchKernelGGL(pf_gramdom_init_kernel, dim3(init_blocks), dim3(256), 0, st, a, (const float*)xq_part, Sx,
                      (const float*)xk_part, Sxk, bkv, Sq, Sk);

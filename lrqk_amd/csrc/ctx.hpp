@@ -119,8 +119,11 @@ int score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, const
                       bool want_new_idx = true);
 // Prefill iterations on Gram matrices (bf16 input, d = 128, r <= 32); see als_prefill_gram.hip.
 int prefill_gram_domain(lrqk_ctx* ctx, const void* q, const void* k, const float* partQ, const float* partK, int S,
-                        float* b_q, float* b_k, int b, int hq, int hkv, int64_t l, int r, int iters, float tol, int* flags,
-                        float** mt_q, float** mt_k, hipStream_t st);
+                        const float* a_q0, float* b_q, float* b_k, int b, int hq, int hkv, int64_t l, int r, int iters,
+                        float tol, int* flags, float** mt_q, float** mt_k, hipStream_t st);
+// A_K = K Mk with K read once per kv head (bf16 rows of 128); false: no kernel for this head grouping.
+bool prefill_apply_shared(const void* k, const float* mt_k, float* a_k, int b, int hq, int hkv, int64_t l, int r,
+                          hipStream_t st, int* rc_out);
 // The factor update with the ring append of (k_new, v_new) at slot `slot` as token `token` folded
 // into its first kernel.
 int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
