@@ -1032,7 +1032,6 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   float* Mt = partK + n_part;
   float* deltas = Mt + n_mt;
   int* flags = (int*)(deltas + n_delta);
-  LRQK_HIP_CHECK(hipMemsetAsync(flags, 0, (size_t)(iters + 1) * sizeof(int), st));
 
   PfPassFn<T> pass = pf_pass_generic_kernel<T>;
   size_t smem_pass = ((size_t)kPfTile * (d + 1) + (size_t)kPfTile * (r + 1) + (size_t)r * (d + 1)) * sizeof(float);
@@ -1067,6 +1066,8 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   // reading of Q), the K side's by the pass below (A_K has a head per query head, K per kv head)
   const bool gram_domain = sizeof(T) == 2 && mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
   const bool fused_sums = gram_domain && !getenv("LRQK_PREFILL_SEPARATE_SUMS");  // (the Q side's, with Q^T Q)
+  // (the iteration on Gram matrices writes every stopping flag before it reads it)
+  if (!gram_domain) LRQK_HIP_CHECK(hipMemsetAsync(flags, 0, (size_t)(iters + 1) * sizeof(int), st));
   {
     PfPassFn<T> first = pass;  // the sums over the given initial factors
     if constexpr (sizeof(T) == 2) {
