@@ -185,22 +185,24 @@ def prefill_als(a):
     bkv = w.batch * w.num_kv_heads
     if e == 2 and d == 128 and r <= 32 and not os.environ.get("LRQK_PREFILL_ROWWISE"):
         # bf16 rows of 128 elements: the iterations run on d x d Gram matrices (fp64, 32 small independent problems),
-        # and the long axis is read three times whatever the iteration count: initial Grams of the given factors,
-        # X^T X, and the final A = X M.  HBM bytes: 3 x (Q + K, K once per kv head) + the initial factors read
-        # + the final factors written (fp32).
-        bytes_g = 3.0 * (bh + bkv) * l * d * e + 4.0 * bh * l * r * 4
+        # and the long axis is read a fixed number of times whatever the iteration count: Q twice (sums over the
+        # given factors together with Q^T Q; the final A_Q = Q Mq), K three times, once per kv head (sums over the
+        # given factors, K^T K, the final A_K = K Mk).  HBM bytes: those + the initial factors read + the final
+        # factors written (fp32).
+        bytes_g = (2.0 * bh + 3.0 * bkv) * l * d * e + 4.0 * bh * l * r * 4
         gbs = bytes_g / (ms * 1e-3) / 1e9
         # executed bf16 MFMAs of 32x32x16 per 32 rows: 40 per side (initial Grams, three-piece operands),
         # 32 per input head (X^T X), 24 per side (apply)
         exec_flops = (l / 32.0) * (bh * 2 * (40 + 24) + (bh + bkv) * 32) * 2.0 * 32 * 32 * 16
-        roof = {"bound": "hbm", "kernel": "pf_pass_bf16_kernel + pf_xtx_kernel (three readings of the long axis); "
-                                          "pf_gramdom_kernel (fp64 d x d algebra per head, latency-bound) between them",
+        roof = {"bound": "hbm", "kernel": "pf_sums_kernel + pf_pass_bf16_kernel + pf_xtx_kernel + pf_apply_shared_kernel "
+                                          "(two readings of Q, three of K); pf_gramdom_kernel (fp64 d x d algebra per "
+                                          "head, latency-bound) between them",
                 "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                 "traffic": None, "hbm_bytes_per_call": round(bytes_g),
                 "algorithmic_flops_per_call": round(flops), "algorithmic_equiv_tflops": round(tf, 2),
                 "executed_bf16_mfma_tflops": round(exec_flops / (ms * 1e-3) / 1e12, 1),
                 "executed_bf16_mfma_frac": round(exec_flops / (ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
-                "readings_of_the_long_axis": 3, "row_by_row_formulation_readings": 1 + iters}
+                "readings_of_the_long_axis": {"Q": 2, "K": 3}, "row_by_row_formulation_readings": 1 + iters}
     elif e == 2 and d <= 128:
         # bf16 input: the passes run on the bf16 matrix cores (fp32 operands as three bf16 pieces), where the
         # arithmetic is far from any limit; what bounds them is the stream over X and A
