@@ -318,208 +318,6 @@ __global__ __launch_bounds__(kXtxThreads) void pf_sums_kernel(const bf16_t* __re
   }
 }
 
-// ----------------------------------------------------------------------------- the K side's sums, four heads per kv head
-// The four query heads of a kv head factorise the same rows of K, each from its own given A_K.  Side by side
-// their A_K are one l x 128 matrix A4, and their sums are blocks of two products of the X^T X kind:
-//     A4^T K   (128 x 128: rows 32 h .. of it are head h's A_K^T K)      and the diagonal blocks of A4^T A4.
-// So the workgroup stages 128 rows of K per step (bf16, as they are) and of A4 (fp32, split into three bf16 pieces:
-// three more tiles) and its waves own output tiles, each contracting over all rows of the step with operands from
-// the transposing LDS read: wave (h, c) = (w / 2, w % 2) takes A_K[h]^T K column blocks 2 c, 2 c + 1 (three pieces
-// each), the blocks (h, 2 c), (h, 2 c + 1) of K^T K, and of A_K[h]^T A_K[h] the 32-row tiles t with t % 2 = c.
-// A^T A = D + P + P^T with D = hi^T hi + mid^T mid and P = hi^T mid + hi^T lo + mid^T lo (lo^T lo is dropped: 2^-32):
-// five products per k step instead of eight, P is transposed once, at the end.  K is read once per kv head, and
-// K^T K comes out of the same reading.  Every 32-row tile in fresh accumulators.  r % 4 = 0.
-// part: [head][S][r][r + d]; xtx_part: [kv head][S][d][d].  Dynamic LDS: 4 tiles of 128 x 144 bf16.
-constexpr int kSkLd = kXtxD + 16;
-constexpr size_t kSkSmem = (size_t)4 * kXtxRows * kSkLd * sizeof(uint16_t);
-__global__ __launch_bounds__(kXtxThreads) void pf_sums_k4_kernel(const bf16_t* __restrict__ X, int64_t l,
-                                                                 const float* __restrict__ A, int r,
-                                                                 float* __restrict__ part, float* __restrict__ xtx_part,
-                                                                 int S) {
-  extern __shared__ __align__(16) uint16_t sk_s[];
-  uint16_t* x_s = sk_s;                         // [128][kSkLd]   K
-  uint16_t* ap_s = sk_s + kXtxRows * kSkLd;     // [3][128][kSkLd] pieces of A4 (column 32 h + j: head h)
-  const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
-  const int col = lane & 31, half = lane >> 5;
-  const int xh = blockIdx.y, s = blockIdx.x;
-  const bf16_t* Xh = X + (int64_t)xh * l * kXtxD;
-  const int hl = wave >> 1, ch = wave & 1;
-  typedef short gd_v4s __attribute__((ext_vector_type(4)));
-  typedef gd_v4s __attribute__((address_space(3))) * gd_lds_v4s;
-  auto operand = [&](const uint16_t* tile, int row0, int nb) {  // rows row0 + 8 half .. + 7 of column 32 nb + col
-    const int s16 = lane & 15;
-    const uint16_t* p = &tile[(row0 + 8 * half + (s16 >> 2)) * kSkLd + 32 * nb + (col & 16) + 4 * (s16 & 3)];
-    const gd_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)p);
-    const gd_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)(p + 4 * kSkLd));
-    return __builtin_bit_cast(gd_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-  };
-  // K: four 16-byte loads per thread and step, one step ahead; A4: thread (row, head) = (tid / 4, tid % 4) takes the
-  // head's row of the current step (r floats), requested at the start of the step
-  uint4 kx0 = make_uint4(0, 0, 0, 0), kx1 = kx0, kx2 = kx0, kx3 = kx0;
-  auto issue_k = [&](int64_t t0) {
-    auto ld = [&](int i) {
-      const int e = (i * kXtxThreads + tid) * 8;
-      const int64_t row = t0 + e / kXtxD;
-      return *reinterpret_cast<const uint4*>(Xh + min(row, l - 1) * kXtxD + e % kXtxD);
-    };
-    kx0 = ld(0);
-    kx1 = ld(1);
-    kx2 = ld(2);
-    kx3 = ld(3);
-  };
-  auto stage_k = [&](int i, const uint4& v, int64_t t0) {
-    const int e = (i * kXtxThreads + tid) * 8;
-    const int row = e / kXtxD;
-    *reinterpret_cast<uint4*>(&x_s[row * kSkLd + e % kXtxD]) = t0 + row < l ? v : make_uint4(0, 0, 0, 0);
-  };
-  const int arow = tid >> 2, ahead = tid & 3;
-  const float* Ah = A + ((int64_t)xh * 4 + ahead) * l * r;
-  gd_floatx16 accC[2], accX[2], accD, accP;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) accC[0][v] = accC[1][v] = accX[0][v] = accX[1][v] = accD[v] = accP[v] = 0.0f;
-  const int64_t stride = (int64_t)S * kXtxRows;
-  const int64_t first = (int64_t)s * kXtxRows;
-  if (first < l) issue_k(first);
-  for (int64_t t0 = first; t0 < l; t0 += stride) {
-    stage_k(0, kx0, t0);
-    stage_k(1, kx1, t0);
-    stage_k(2, kx2, t0);
-    stage_k(3, kx3, t0);
-    // this thread's row of A4 (clamped; rows beyond l and columns beyond r become zero below)
-    float4 av[8];
-    {
-      const float* src = Ah + min(t0 + arow, l - 1) * r;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) av[j] = *reinterpret_cast<const float4*>(src + min(4 * j, r - 4));
-    }
-    __syncthreads();
-    if (t0 + stride < l) issue_k(t0 + stride);
-    const int tiles = (int)min((int64_t)4, (l - t0 + 31) / 32);
-    // the blocks of K^T K (they need the K tile only: the rows of A4 arrive meanwhile)
-    for (int tile = 0; tile < tiles; ++tile) {
-      gd_floatx16 t0a, t1a;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) t0a[v] = t1a[v] = 0.0f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const int row0 = 32 * tile + 16 * kb;
-        const gd_bf16x8 a = operand(x_s, row0, hl);
-        const gd_bf16x8 b0 = operand(x_s, row0, 2 * ch), b1 = operand(x_s, row0, 2 * ch + 1);
-        t0a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, t0a, 0, 0, 0);
-        t1a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, t1a, 0, 0, 0);
-      }
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        accX[0][v] += t0a[v];
-        accX[1][v] += t1a[v];
-      }
-    }
-    // the three pieces of this thread's row of A4 into their tiles
-    {
-      const bool row_ok = t0 + arow < l;
-#pragma unroll
-      for (int j8 = 0; j8 < 4; ++j8) {  // eight columns at a time
-        uint32_t pc[3][8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const int c = 8 * j8 + q;
-          const float4 f4 = av[c >> 2];
-          const float x = (c & 3) == 0 ? f4.x : (c & 3) == 1 ? f4.y : (c & 3) == 2 ? f4.z : f4.w;
-          gd_split3(row_ok && c < r ? x : 0.0f, pc[0][q], pc[1][q], pc[2][q]);
-        }
-#pragma unroll
-        for (int pp = 0; pp < 3; ++pp)
-          *reinterpret_cast<uint4*>(&ap_s[(pp * kXtxRows + arow) * kSkLd + 32 * ahead + 8 * j8]) =
-              make_uint4(gd_pack2(pc[pp][0], pc[pp][1]), gd_pack2(pc[pp][2], pc[pp][3]), gd_pack2(pc[pp][4], pc[pp][5]),
-                         gd_pack2(pc[pp][6], pc[pp][7]));
-      }
-    }
-    __syncthreads();
-    const uint16_t* a0 = ap_s;
-    const uint16_t* a1 = ap_s + kXtxRows * kSkLd;
-    const uint16_t* a2 = ap_s + 2 * kXtxRows * kSkLd;
-    for (int tile = 0; tile < tiles; ++tile) {
-      gd_floatx16 tc0, tc1;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) tc0[v] = tc1[v] = 0.0f;
-      const bool mine = (tile & 1) == ch;  // (wave-uniform) this wave's share of A^T A
-      gd_floatx16 td, tp;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) td[v] = tp[v] = 0.0f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const int row0 = 32 * tile + 16 * kb;
-        const gd_bf16x8 p0 = operand(a0, row0, hl), p1 = operand(a1, row0, hl), p2 = operand(a2, row0, hl);
-        const gd_bf16x8 b0 = operand(x_s, row0, 2 * ch), b1 = operand(x_s, row0, 2 * ch + 1);
-        tc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, b0, tc0, 0, 0, 0);
-        tc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, b1, tc1, 0, 0, 0);
-        tc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, b0, tc0, 0, 0, 0);
-        tc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, b1, tc1, 0, 0, 0);
-        tc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p0, b0, tc0, 0, 0, 0);
-        tc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p0, b1, tc1, 0, 0, 0);
-        if (mine) {
-          tp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, p2, tp, 0, 0, 0);
-          tp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p0, p2, tp, 0, 0, 0);
-          tp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p0, p1, tp, 0, 0, 0);
-          td = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, p1, td, 0, 0, 0);
-          td = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p0, p0, td, 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        accC[0][v] += tc0[v];
-        accC[1][v] += tc1[v];
-        accD[v] += td[v];
-        accP[v] += tp[v];
-      }
-    }
-    __syncthreads();
-  }
-  {
-    float* out = xtx_part + ((int64_t)xh * S + s) * kXtxD * kXtxD;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int i = 32 * hl + gd_mfma_row(lane, v);
-      out[i * kXtxD + 32 * (2 * ch) + col] = accX[0][v];
-      out[i * kXtxD + 32 * (2 * ch + 1) + col] = accX[1][v];
-    }
-  }
-  const int ne = r * (r + kXtxD);
-  float* outp = part + (((int64_t)xh * 4 + hl) * S + s) * ne;
-  // A_K[h]^T K: this wave owns its two column blocks
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int m = gd_mfma_row(lane, v);
-    if (m < r) {
-      outp[m * (r + kXtxD) + r + 32 * (2 * ch) + col] = accC[0][v];
-      outp[m * (r + kXtxD) + r + 32 * (2 * ch + 1) + col] = accC[1][v];
-    }
-  }
-  // A_K[h]^T A_K[h] = sum over the head's two waves of D + P + P^T, through LDS (the tiles are no longer needed)
-  float* sm = reinterpret_cast<float*>(sk_s);
-  {
-    float* mine_d = sm + (wave * 2 + 0) * 1024;
-    float* mine_p = sm + (wave * 2 + 1) * 1024;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      mine_d[gd_mfma_row(lane, v) * 32 + col] = accD[v];
-      mine_p[gd_mfma_row(lane, v) * 32 + col] = accP[v];
-    }
-  }
-  __syncthreads();
-  for (int o = tid; o < 4 * 1024; o += kXtxThreads) {
-    const int h = o >> 10, e = o & 1023, m = e >> 5, n = e & 31;
-    float v = 0.0f;
-#pragma unroll
-    for (int c2 = 0; c2 < 2; ++c2) {
-      const float* d_t = sm + ((2 * h + c2) * 2 + 0) * 1024;
-      const float* p_t = sm + ((2 * h + c2) * 2 + 1) * 1024;
-      v += d_t[m * 32 + n] + p_t[m * 32 + n] + p_t[n * 32 + m];
-    }
-    if (m < r && n < r) part[(((int64_t)xh * 4 + h) * S + s) * ne + m * (r + kXtxD) + n] = v;
-  }
-}
-
 // ----------------------------------------------------------------------------- A = X Mt^T for heads that share X
 // The K side's last pass: the NH query heads of a kv head take their rows of A_K from the same rows of K, so one
 // workgroup stages 128 rows of K per step (as pf_xtx_kernel does) and applies the NH heads' Mt to them: K is read
