@@ -666,7 +666,9 @@ def test_als_prefill_long_sums(ops, ws, oracle):
                           (torch.bfloat16, 4, 2, 2000, 128, 16, 3, 0.0), (torch.bfloat16, 2, 1, 1500, 128, 24, 1, 0.0),
                           (torch.bfloat16, 2, 1, 1200, 128, 32, 6, 1e30), (torch.bfloat16, 4, 2, 1500, 128, 20, 6, 5e-2),
                           # head groupings: one query head per kv head and eight (the last pass then goes head by head)
-                          (torch.bfloat16, 2, 2, 900, 128, 32, 2, 0.0), (torch.bfloat16, 8, 1, 1100, 128, 16, 2, 0.0)])
+                          (torch.bfloat16, 2, 2, 900, 128, 32, 2, 0.0), (torch.bfloat16, 8, 1, 1100, 128, 16, 2, 0.0),
+                          # a rank that is no multiple of the four pivots of an elimination step
+                          (torch.bfloat16, 4, 1, 600, 128, 6, 2, 0.0)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
