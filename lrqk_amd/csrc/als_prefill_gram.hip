@@ -192,6 +192,11 @@ __global__ __launch_bounds__(kXtxThreads) void pf_sums_kernel(const bf16_t* __re
   float arow[16];  // this wave's rows of A of the step being multiplied, requested at the start of the step
   auto step = [&](int64_t t0, uint4 (&cur)[NL]) {
 #pragma unroll
+    for (int v = 0; v < 16; ++v) {  // (requested first, consumed after the blocks of X^T X below)
+      const int64_t row = min(t0 + 32 * wa + gd_mfma_row(lane, v), l - 1);
+      arow[v] = Ah[row * r + min(col, r - 1)];
+    }
+#pragma unroll
     for (int i = 0; i < NL; ++i) {
       const int e = (i * kXtxThreads + tid) * 8;
       const int row = e / kXtxD;
@@ -199,11 +204,6 @@ __global__ __launch_bounds__(kXtxThreads) void pf_sums_kernel(const bf16_t* __re
     }
     __syncthreads();
     if (t0 + stride < l) issue(t0 + stride, cur);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {  // (consumed after the blocks of X^T X below)
-      const int64_t row = min(t0 + 32 * wa + gd_mfma_row(lane, v), l - 1);
-      arow[v] = Ah[row * r + min(col, r - 1)];
-    }
     const int tiles = (int)min((int64_t)4, (l - t0 + 31) / 32);
     for (int tile = 0; tile < tiles; ++tile) {
       gd_floatx16 t0a, t1a;
