@@ -287,7 +287,7 @@ __global__ __launch_bounds__(kXtxThreads) void pf_sums_kernel(const bf16_t* __re
       out[i * kXtxD + 32 * (nb2 + 1) + col] = acc1[v];
     }
   }
-  // the waves' sums: round 0 is A^T A (all waves), rounds 1, 2 the column blocks 2 ch + 0 / + 1 of A^T X (the waves
+  // the waves' sums: pass 0 is A^T A (all waves), passes 1, 2 the column blocks 2 ch + 0 / + 1 of A^T X (the waves
   // with the same ch)
   float* sm = reinterpret_cast<float*>(x_s);
   const int ne = r * (r + kXtxD);

@@ -31,8 +31,8 @@ def _rel(a, b):
     return float((a - b).norm() / (b.norm() + 1e-300))
 
 
-# Largest deviation seen per (trace, quantity) in this session: printed (and written next to the other GPU
-# results when that folder exists) so that every tolerance below can be read against what was measured.
+# Largest deviation seen per (trace, quantity) in this session: printed (and written as JSON into the directory
+# that LRQK_PARITY_OUT names, if it is set) so that every tolerance below can be read against what was measured.
 DEVIATIONS = {}
 
 
@@ -52,8 +52,8 @@ def _report_deviations():
     import os
     lines = [f"  {k}: {v:.3e}" for k, v in sorted(DEVIATIONS.items())]
     print("\nmeasured deviations (max over steps):\n" + "\n".join(lines), flush=True)
-    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
-    if os.path.isdir(out):
+    out = os.environ.get("LRQK_PARITY_OUT", "")
+    if out and os.path.isdir(out):
         with open(os.path.join(out, "parity_deviations_engine.json"), "w") as f:
             json.dump(DEVIATIONS, f, indent=1, sort_keys=True)
 
