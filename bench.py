@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # workload at its default context (the scaling factors come from this library's own probe kernels of known size in
 # the same runs).  The summary of those runs is kept under profiles/.
 # Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
-# 8-bit copy (36 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
+# 8-bit copy (34 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
 MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (83860.8 * 2.000 + 867.4 * 1.000) * 1024,
                           ("llama8b_128k_bf16", False): (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
 
@@ -482,10 +482,10 @@ def main():
 
     sidx_on = (not a.no_score_index) and w.r in (16, 32, 64)
     # Bytes one launch of the scan has to move.  Without the score index: the A_K rows.  With it: the 8-bit copy
-    # (r + 4 bytes per row) plus the rows it rescores exactly from A_K (counted by the kernel; last launch) plus
+    # (r + 2 bytes per row) plus the rows it rescores exactly from A_K (counted by the kernel; last launch) plus
     # the candidate pairs it writes -- fewer bytes than the reference's scan reads, which is the point of it.
     if sidx_on and rows_scanned:
-        must_move = bh * m_avg * (w.r + 4) + rows_rescored * w.r * e + 8.0 * rows_rescored
+        must_move = bh * m_avg * (w.r + 2) + rows_rescored * w.r * e + 8.0 * rows_rescored
     else:
         must_move = scan_bytes
     achieved = must_move / (kern_us * 1e-6) / 1e9 if launches else 0.0

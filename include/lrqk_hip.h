@@ -132,7 +132,7 @@ int lrqk_ctx_set_fetch_mode(lrqk_ctx* ctx, int mode, int host_threads);
 
 /* Score index for the scan (no counterpart in the reference; a new ctx has it off, the Python
  * engine switches it on).  The ctx keeps an
- * 8-bit copy of the A_K rows (one scale per row, 36 instead of 64 bytes per row for r = 32) and the
+ * 8-bit copy of the A_K rows (one 16-bit scale per row, 34 instead of 64 bytes per row for r = 32) and the
  * scan of lrqk_score_select / lrqk_score_select_diff / lrqk_decode_step reads that copy: it bounds
  * every row's score and rescores exactly, from a_k itself, only the rows whose bound reaches the
  * filter threshold.  Results are identical.  The copy is built on demand for rows [0, m) and

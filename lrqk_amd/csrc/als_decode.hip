@@ -691,7 +691,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
       ctx->sidx_head_rows == head_stride / r && ctx->sidx_dtype == (sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16)) {
     // the appended row also goes into the score index; rows stay contiguous as long as rows are appended in order
     fa.qa = (uint8_t*)ctx->sidx_qa.p;
-    fa.qs = (float*)ctx->sidx_qs.p;
+    fa.qs = (uint16_t*)ctx->sidx_qs.p;
     fa.qw = (const float*)ctx->sidx_wm.p;
     fa.q_head_rows = ctx->sidx_head_rows;
     if (append_row == ctx->sidx_valid) ctx->sidx_valid = append_row + 1;  // (a gap is indexed on demand later)

@@ -63,7 +63,7 @@ struct FinishArgs {
   void* a_k;
   int64_t head_stride, append_row;
   uint8_t* qa;       // score index (8-bit copy of A_K) to extend with the appended row, or nullptr
-  float* qs;
+  uint16_t* qs;      // its rows' scales (fp16 bit patterns)
   const float* qw;   // its per-head transforms [bh][r*r + r]
   int64_t q_head_rows;
 };
@@ -83,7 +83,7 @@ __device__ __forceinline__ void als_index_append_rows(const FinishArgs& fa, int 
   float scale;
   const uint8_t u = score_index_encode_row<R>(v, wcol, &scale);
   if (lane < R) fa.qa[((int64_t)h * fa.q_head_rows + fa.append_row) * R + lane] = u;
-  if (lane == 0) fa.qs[(int64_t)h * fa.q_head_rows + fa.append_row] = scale;
+  if (lane == 0) fa.qs[(int64_t)h * fa.q_head_rows + fa.append_row] = sidx_scale_bits(scale);
 }
 template <typename T>
 __device__ __forceinline__ void als_index_append_body(const FinishArgs& fa, int h) {

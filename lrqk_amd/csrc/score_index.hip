@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void score_index_factor_kernel(const float* __
 template <typename T, int R>
 __global__ __launch_bounds__(256) void score_index_build_kernel(const T* __restrict__ a_k, int64_t head_stride,
                                                                 int64_t row0, int64_t row1, uint8_t* __restrict__ qa,
-                                                                float* __restrict__ qs, const float* __restrict__ wm,
+                                                                uint16_t* __restrict__ qs, const float* __restrict__ wm,
                                                                 int64_t head_rows) {
   const int h = blockIdx.y;
   const int lane = lane_id();
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void score_index_build_kernel(const T* __restr
     float scale;
     const uint8_t u = score_index_encode_row<R>(v, wcol, &scale);
     if (lane < R) qa[((int64_t)h * head_rows + row) * R + lane] = u;
-    if (lane == 0) qs[(int64_t)h * head_rows + row] = scale;
+    if (lane == 0) qs[(int64_t)h * head_rows + row] = sidx_scale_bits(scale);
   }
 }
 
@@ -154,7 +154,7 @@ typedef float sidx_v16f __attribute__((ext_vector_type(16)));
 template <typename T>
 __global__ __launch_bounds__(256) void score_index_build32_kernel(const T* __restrict__ a_k, int64_t head_stride,
                                                                   int64_t row0, int64_t row1, uint8_t* __restrict__ qa,
-                                                                  float* __restrict__ qs, const float* __restrict__ wm,
+                                                                  uint16_t* __restrict__ qs, const float* __restrict__ wm,
                                                                   int64_t head_rows) {
   constexpr int R = 32, VEC = Vec16<T>::N;
   const int h = blockIdx.y;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void score_index_build32_kernel(const T* __res
       const int64_t orow = r0 + (v >> 2) * 8 + kh * 4 + (v & 3);
       if (orow < row1) {
         qa[((int64_t)h * head_rows + orow) * R + m] = u;
-        if (m == 0) qs[(int64_t)h * head_rows + orow] = scale;
+        if (m == 0) qs[(int64_t)h * head_rows + orow] = sidx_scale_bits(scale);
       }
     }
   }
@@ -223,12 +223,12 @@ static void launch_build(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, in
   if (R == 32 && upto - from >= 32) {
     const unsigned blocks = (unsigned)std::min<int64_t>(1024, (upto - from + 127) / 128);
     hipLaunchKernelGGL((score_index_build32_kernel<T>), dim3(blocks, (unsigned)bh), dim3(256), 0, st, (const T*)a_k,
-                       head_stride, from, upto, (uint8_t*)ctx->sidx_qa.p, (float*)ctx->sidx_qs.p, wm, head_rows);
+                       head_stride, from, upto, (uint8_t*)ctx->sidx_qa.p, (uint16_t*)ctx->sidx_qs.p, wm, head_rows);
     return;
   }
   const unsigned blocks = (unsigned)std::min<int64_t>(2048, (upto - from + 3) / 4);
   hipLaunchKernelGGL((score_index_build_kernel<T, R>), dim3(blocks, (unsigned)bh), dim3(256), 0, st, (const T*)a_k,
-                     head_stride, from, upto, (uint8_t*)ctx->sidx_qa.p, (float*)ctx->sidx_qs.p, wm, head_rows);
+                     head_stride, from, upto, (uint8_t*)ctx->sidx_qa.p, (uint16_t*)ctx->sidx_qs.p, wm, head_rows);
 }
 
 int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t m, int r, int dtype,
@@ -242,7 +242,7 @@ int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int
   if (!bound) {
     int rc;
     if ((rc = ctx->sidx_qa.ensure((size_t)bh * head_rows * r))) return rc;
-    if ((rc = ctx->sidx_qs.ensure((size_t)bh * head_rows * sizeof(float)))) return rc;
+    if ((rc = ctx->sidx_qs.ensure((size_t)bh * head_rows * sizeof(uint16_t)))) return rc;
     if ((rc = ctx->sidx_wm.ensure((size_t)bh * (r * r + r) * sizeof(float)))) return rc;
     if ((rc = ctx->sidx_part.ensure((size_t)bh * kSidxParts * r * r * sizeof(float)))) return rc;
     ctx->sidx_a_k = a_k;
@@ -269,7 +269,7 @@ int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int
     ctx->sidx_valid = upto;
   }
   view->qa = (const uint8_t*)ctx->sidx_qa.p;
-  view->qs = (const float*)ctx->sidx_qs.p;
+  view->qs = (const uint16_t*)ctx->sidx_qs.p;
   view->wm = (const float*)ctx->sidx_wm.p;
   view->head_rows = head_rows;
   return 1;

@@ -1,5 +1,5 @@
 // Score index: an 8-bit copy of the A_K rows, in whitened coordinates, that lets the proxy-score
-// scan read 36 instead of 64 bytes per cached token.  The scan bounds every row's score from the
+// scan read 34 instead of 64 bytes per cached token.  The scan bounds every row's score from the
 // copy and rescores exactly (from A_K itself) only the rows whose bound reaches the filter
 // threshold, so the candidate list -- and everything after it -- is unchanged.
 //
@@ -28,7 +28,7 @@ constexpr float kSidxDFactor = 0.511f;
 
 struct ScoreIndexView {
   const uint8_t* qa;  // [bh][head_rows][r]
-  const float* qs;    // [bh][head_rows]
+  const uint16_t* qs; // [bh][head_rows] the rows' scales as fp16 bit patterns (score_index_scale returns such values)
   const float* wm;    // [bh][r*r + r]: W row-major (zeros below the diagonal), then 1 / W_jj
   int64_t head_rows;  // rows per head of qa and qs (= rows per head of A_K)
 };
@@ -36,9 +36,20 @@ struct ScoreIndexView {
 // Scale of a row from max_j |a'_j| and max_j g_j.  The floor keeps the bound above anything a
 // flush of subnormal products could lose (r * 1.2e-38 per element); a row with a NaN or an
 // infinity gets a NaN scale, which makes the scan rescore it exactly every time.
+// The scale is stored in 16 bits: any scale at least as large as the one required keeps the bound valid (the codes
+// are formed with the stored value), so it is rounded up to the next fp16 number (at most 0.1 % more; +infinity
+// beyond the fp16 range, which like the NaN makes the scan rescore the row every time).
+__device__ __forceinline__ float sidx_round_up_f16(float x) {
+  _Float16 h = (_Float16)x;
+  if ((float)h < x) h = __builtin_bit_cast(_Float16, (uint16_t)(__builtin_bit_cast(uint16_t, h) + 1));  // (x > 0)
+  return (float)h;
+}
+__device__ __forceinline__ uint16_t sidx_scale_bits(float scale) { return __builtin_bit_cast(uint16_t, (_Float16)scale); }
+__device__ __forceinline__ float sidx_scale_from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 __device__ __forceinline__ float score_index_scale(float row_max, float g_max, int r) {
   const float coef = 5.0f * (float)(r + 2) * 5.9604645e-8f * (1.000001f / kSidxBeta);
   float scale = fmaxf(fmaxf(row_max * (1.0f / 127.0f), g_max * coef), 1e-30f);
+  scale = sidx_round_up_f16(scale);
   if (!(g_max < INFINITY)) scale = NAN;
   return scale;
 }

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
 
 // --------------------------------------------------------------------------- score + filter through the score index
 // Same output as score_filter_kernel (the candidate list of all rows with key >= bound), read from
-// the 8-bit copy of A_K in whitened coordinates: 36 bytes per row instead of 64.  Every wave solves
+// the 8-bit copy of A_K in whitened coordinates: 34 bytes per row instead of 64.  Every wave solves
 // W q' = q (back substitution, lane i holds row i of W; q' ends up in scalar registers); for every
 // row an upper bound of its (rounded) score follows from the copy:
 //   |score - s~| <= D = scale * |q'|_1 * kSidxDFactor,   s~ = scale * sum_j (u_j - 128) q'_j
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
   const int tid = threadIdx.x, lane = lane_id();
   const T* A = a_k + (int64_t)h * head_stride;
   const uint8_t* QA = six.qa + (int64_t)h * six.head_rows * R;
-  const float* QS = six.qs + (int64_t)h * six.head_rows;
+  const uint16_t* QS = six.qs + (int64_t)h * six.head_rows;
   RowScorer<T, R> rs;
   if (tid == 0) {
     l_count = 0;
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     const int64_t i = min(base0 + it * kFiltThreads + tid, m - 1);
 #pragma unroll
     for (int c = 0; c < QV; ++c) pre[it][c] = reinterpret_cast<const uint4*>(QA + i * R)[c];
-    pre_s[it] = QS[i];
+    pre_s[it] = sidx_scale_from_bits(QS[i]);
   }
   if (pending) {
     const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
         uint4 row[QV];
 #pragma unroll
         for (int c = 0; c < QV; ++c) row[c] = reinterpret_cast<const uint4*>(QA + ic * R)[c];
-        ub = bound_of(row, QS[ic]);
+        ub = bound_of(row, sidx_scale_from_bits(QS[ic]));
       }
       if (any && i < m && !(ub < thr_lo)) mask |= 1u << it;
     }
