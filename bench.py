@@ -492,9 +492,12 @@ def main():
     traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) \
         if a.context is None and a.variant == "default" and w.batch == 1 else None
 
-    read_gbs = copy_gbs = None
+    read_gbs = copy_gbs = pair_us = None
     if a.probe_mb > 0:
         read_gbs, copy_gbs = ops_mod.probe_bandwidth(a.probe_mb << 20, 10, dev)
+        # what the same event bracket reads around a kernel that does nothing: the share of kernel_us that
+        # is the two event packets and the launch itself (a profiler's kernel duration has neither)
+        pair_us = ops_mod.probe_event_pair(64, dev)
 
     if a.calib_copy_mb > 0:
         src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -558,6 +561,7 @@ def main():
                      "traffic": round(traffic) if traffic else None,
                      "traffic_gbs": round(traffic / (kern_us * 1e-6) / 1e9, 1) if traffic and launches else None,
                      "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(must_move),
+                     "event_pair_around_empty_kernel_us": round(pair_us, 2) if pair_us is not None else None,
                      "rows_rescored_per_launch": rows_rescored,
                      "algorithmic_bytes_per_launch": round(scan_bytes),
                      "algorithmic_equiv_gbs": round(scan_bytes / (kern_us * 1e-6) / 1e9, 1) if launches else None,

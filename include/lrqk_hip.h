@@ -246,6 +246,10 @@ int lrqk_timing_read(lrqk_ctx* ctx, double* total_ms, int* launches);
  * src, dst: device memory, 16-byte aligned, bytes a multiple of 16. */
 int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, int reps, double* read_ms, double* copy_ms,
                          void* stream);
+/* No counterpart in the reference.  What a pair of HIP events reads around a kernel that does nothing (average
+ * microseconds over `reps` <= 256 pairs on the caller's stream, each pair between two other launches; waits for the
+ * stream): the part of an event-bracketed kernel time (lrqk_timing_read) that is not the kernel. */
+int lrqk_probe_event_pair(int reps, double* pair_us, void* stream);
 
 /* Host-side row gathers with the reference's native signatures (the staged fetch path
  * and API parity); multi-threaded memcpy.

@@ -37,9 +37,48 @@ __global__ __launch_bounds__(kProbeThreads) void probe_copy_kernel(const uint4* 
   }
 }
 
+// Does nothing: what a pair of events around a launch reads when the kernel itself takes no time.
+__global__ void probe_empty_kernel() {}
+
 }  // namespace lrqk
 
 using namespace lrqk;
+
+extern "C" int lrqk_probe_event_pair(int reps, double* pair_us, void* stream) {
+  LRQK_REQUIRE(pair_us != nullptr && reps > 0 && reps <= 256, LRQK_EINVAL, "bad arguments reps=%d", reps);
+  hipStream_t st = (hipStream_t)stream;
+  hipEvent_t* ev = new hipEvent_t[2 * (size_t)reps];
+  int made = 0, rc = LRQK_OK;
+  for (; made < 2 * reps; ++made) {
+    if (hipEventCreate(&ev[made]) != hipSuccess) {
+      rc = LRQK_EHIP;
+      break;
+    }
+  }
+  double sum = 0.0;
+  if (rc == LRQK_OK) {
+    // as in the timed step: a kernel before the pair, the bracketed launch, a kernel after it
+    for (int i = 0; i < reps && rc == LRQK_OK; ++i) {
+      hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, st);
+      if (hipEventRecord(ev[2 * i], st) != hipSuccess) rc = LRQK_EHIP;
+      hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, st);
+      if (hipEventRecord(ev[2 * i + 1], st) != hipSuccess) rc = LRQK_EHIP;
+      hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, st);
+    }
+    if (rc == LRQK_OK && hipStreamSynchronize(st) != hipSuccess) rc = LRQK_EHIP;
+    for (int i = 0; i < reps && rc == LRQK_OK; ++i) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = LRQK_EHIP;
+      sum += ms;
+    }
+  }
+  for (int i = 0; i < made; ++i) (void)hipEventDestroy(ev[i]);
+  delete[] ev;
+  (void)hipGetLastError();
+  LRQK_REQUIRE(rc == LRQK_OK, LRQK_EHIP, "HIP event calls failed");
+  *pair_us = sum * 1e3 / reps;
+  return LRQK_OK;
+}
 
 extern "C" int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, int reps, double* read_ms,
                                     double* copy_ms, void* stream) {

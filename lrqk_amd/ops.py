@@ -369,6 +369,14 @@ def probe_bandwidth(nbytes: int, reps: int = 10, device="cuda:0"):
     return nbytes / (r_ms.value * 1e-3) / 1e9, 2 * nbytes / (c_ms.value * 1e-3) / 1e9
 
 
+def probe_event_pair(reps: int = 64, device="cuda:0") -> float:
+    """Microseconds that a pair of HIP events reads around a kernel that does nothing (average of ``reps`` pairs)."""
+    us = ctypes.c_double()
+    with torch.cuda.device(device):
+        check(_lib.load().lrqk_probe_event_pair(reps, ctypes.byref(us), torch.cuda.current_stream().cuda_stream))
+    return us.value
+
+
 # --------------------------------------------------------------------------- host gathers
 
 def d0_index_select(src: torch.Tensor, indices: torch.Tensor, threads: int = 8) -> torch.Tensor:
