@@ -129,11 +129,13 @@ __device__ __forceinline__ void attn_scan_w(const float* __restrict__ w, float s
   }
 }
 
-// Merges the lane groups of a wave, then the waves of the workgroup; afterwards threads c < d + 2
-// hold element c of the workgroup's (m, l, acc[d]) triple in the return value.
+// Merges the lane groups of a wave, then the waves of the workgroup, and writes the workgroup's (m, l, acc[d])
+// triple to pout[0 .. d + 2): thread t writes element t, and the first threads also the elements beyond the
+// workgroup's thread count (d + 2 exceeds it for rows of 256 elements).
 // red: [NW][2 + 256] floats of LDS.
 template <int VEC, int NW>
-__device__ __forceinline__ float attn_block_merge(AttnAcc<VEC>& st, int lpr_log2, int d, float (*red)[2 + 256]) {
+__device__ __forceinline__ void attn_block_merge(AttnAcc<VEC>& st, int lpr_log2, int d, float (*red)[2 + 256],
+                                                 float* __restrict__ pout) {
   const int lane = lane_id(), wave = wave_id();
   const int lpr = 1 << lpr_log2;
   const int sub = lane & (lpr - 1);
@@ -164,18 +166,19 @@ __device__ __forceinline__ float attn_block_merge(AttnAcc<VEC>& st, int lpr_log2
   float M = -INFINITY;
 #pragma unroll
   for (int w = 0; w < NW; ++w) M = fmaxf(M, red[w][0]);
-  float v = 0.0f;
-  const int c = threadIdx.x;
-  if (c == 0) {
-    v = M;
-  } else if (c < d + 2) {
+  for (int c = threadIdx.x; c < d + 2; c += NW * kWave) {
+    float v = 0.0f;
+    if (c == 0) {
+      v = M;
+    } else {
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const float f = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
-      v += red[w][c] * f;
+      for (int w = 0; w < NW; ++w) {
+        const float f = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
+        v += red[w][c] * f;
+      }
     }
+    pout[c] = v;
   }
-  return v;
 }
 
 template <typename T>
@@ -228,8 +231,7 @@ __device__ __forceinline__ void attn_partial_body(const T* __restrict__ q, const
       return i;
     }, st);
   }
-  const float v = attn_block_merge<VEC, kAttnWaves>(st, lpr_log2, d, red);
-  if ((int)threadIdx.x < d + 2) part[((int64_t)h * stride_s + s) * (d + 2) + threadIdx.x] = v;
+  attn_block_merge<VEC, kAttnWaves>(st, lpr_log2, d, red, part + ((int64_t)h * stride_s + s) * (d + 2));
 }
 
 template <typename T>
@@ -407,7 +409,10 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
   }
   // merge the row groups: V lane (jl, cv) owns columns cv*VEC .. of group jl
   const int groups = rpb;  // <= 8 for rows of >= 512 bytes; larger counts are merged in rounds of 8
-  float M = -INFINITY, Lsum = 0.0f, col = 0.0f;  // thread t < d + 2 accumulates element t of the result
+  // thread t accumulates element t of the result (m, l, acc[d]); threads 0 and 1 also the two elements beyond
+  // the workgroup's thread count that rows of 256 elements have
+  const int tid2 = tid + kAttnThreads;
+  float M = -INFINITY, Lsum = 0.0f, col = 0.0f, col2 = 0.0f;
   for (int g0 = 0; g0 < groups; g0 += 8) {
     __syncthreads();
     if (!is_k && jl >= g0 && jl < g0 + 8 && jl < groups) {
@@ -426,14 +431,17 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
     const float a_old = (Mg == -INFINITY) ? 0.0f : exp2f(M - Mg);
     Lsum *= a_old;
     col *= a_old;
+    col2 *= a_old;
     for (int g = 0; g < ng; ++g) {
       const float fg = (Mg == -INFINITY || accs[g][0] == -INFINITY) ? 0.0f : exp2f(accs[g][0] - Mg);
       Lsum = fmaf(accs[g][1], fg, Lsum);
       if (tid >= 2 && tid < d + 2) col = fmaf(accs[g][tid], fg, col);
+      if (tid2 < d + 2) col2 = fmaf(accs[g][tid2], fg, col2);
     }
     M = Mg;
   }
   if (tid < d + 2) pout[tid] = tid == 0 ? M : (tid == 1 ? Lsum : col);
+  if (tid2 < d + 2) pout[tid2] = col2;
 }
 
 // Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their

@@ -412,6 +412,17 @@ def test_qwen_shape_fp32_short(lrqk, oracle):
     assert n > 0
 
 
+@pytest.mark.parametrize("hq,hkv,d,r,k,L,l", [(8, 2, 64, 16, 128, 8, 700), (4, 1, 256, 32, 256, 16, 1200)])
+def test_other_head_widths(lrqk, oracle, hq, hkv, d, r, k, L, l):
+    """bf16 heads of 64 and 256 elements (rows of 128 and 512 bytes): the kernels written for rows of 128 elements
+    do not take these, so the whole trace runs on the general ones -- with the score index, whose ranks 16 and 32
+    do not depend on the head width."""
+    _say("head width", d)
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=hq, hkv=hkv, d=d, l=l, r=r, k=k, L=L, steps=30, dtype=torch.bfloat16,
+                        max_iter=(2, 2), tol=(1e-8, 1e-8), rho=2 * r, capacity=2048, tag="d%d" % d)
+    assert n > 0
+
+
 def test_llama_shape_bf16_short(lrqk, oracle):
     """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, r 32, k 2048, L 64, bf16) at an
     8K context, long enough (70 steps) for the 64-token ring to be flushed to the host store once."""

@@ -512,7 +512,9 @@ def test_gather_append_flush(ops, oracle):
 # ---------------------------------------------------------------- attention
 
 @pytest.mark.parametrize("dtype,d,n", [(torch.bfloat16, 128, 2112), (torch.float32, 128, 544), (torch.float32, 16, 12),
-                                       (torch.bfloat16, 64, 1), (torch.float32, 8, 100)])
+                                       (torch.bfloat16, 64, 1), (torch.float32, 8, 100),
+                                       # other head widths: 64 (eight lanes per row) and 256 (a row fills half a wave)
+                                       (torch.bfloat16, 64, 300), (torch.bfloat16, 256, 500), (torch.float32, 256, 130)])
 def test_attention(ops, ws, oracle, dtype, d, n):
     _say("attention", dtype, d, n)
     g = torch.Generator().manual_seed(n)
@@ -542,7 +544,10 @@ def _als_inputs(g, b, hq, hkv, n, d, r, cap, dtype):
 
 
 @pytest.mark.parametrize("dtype,hq,hkv,n,d,r", [(torch.float32, 4, 2, 12, 16, 4), (torch.float32, 28, 4, 544, 128, 16),
-                                                (torch.bfloat16, 32, 8, 2112, 128, 32), (torch.float32, 2, 2, 70, 8, 3)])
+                                                (torch.bfloat16, 32, 8, 2112, 128, 32), (torch.float32, 2, 2, 70, 8, 3),
+                                                # head widths 64 and 256 (bf16 rows that the d = 128 kernel does not take)
+                                                (torch.bfloat16, 8, 2, 300, 64, 16), (torch.bfloat16, 4, 1, 272, 256, 32),
+                                                (torch.float32, 4, 2, 150, 64, 8)])
 @pytest.mark.parametrize("max_iter,tol", [(1, 0.0), (2, 0.0), (3, 1e30), (4, 1e-6)])
 def test_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol)
@@ -727,3 +732,15 @@ def test_als_prefill_benchmark_configuration(ops, ws, oracle):
     print("  residual K: kernel %.6f oracle %.6f; residual Q: kernel %.6f oracle %.6f" % (res_g, res_o, resq_g, resq_o),
           flush=True)
     assert abs(res_g - res_o) < 1e-4 and abs(resq_g - resq_o) < 1e-4
+
+
+def test_measurement_probes(ops):
+    """The plain read / copy kernels and the event-pair calibration that the bench line carries: the copy
+    really copies, the rates and the bracket are finite and of a plausible order of magnitude."""
+    print("probes: bandwidth + event pair", flush=True)
+    read_gbs, copy_gbs = ops.probe_bandwidth(64 << 20, 3, DEV)
+    assert 50.0 < read_gbs < 20000.0 and 50.0 < copy_gbs < 20000.0, (read_gbs, copy_gbs)
+    pair = ops.probe_event_pair(16, DEV)
+    assert 0.0 < pair < 500.0, pair
+    with pytest.raises(ValueError):
+        ops.probe_event_pair(0, DEV)
