@@ -423,6 +423,15 @@ def test_other_head_widths(lrqk, oracle, hq, hkv, d, r, k, L, l):
     assert n > 0
 
 
+def test_active_set_beyond_the_fused_diff(lrqk, oracle):
+    """k = 4200 resident tokens: more than the select kernel's in-kernel diff takes (4096), so the step runs the
+    ordered selection, a separate diff launch and the fetch without the victim cache."""
+    _say("k = 4200 trace")
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=128, l=9000, r=16, k=4200, L=32, steps=12,
+                        dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=32, capacity=16384, tag="k4200")
+    assert n > 0
+
+
 def test_llama_shape_bf16_short(lrqk, oracle):
     """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, r 32, k 2048, L 64, bf16) at an
     8K context, long enough (70 steps) for the 64-token ring to be flushed to the host store once."""

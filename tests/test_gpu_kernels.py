@@ -319,6 +319,7 @@ def test_score_select_diff_fused(ops, oracle, m, cap, k, H, dtype):
                                                        (262144, 2048, 2, torch.bfloat16, 16, True, False),
                                                        (131500, 2048, 2, torch.bfloat16, 32, False, False),
                                                        (30000, 4096, 2, torch.float32, 16, True, False),
+                                                       (90000, 8192, 1, torch.bfloat16, 32, True, False),
                                                        (9000, 1024, 2, torch.float32, 8, False, True)])
 def test_score_select_diff_unordered(ops, oracle, m, k, H, dtype, r, index, ties):
     """The decode step's form of the fused select + diff (no ascending list; lrqk_score_select_diff with
@@ -399,7 +400,7 @@ def test_diff_docstring_vector(ops, oracle):
     assert hit.view(-1).tolist() == [0, 4, 2, 6, 5] and ev.view(-1).tolist() == [0, 1, 0, 0, 1]
 
 
-@pytest.mark.parametrize("k,seq", [(8, 32), (512, 4096), (2048, 40000), (2500, 5000)])
+@pytest.mark.parametrize("k,seq", [(8, 32), (512, 4096), (2048, 40000), (2500, 5000), (8192, 60000)])
 def test_diff_random(ops, oracle, k, seq):
     _say("diff random", k, seq)
     g = torch.Generator().manual_seed(k)
@@ -435,7 +436,8 @@ def test_replace_all(ops):
 
 # ---------------------------------------------------------------- row movers
 
-@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float32, 128), (torch.float32, 8)])
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float32, 128), (torch.float32, 8),
+                                     (torch.bfloat16, 64), (torch.bfloat16, 256)])
 @pytest.mark.parametrize("pinned", [True, False])
 def test_fetch_rows(ops, oracle, dtype, d, pinned):
     _say("fetch", dtype, d, pinned)
@@ -553,7 +555,7 @@ def test_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol)
 
 
-@pytest.mark.parametrize("n", [1100, 2000, 2700, 3500, 4160, 6000])
+@pytest.mark.parametrize("n", [1100, 2000, 2700, 3500, 4160, 6000, 8256])
 def test_als_decode_split_counts(ops, ws, oracle, n):
     """The Gram sums arrive in ceil(n / 128) partials (at most 32) and the solve kernel is compiled per
     group of four of that count: one case per group not met by the shapes above."""
