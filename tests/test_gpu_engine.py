@@ -412,13 +412,16 @@ def test_qwen_shape_fp32_short(lrqk, oracle):
     assert n > 0
 
 
-@pytest.mark.parametrize("hq,hkv,d,r,k,L,l", [(8, 2, 64, 16, 128, 8, 700), (4, 1, 256, 32, 256, 16, 1200)])
-def test_other_head_widths(lrqk, oracle, hq, hkv, d, r, k, L, l):
-    """bf16 heads of 64 and 256 elements (rows of 128 and 512 bytes): the kernels written for rows of 128 elements
-    do not take these, so the whole trace runs on the general ones -- with the score index, whose ranks 16 and 32
-    do not depend on the head width."""
-    _say("head width", d)
-    _, _, n = _lockstep(lrqk, oracle, b=1, hq=hq, hkv=hkv, d=d, l=l, r=r, k=k, L=L, steps=30, dtype=torch.bfloat16,
+@pytest.mark.parametrize("hq,hkv,d,r,k,L,l,dtype", [(8, 2, 64, 16, 128, 8, 700, torch.bfloat16),
+                                                     (4, 1, 256, 32, 256, 16, 1200, torch.bfloat16),
+                                                     (4, 2, 256, 16, 64, 8, 500, torch.float32)])
+def test_other_head_widths(lrqk, oracle, hq, hkv, d, r, k, L, l, dtype):
+    """Heads of 64 and 256 elements: the kernels written for bf16 rows of 128 elements do not take these, so the
+    whole trace runs on the general ones -- with the score index, whose ranks 16 and 32 do not depend on the head
+    width.  An fp32 [K|V] row of 256 elements (2 KB) is wider than a wave: the step then ends with the separate
+    fetch and attention launches."""
+    _say("head width", d, dtype)
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=hq, hkv=hkv, d=d, l=l, r=r, k=k, L=L, steps=30, dtype=dtype,
                         max_iter=(2, 2), tol=(1e-8, 1e-8), rho=2 * r, capacity=2048, tag="d%d" % d)
     assert n > 0
 
@@ -429,6 +432,18 @@ def test_active_set_beyond_the_fused_diff(lrqk, oracle):
     _say("k = 4200 trace")
     _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=128, l=9000, r=16, k=4200, L=32, steps=12,
                         dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=32, capacity=16384, tag="k4200")
+    assert n > 0
+
+
+@pytest.mark.parametrize("hq,hkv,d,l,r,k,L,dtype", [(2, 1, 16, 30, 4, 8, 1, torch.float32),
+                                                     (3, 3, 128, 1111, 24, 333, 7, torch.bfloat16),
+                                                     (6, 2, 128, 2000, 8, 100, 5, torch.bfloat16)])
+def test_odd_sizes(lrqk, oracle, hq, hkv, d, l, r, k, L, dtype):
+    """A ring of one token (flushed at every step); sizes that are multiples of nothing (three heads, k + L = 340
+    slots, rank 24, which the score index does not cover); a short active set of 105 slots."""
+    _say("odd sizes", hq, hkv, d, l, r, k, L)
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=hq, hkv=hkv, d=d, l=l, r=r, k=k, L=L, steps=20, dtype=dtype,
+                        max_iter=(2, 2), tol=(1e-8, 1e-8), rho=2 * r, capacity=64, tag="odd%d" % L)
     assert n > 0
 
 
