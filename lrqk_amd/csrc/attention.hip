@@ -166,18 +166,22 @@ __device__ __forceinline__ void attn_block_merge(AttnAcc<VEC>& st, int lpr_log2,
   float M = -INFINITY;
 #pragma unroll
   for (int w = 0; w < NW; ++w) M = fmaxf(M, red[w][0]);
-  for (int c = threadIdx.x; c < d + 2; c += NW * kWave) {
-    float v = 0.0f;
-    if (c == 0) {
-      v = M;
-    } else {
+  float f[NW];
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        const float f = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
-        v += red[w][c] * f;
-      }
-    }
-    pout[c] = v;
+  for (int w = 0; w < NW; ++w) f[w] = (M == -INFINITY) ? 0.0f : exp2f(red[w][0] - M);
+  const int c = threadIdx.x;
+  if (c < d + 2) {
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += red[w][c] * f[w];
+    pout[c] = c == 0 ? M : v;
+  }
+  const int c2 = c + NW * kWave;
+  if (c2 < d + 2) {  // (rows of 256 elements only)
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += red[w][c2] * f[w];
+    pout[c2] = v;
   }
 }
 
@@ -409,10 +413,7 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
   }
   // merge the row groups: V lane (jl, cv) owns columns cv*VEC .. of group jl
   const int groups = rpb;  // <= 8 for rows of >= 512 bytes; larger counts are merged in rounds of 8
-  // thread t accumulates element t of the result (m, l, acc[d]); threads 0 and 1 also the two elements beyond
-  // the workgroup's thread count that rows of 256 elements have
-  const int tid2 = tid + kAttnThreads;
-  float M = -INFINITY, Lsum = 0.0f, col = 0.0f, col2 = 0.0f;
+  float M = -INFINITY, Lsum = 0.0f, col = 0.0f;  // thread t < d + 2 accumulates element t of the result
   for (int g0 = 0; g0 < groups; g0 += 8) {
     __syncthreads();
     if (!is_k && jl >= g0 && jl < g0 + 8 && jl < groups) {
@@ -431,17 +432,25 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
     const float a_old = (Mg == -INFINITY) ? 0.0f : exp2f(M - Mg);
     Lsum *= a_old;
     col *= a_old;
-    col2 *= a_old;
     for (int g = 0; g < ng; ++g) {
       const float fg = (Mg == -INFINITY || accs[g][0] == -INFINITY) ? 0.0f : exp2f(accs[g][0] - Mg);
       Lsum = fmaf(accs[g][1], fg, Lsum);
       if (tid >= 2 && tid < d + 2) col = fmaf(accs[g][tid], fg, col);
-      if (tid2 < d + 2) col2 = fmaf(accs[g][tid2], fg, col2);
     }
     M = Mg;
   }
   if (tid < d + 2) pout[tid] = tid == 0 ? M : (tid == 1 ? Lsum : col);
-  if (tid2 < d + 2) pout[tid2] = col2;
+  // Rows of 256 elements have two elements more than the workgroup has threads.  Such rows fill a wave, so the
+  // workgroup has four row groups and the loop above made one round: the groups' triples are still in place.
+  // (A second accumulator inside that loop cost the kernel 54 registers and half of its occupancy.)
+  if (d + 2 > kAttnThreads && tid < d + 2 - kAttnThreads) {
+    float c2 = 0.0f;
+    for (int g = 0; g < groups; ++g) {
+      const float fg = (M == -INFINITY || accs[g][0] == -INFINITY) ? 0.0f : exp2f(accs[g][0] - M);
+      c2 = fmaf(accs[g][tid + kAttnThreads], fg, c2);
+    }
+    pout[tid + kAttnThreads] = c2;
+  }
 }
 
 // Decode step: workgroups x < n_fetch copy this head's missed rows from the store into their
