@@ -1194,7 +1194,7 @@ __device__ __forceinline__ void step_find_digits(const uint32_t* hist_a, const u
 // outgoing tokens (i32 [k] each), freed slots (u16 [k]).
 static inline size_t step_select_words4(int64_t m) { return (size_t)(((m + 31) >> 5) + 3) & ~(size_t)3; }
 static inline size_t step_select_smem(int64_t m, int k) {
-  return step_select_words4(m) * (3 * 4 + 2) + (size_t)k * (4 + 4 + 2) + 16;
+  return step_select_words4(m) * (3 * 4 + 2) + (size_t)k * (4 + 4 + 4 + 2) + 16;
 }
 
 template <int CPT>
@@ -1209,7 +1209,8 @@ __device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* _
   uint16_t* wpre = reinterpret_cast<uint16_t*>(bmH + words4);  // [words4] marked tokens in the words before
   int32_t* miss_s = reinterpret_cast<int32_t*>(wpre + words4);  // [k] incoming tokens, ascending
   int32_t* ev_old = miss_s + k;                                 // [k] tokens of the freed slots
-  uint16_t* ev_slot = reinterpret_cast<uint16_t*>(ev_old + k);  // [k] freed slots, ascending
+  int32_t* hit_s = ev_old + k;                                  // [k] resident token of every slot (as the step found it)
+  uint16_t* ev_slot = reinterpret_cast<uint16_t*>(hit_s + k);   // [k] freed slots, ascending
   uint32_t* hist = L.hist;
   uint32_t* hist_b = L.hist_b;
   uint32_t* bmM = L.hist;             // incoming tokens (takes the place of the two histograms, 2 * kBins words)
@@ -1234,11 +1235,15 @@ __device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* _
     if (tid < 2) L.wred[tid] = 0;
   }
   __syncthreads();
-  // ---- resident bitmap; range of the keys
+  // ---- resident bitmap (the ids also go to LDS: they are needed again after the selection, and registers held
+  // that long were spilled); range of the keys
 #pragma unroll
   for (int u = 0; u < kIpt; ++u) {
     const int32_t v = hv[u];
-    if (u < ipt && tid * ipt + u < k && v >= 0 && v < m) atomicOr(&bmH[v >> 5], 1u << (v & 31));
+    if (u < ipt && tid * ipt + u < k) {
+      hit_s[tid * ipt + u] = v;
+      if (v >= 0 && v < m) atomicOr(&bmH[v >> 5], 1u << (v & 31));
+    }
   }
   uint32_t vmax = 0u, vor = 0u;
 #pragma unroll
@@ -1364,8 +1369,8 @@ __device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* _
   int n_ev = 0;
 #pragma unroll
   for (int u = 0; u < kIpt; ++u) {
-    const int32_t v = hv[u];
     const bool live = u < ipt && tid * ipt + u < k;
+    const int32_t v = hit_s[live ? tid * ipt + u : 0];
     const bool in_range = v >= 0 && v < m;
     const bool found = in_range && ((bmS[in_range ? (v >> 5) : 0] >> (v & 31)) & 1u);
     ev[u] = live && !found;
@@ -1391,7 +1396,7 @@ __device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* _
   for (int u = 0; u < kIpt; ++u) {
     if (ev[u]) {
       ev_slot[ex_ev] = (uint16_t)(tid * ipt + u);
-      ev_old[ex_ev] = hv[u];
+      ev_old[ex_ev] = hit_s[tid * ipt + u];
       ++ex_ev;
     }
   }
@@ -1469,7 +1474,9 @@ __global__ __launch_bounds__(kSelThreads) void select_step_kernel(const uint2* _
     const uint2* cand = cand_all + (int64_t)h * cand_cap;
     const uint32_t lo = st.t_used[h];
     const int k2 = bound_rank(k, level, n);
-    if (n <= 8 * kSelThreads)
+    if (n <= 4 * kSelThreads)
+      select_step_fast<4>(L, cand, n, lo, st, h, m, k, k2, df);
+    else if (n <= 8 * kSelThreads)
       select_step_fast<8>(L, cand, n, lo, st, h, m, k, k2, df);
     else
       select_step_fast<16>(L, cand, n, lo, st, h, m, k, k2, df);
