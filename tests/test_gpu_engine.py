@@ -447,6 +447,19 @@ def test_odd_sizes(lrqk, oracle, hq, hkv, d, l, r, k, L, dtype):
     assert n > 0
 
 
+def test_long_run_with_wrapping_caches(lrqk, oracle):
+    """300 steps of three sequences with one query head per kv head, a ring of 128 tokens (flushed twice), a
+    victim cache of 96 rows per head (its FIFO wraps many times), the score index extended row by row, and the
+    factor buffer and host store growing once on the way."""
+    _say("long run")
+    def configure(e):
+        e.victim_rows = 96
+    eng, orc, n = _lockstep(lrqk, oracle, b=3, hq=4, hkv=4, d=128, l=3000, r=32, k=256, L=128, steps=300,
+                            dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=64, capacity=3200,
+                            tag="long", configure=configure, compare_every=25, oracle_heads=(0, 3))
+    assert n > 0 and eng._A_K.capacity > 3200 and len(eng.KVcpu) == 3000 + 2 * 128
+
+
 def test_llama_shape_bf16_short(lrqk, oracle):
     """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, r 32, k 2048, L 64, bf16) at an
     8K context, long enough (70 steps) for the 64-token ring to be flushed to the host store once."""
