@@ -45,7 +45,9 @@ def parse():
     p.add_argument("--workload", default="llama8b_128k_bf16")
     p.add_argument("--context", type=int, default=None, help="override the context length")
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--cpu-steps", type=int, default=3, help="oracle steps timed for cpu_baseline (0 = skip)")
+    p.add_argument("--cpu-steps", type=int, default=160,
+                   help="decode mode: oracle steps timed for cpu_baseline (about 12 s of host work at the 128K "
+                        "configuration); the other modes only ask whether it is 0 (= no cpu_baseline)")
     p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
     p.add_argument("--event-every", type=int, default=0,
                    help="bracket every n-th proxy-score launch of the timed region with HIP events (each pair "
