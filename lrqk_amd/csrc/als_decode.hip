@@ -462,8 +462,11 @@ __device__ __forceinline__ float sum_lanes_0_31(float x) {
 // deltas: [bh][max_iter] sum over r of (k_hat - k_hat')^2.
 // KS: compile-time bound of the number of Gram splits S (S <= KS): that many 16-byte loads per thread
 // are in flight for the partial sums, so the bound follows S closely.
+// (Two workgroups per CU as the launch bound where the partial sums leave room: with at most 256 registers per
+// lane the matrix cores take their accumulators in ordinary registers, and a sweep reads its pivot row without
+// copying the whole tile out of the accumulation registers.)
 template <int KS>
-__global__ __launch_bounds__(kSolveThreads) void als_solve_kernel(const float* __restrict__ pre,
+__global__ __launch_bounds__(kSolveThreads, KS <= 16 ? 2 : 1) void als_solve_kernel(const float* __restrict__ pre,
                                                                   const float* __restrict__ part, int S, int r,
                                                                   int max_iter, float* __restrict__ iter_out,
                                                                   float* __restrict__ deltas) {

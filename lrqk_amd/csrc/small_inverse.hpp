@@ -50,6 +50,10 @@ __device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, 
   }
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] *= sc[v];
+  // The lane-dependent cases are taken by weights of 0 and 1, not by selects: selects between expressions
+  // compile to divergent branches, which cost more than the sweep's arithmetic.  (The matrix is finite, so a
+  // product with a weight of 0 is 0.)
+  const float in0 = half == 0 ? 1.0f : 0.0f, in1 = 1.0f - in0;
 #pragma unroll
   for (int p = 0; p < 32; ++p) {
     if (p < r) {  // (wave-uniform)
@@ -58,9 +62,13 @@ __device__ __forceinline__ void invert_sweep_mfma(GetG&& g, int r, float* sbuf, 
       const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rv), p + 32 * hp));
       float rc = __builtin_amdgcn_rcpf(d);
       rc = fmaf(fmaf(-d, rc, 1.0f), rc, rc);
-      const bool inhalf = half == hp, isp = col == p;
-      const float A = inhalf ? (isp ? 1.0f - rc : rv * rc) : (isp ? 2.0f : 0.0f);
-      const float B = inhalf ? (isp ? d - 1.0f : rv) : (isp ? 1.0f : 0.0f);
+      const float win = hp ? in1 : in0, wout = hp ? in0 : in1;  // this lane's half holds row p / the other half
+      const float wp = col == p ? 1.0f : 0.0f;
+      // A = in: (p: 1 - rc, else rv rc); out: (p: 2, else 0).   B = in: (p: d - 1, else rv); out: (p: 1, else 0)
+      const float a_in = fmaf(wp, (1.0f - rc) - rv * rc, rv * rc);
+      const float b_in = fmaf(wp, (d - 1.0f) - rv, rv);
+      const float A = fmaf(win, a_in, wout * (2.0f * wp));
+      const float B = fmaf(win, b_in, wout * wp);
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(-A, B, acc, 0, 0, 0);
     }
   }
