@@ -13,16 +13,27 @@ constexpr int kFinThreads = 256;
 // mean over all heads of |k_hat - k_hat'|^2 is below tol.  deltas: [bh][max_iter] per-head sums.
 // Executed by one whole wave; every lane returns the index of the iterate to keep.  The sums are
 // formed in one fixed order, so every caller reaches the same decision.
-// MAXIT >= max_iter bounds the register arrays; all loads are independent (one memory latency).
+// MAXIT >= max_iter bounds the register arrays.  Every load is unconditional (index clamped, value masked): a
+// conditional load compiles to a branch with a full wait, which would put one memory latency per iteration on the
+// chain of whoever calls this; as it is they all go out together.
 template <int MAXIT>
 __device__ __forceinline__ void als_delta_sums(const float* __restrict__ deltas, int bh, int max_iter,
                                                float (&sacc)[MAXIT]) {
+  // the first 64 heads in straight-line code (the caller's other requests can go out before these are waited for)
+  {
+    const int hh = min(lane_id(), bh - 1);
+    float v[MAXIT];
 #pragma unroll
-  for (int it = 0; it < MAXIT; ++it) sacc[it] = 0.0f;
-  for (int hh = lane_id(); hh < bh; hh += kWave) {
+    for (int it = 0; it < MAXIT; ++it) v[it] = deltas[(int64_t)hh * max_iter + min(it, max_iter - 1)];
 #pragma unroll
-    for (int it = 0; it < MAXIT; ++it)
-      if (it < max_iter) sacc[it] += deltas[(int64_t)hh * max_iter + it];
+    for (int it = 0; it < MAXIT; ++it) sacc[it] = (lane_id() < bh && it < max_iter) ? v[it] : 0.0f;
+  }
+  for (int hh = lane_id() + kWave; hh < bh; hh += kWave) {
+    float v[MAXIT];
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) v[it] = deltas[(int64_t)hh * max_iter + min(it, max_iter - 1)];
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) sacc[it] += it < max_iter ? v[it] : 0.0f;
   }
 }
 template <int MAXIT>

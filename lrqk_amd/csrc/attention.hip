@@ -113,6 +113,10 @@ __device__ __forceinline__ void attn_scan_w(const float* __restrict__ w, float s
       wl[u] = w[rr];
       vv[u].load(Vh + (int64_t)rr * d + sub * VEC);
     }
+    // (the products are only used for rows that count; without this the compiler moves each of their loads into
+    // that condition, where it becomes a branch with a full wait per row group)
+#pragma unroll
+    for (int u = 0; u < U; ++u) asm volatile("" : "+v"(wl[u]));
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float vf[VEC];
