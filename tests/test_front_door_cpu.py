@@ -110,3 +110,44 @@ def test_state_table():
         cache[0]
     with pytest.raises(NotImplementedError):
         iter(cache)
+
+
+class _WideRecorder(_Recorder):
+    """An engine stand-in that returns an 'active set' of the width it was given."""
+
+    def decode(self, q, k, v):
+        self.decoded += 1
+        self.length += 1
+        self.last = (q.clone(), k.clone(), v.clone())
+        return torch.cat([k, k], 2).repeat_interleave(2, 1), torch.cat([v, v], 2).repeat_interleave(2, 1)
+
+
+def test_other_head_widths_are_padded_for_the_engine():
+    """Rows of 96 fp32 elements reach the engine as rows of 128 with zero columns; the caller gets its own
+    tensors back from the prompt call and rows of 96 from a decode call.  Widths the kernels take as they are
+    (powers of two of at least 16 bytes) pass through untouched."""
+    assert [DynamicLRQKCache._padded_width(d, 2) for d in (96, 80, 128, 64, 8, 4, 192, 256)] == \
+        [128, 128, 128, 64, 8, 8, 256, 256]
+    assert [DynamicLRQKCache._padded_width(d, 4) for d in (96, 4, 3, 2)] == [128, 4, 4, 4]
+    _Recorder.made.clear()
+    cache = DynamicLRQKCache(r=4, num_active_tokens=8, lite_tokens=2, num_key_value_groups=2, lwattn_factory=_WideRecorder)
+    q, k, v = _pieces(9, d=96)
+    K, V = cache.update(q, k, v, 0)
+    eng = cache.lwattn[0]
+    assert K is k and V is v
+    for given, seen in zip((q, k, v), eng.prefilled):
+        assert seen.shape[-1] == 128 and torch.equal(seen[..., :96], given) and seen[..., 96:].abs().sum() == 0
+    q1, k1, v1 = _pieces(1, d=96)
+    K, V = cache.update(q1, k1, v1, 0)
+    assert eng.last[0].shape[-1] == 128 and torch.equal(eng.last[1][..., :96], k1)
+    assert K.shape == (2, 4, 2, 96) and torch.equal(K[:, ::2, :1], k1) and torch.equal(V[:, ::2, :1], v1)
+    eng.attn_in_step = True
+    with pytest.raises(NotImplementedError):
+        cache.update(q1, k1, v1, 0)
+    # a width the kernels take: the engine gets the caller's own tensors
+    q, k, v = _pieces(9, d=64)
+    cache.update(q, k, v, 1)
+    assert cache.lwattn[1].prefilled[1].shape[-1] == 64
+    q1, k1, v1 = _pieces(1, d=64)
+    K, V = cache.update(q1, k1, v1, 1)
+    assert K.shape[-1] == 64 and cache.lwattn[1].last[1].data_ptr() != k1.data_ptr()  # (the stand-in clones)

@@ -696,6 +696,60 @@ def test_cache_front_door(lrqk, oracle):
         cache.update(q, kk, vv, 2)
 
 
+@pytest.mark.parametrize("d,dtype", [(96, torch.bfloat16), (80, torch.float32)])
+def test_front_door_pads_other_head_widths(lrqk, oracle, d, dtype):
+    """Heads of 96 and 80 elements through DynamicLRQKCache: the engine works on rows padded with zero columns, the
+    caller sees its own width.  Lock-step with the oracle at the true width (continued from the GPU's factors, as in
+    the other traces): selected tokens and returned K, V bit-exact, factor outputs within the bf16 / fp32 limits, and
+    the padded columns of B_Q, B_K exactly zero all along."""
+    _say("front door, head width", d)
+    from lrqk_amd import synth
+    b, hq, hkv, l, r, k, L, steps = 1, 4, 2, 700, 16, 128, 8, 24
+    g = hq // hkv
+    gen = torch.Generator().manual_seed(d)
+    Q, WQ = synth.low_rank_noise(gen, b, hq, l, d, 32, 0.01, dtype)
+    K, WK = synth.low_rank_noise(gen, b, hkv, l, d, 32, 0.01, dtype)
+    V, WV = synth.low_rank_noise(gen, b, hkv, l, d, 32, 0.01, dtype)
+    A_Q0 = torch.randn((b, hq, l, r), generator=gen)
+    A_K0 = torch.randn((b, hq, l, r), generator=gen)
+    cache = lrqk.DynamicLRQKCache(r=r, num_active_tokens=k, lite_tokens=L, max_iter=(2, 2), tol=1e-8,
+                                  max_sequence_length=1024, num_key_value_groups=g)
+    eng = cache.lwattn[0]
+    eng.init_factors = (A_Q0, A_K0)
+    Kd, Vd = K.to(DEV), V.to(DEV)
+    K0, V0 = cache.update(Q.to(DEV), Kd, Vd, 0)
+    assert K0 is Kd and V0 is Vd and cache.sequence_state[0] == cache.State.decoding
+    w = eng.B_Q.shape[-1]
+    assert w == 128 and eng.Kgpu.shape[-1] == w
+    orc = oracle.OracleLayer(num_lite_tokens=L, attn_topk=k, num_key_value_groups=g, r=r, max_iter=(2, 2),
+                             tol=(1e-8, 1e-8), capacity=1024, compute_dtype=torch.float64)
+    A_Q_full = torch.zeros((b, hq, l, r), dtype=dtype)
+    A_Q_full[:, :, -1:] = eng.last_A_Q_row.cpu()
+    orc.prefill(Q, K, V, als_result=(A_Q_full, eng.B_Q[..., :d].cpu(), eng.A_K.cpu(), eng.B_K[..., :d].cpu()))
+    assert torch.equal(eng.hit_indices.cpu(), orc.hit_indices)
+    # the prefill's factors against the fp64 oracle, through their products (as in the other traces)
+    ref = oracle.cast_lrqk_prefill(Q, oracle.repeat_kv(K, g), r, 2, 1e-8, A_Q0=A_Q0, A_K0=A_K0, compute_dtype=torch.float64)
+    _note("pad%d" % d, "prefill A_K B_K", _rel(eng.A_K.cpu().double() @ eng.B_K[..., :d].cpu().double(),
+                                                ref[2].double() @ ref[3].double()), 1e-2)
+    stream = synth.DecodeStream(synth.Workload("t", hq, hkv, d, b, dtype, l, r, k, L, (2, 2), (1e-8, 1e-8), steps, 32, 0.01),
+                                Q[:, :, -1:], (WQ, WK, WV), gen)
+    lim = 1e-3
+    for step in range(steps):
+        q, kk, vv = [t.cpu() for t in stream.next()]
+        Kg, Vg = cache.update(q.to(DEV), kk.to(DEV), vv.to(DEV), 0)
+        oB_Q, oB_K, ohq, ohk = orc.begin_decode(q, kk, vv)
+        for name, got, exp in (("q_hat", eng.last_q_hat, ohq), ("k_hat", eng.last_k_hat, ohk),
+                               ("B_Q", eng.B_Q[..., :d], oB_Q), ("B_K", eng.B_K[..., :d], oB_K)):
+            _note("pad%d" % d, name, _rel(got, exp), lim)
+        assert eng.B_Q[..., d:].abs().sum() == 0 and eng.B_K[..., d:].abs().sum() == 0, step
+        oK, oV = orc.finish_decode(eng.B_Q[..., :d].cpu(), eng.B_K[..., :d].cpu(), eng.last_q_hat.cpu(), eng.last_k_hat.cpu())
+        assert Kg.shape == oK.shape and torch.equal(Kg.cpu(), oK) and torch.equal(Vg.cpu(), oV), step
+        assert torch.equal(eng.hit_indices.cpu(), orc.hit_indices), step
+    eng.attn_in_step = True
+    with pytest.raises(NotImplementedError):
+        cache.update(q.to(DEV), kk.to(DEV), vv.to(DEV), 0)
+
+
 def test_cast_functions(lrqk, oracle):
     _say("cast functions")
     g = torch.Generator().manual_seed(2)
