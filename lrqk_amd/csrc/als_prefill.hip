@@ -23,7 +23,7 @@ namespace lrqk {
 
 constexpr int kPfThreads = 256;
 constexpr int kPfTile = 32;
-constexpr int kPfMaxPer = 32;  // accumulators per thread: r*(r+d) <= 256*32
+constexpr int kPfMaxPer = 48;  // accumulators per thread: r*(r+d) <= 256*48 (r = 64 with rows of 128 elements)
 
 // acc[e] += sum_rows a_s[row][j] * (c < r ? a_s[row][c] : x_s[row][c-r]),  e = j*(r+d)+c
 __device__ __forceinline__ void accumulate_gram(const float* a_s, int lda, const float* x_s, int ldx, int rows, int r,
@@ -153,8 +153,7 @@ __global__ __launch_bounds__(kPfThreads) void pf_small_generic_kernel(int stage,
   extern __shared__ __align__(16) float sm[];
   const int ldm = r + d + 1;
   const int ne = r * (r + d);
-  float* G1 = sm;               // [r][r+d] packed (ne)   Gram of the first operand
-  float* G2 = G1 + ne;          // [r][r+d] packed (ne)
+  float* G2 = sm;               // [r][r+d] packed (ne)   the K side's sums (the Q side's go straight into Mx)
   float* Mx = G2 + ne;          // [r][ldm]
   float* Bs = Mx + r * ldm;     // [r][d+1]
   __shared__ int s_done;
@@ -191,12 +190,16 @@ __global__ __launch_bounds__(kPfThreads) void pf_small_generic_kernel(int stage,
 
   const float* pq = partQ + (int64_t)h * S * ne;
   const float* pk = partK + (int64_t)h * S * ne;
+  // sum over the splits of element e of a head's packed [G | C] block, in split order
+  auto summed = [&](const float* part, int e) {
+    float v = 0.0f;
+    for (int s = 0; s < S; ++s) v += part[(int64_t)s * ne + e];
+    return v;
+  };
   if (stage == 0 || stage == 2) {
-    reduce_part(pq, S, ne, G1);
     reduce_part(pk, S, ne, G2);
-    __syncthreads();
     // B_Q = (A_Q^T A_Q)^-1 A_Q^T Q
-    for (int e = tid; e < ne; e += kPfThreads) Mx[(e / (r + d)) * ldm + e % (r + d)] = G1[e];
+    for (int e = tid; e < ne; e += kPfThreads) Mx[(e / (r + d)) * ldm + e % (r + d)] = summed(pq, e);
     __syncthreads();
     solve_multi(Mx, ldm, r, d);
     for (int e = tid; e < r * d; e += kPfThreads) {
@@ -231,12 +234,11 @@ __global__ __launch_bounds__(kPfThreads) void pf_small_generic_kernel(int stage,
     }
   } else {
     // stage 1: Mt_K = (A_Q^T A_Q + B_K B_K^T)^-1 (A_Q^T Q + B_K)
-    reduce_part(pq, S, ne, G1);
     for (int e = tid; e < r * d; e += kPfThreads) Bs[(e / d) * (d + 1) + e % d] = b_k[(int64_t)h * r * d + e];
     __syncthreads();
     for (int e = tid; e < ne; e += kPfThreads) {
       const int i = e / (r + d), c = e % (r + d);
-      float v = G1[e];
+      float v = summed(pq, e);
       if (c < r) {
         float g = 0.0f;
         for (int x = 0; x < d; ++x) g = fmaf(Bs[i * (d + 1) + x], Bs[c * (d + 1) + x], g);
@@ -1052,7 +1054,7 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   }
   auto small = small32 ? pf_small32_kernel : pf_small_generic_kernel;
   const size_t smem_small = small32 ? ((size_t)3 * ne + 4 + (size_t)r * (d + 4)) * sizeof(float)
-                                    : ((size_t)2 * ne + (size_t)r * (r + d + 1) + (size_t)r * (d + 1)) * sizeof(float);
+                                    : ((size_t)ne + (size_t)r * (r + d + 1) + (size_t)r * (d + 1)) * sizeof(float);
   LRQK_REQUIRE(smem_small <= 160 * 1024 && smem_pass <= 160 * 1024, LRQK_ELIMIT, "r=%d d=%d need too much LDS", r, d);
   if (smem_pass > 48 * 1024)
     LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)pass, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));

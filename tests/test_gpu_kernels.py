@@ -675,7 +675,10 @@ def test_als_prefill_long_sums(ops, ws, oracle):
                           # head groupings: one query head per kv head and eight (the last pass then goes head by head)
                           (torch.bfloat16, 2, 2, 900, 128, 32, 2, 0.0), (torch.bfloat16, 8, 1, 1100, 128, 16, 2, 0.0),
                           # a rank that is no multiple of the four pivots of an elimination step
-                          (torch.bfloat16, 4, 1, 600, 128, 6, 2, 0.0)])
+                          (torch.bfloat16, 4, 1, 600, 128, 6, 2, 0.0),
+                          # ranks beyond 32 (the general kernels): 64 with rows of 128 elements, 48, 40
+                          (torch.bfloat16, 4, 2, 1500, 128, 64, 2, 0.0), (torch.float32, 2, 1, 700, 64, 48, 2, 0.0),
+                          (torch.bfloat16, 2, 1, 900, 128, 40, 3, 0.0)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
