@@ -588,6 +588,260 @@ __global__ __launch_bounds__(kSolveThreads, KS <= 16 ? 2 : 1) void als_solve_ker
   }
 }
 
+// ----------------------------------------------------------------------------- ranks beyond one matrix-core tile
+// 32 < r <= 64 (the reference's "accuracy-focused" setting is r = 64, README.md:126): the same two launches in plain
+// fp32 arithmetic, not tuned -- sums over the active rows, then one workgroup per head that forms G_K, G_Q, inverts
+// them (Gauss-Jordan on the matrix scaled to unit diagonal, no pivoting: symmetric positive definite) and runs the
+// alternating rank-1 solves with the formulas of als_solve_kernel.  Same outputs (iter_out, deltas), so the finish
+// stage and the scan take over from there unchanged.
+constexpr int kWideThreads = 256;
+constexpr int kWideTile = 32;   // active rows per step
+constexpr int kWideMaxR = 64;
+
+// part per (head, split): r * r sums A^T A, then r sums A^T w.
+template <typename T>
+__global__ __launch_bounds__(kWideThreads) void als_gram_wide_kernel(
+    const T* __restrict__ a_k, int64_t head_stride, int64_t a_rows, const int32_t* __restrict__ active_idx,
+    int64_t idx_stride, T* k_prev, int kprev_slots, int n, const T* __restrict__ q, int r, int d,
+    float* __restrict__ part, int S, GramAppend ap) {
+  extern __shared__ __align__(16) float wsm[];
+  float* a_s = wsm;                            // [kWideTile][r + 1]
+  float* w_s = a_s + kWideTile * (r + 1);      // [kWideTile]
+  float* q_s = w_s + kWideTile;                // [d]
+  const int tid = threadIdx.x;
+  const int h = blockIdx.y, s = blockIdx.x;
+  const int lda = r + 1;
+  const T* A = a_k + (int64_t)h * head_stride;
+  const T* Kp = k_prev + (int64_t)h * kprev_slots * d;
+  const T* knew_h = Kp;
+  if (ap.slot >= 0) {
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    knew_h = (const T*)ap.k_new + ((int64_t)bb * ap.hkv + kvh) * d;
+  }
+  for (int c = tid; c < d; c += kWideThreads) q_s[c] = ld_f32<T>(q, (int64_t)h * d + c);
+  const int rows_per_split = (n + S - 1) / S;
+  const int s0 = s * rows_per_split, s1 = min(n, s0 + rows_per_split);
+  constexpr int kPer = kWideMaxR * kWideMaxR / kWideThreads;  // 16 sums of A^T A per thread
+  float acc[kPer], racc = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) acc[i] = 0.0f;
+  __syncthreads();
+  for (int t0 = s0; t0 < s1; t0 += kWideTile) {
+    const int rows = min(kWideTile, s1 - t0);
+    // the rows of A_K of the tile's tokens (zero where the slot holds no token or its row does not exist yet)
+    for (int e = tid; e < rows * r; e += kWideThreads) {
+      const int row = e / r, j = e % r;
+      const int t = t0 + row;
+      int32_t tok = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      if (t == ap.slot) tok = ap.token;
+      const bool ok = tok >= 0 && (int64_t)tok < a_rows;
+      a_s[row * lda + j] = ok ? ld_f32<T>(A, (int64_t)tok * r + j) : 0.0f;
+    }
+    // w = K q of the tile's rows: eight lanes per row
+    {
+      const int row = tid >> 3, sub = tid & 7;
+      float wv = 0.0f;
+      if (row < rows) {
+        const int t = t0 + row;
+        const T* kr = t == ap.slot ? knew_h : Kp + (int64_t)t * d;
+        for (int c = sub; c < d; c += 8) wv = fmaf(ld_f32<T>(kr, c), q_s[c], wv);
+      }
+      wv = group_sum(wv, 8);
+      if (sub == 0 && row < kWideTile) w_s[row] = row < rows ? wv : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int e = tid + i * kWideThreads;
+      if (e < r * r) {
+        const int a = e / r, b2 = e % r;
+        float v = acc[i];
+        for (int row = 0; row < rows; ++row) v = fmaf(a_s[row * lda + a], a_s[row * lda + b2], v);
+        acc[i] = v;
+      }
+    }
+    if (tid < r)
+      for (int row = 0; row < rows; ++row) racc = fmaf(w_s[row], a_s[row * lda + tid], racc);
+    __syncthreads();
+  }
+  if (ap.slot >= s0 && ap.slot < s1) {  // this workgroup owns the new token's slot: the ring append
+    const int bb = h / ap.hq, kvh = (h % ap.hq) / (ap.hq / ap.hkv);
+    const T* ks = (const T*)ap.k_new + ((int64_t)bb * ap.hkv + kvh) * d;
+    const T* vs = (const T*)ap.v_new + ((int64_t)bb * ap.hkv + kvh) * d;
+    T* kd = k_prev + ((int64_t)h * kprev_slots + ap.slot) * d;
+    T* vd = (T*)ap.v_act + ((int64_t)h * kprev_slots + ap.slot) * d;
+    for (int c = tid; c < d; c += kWideThreads) {
+      kd[c] = ks[c];
+      vd[c] = vs[c];
+    }
+    if (tid == 0) ap.idx_out[(int64_t)h * idx_stride + ap.slot] = ap.token;
+  }
+  float* pout = part + ((int64_t)h * S + s) * (r * r + r);
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int e = tid + i * kWideThreads;
+    if (e < r * r) pout[e] = acc[i];
+  }
+  if (tid < r) pout[r * r + tid] = racc;
+}
+
+// In-place inverse of the symmetric positive definite r x r matrix G (row stride ld) by the whole workgroup:
+// scaled to unit diagonal, Gauss-Jordan without pivoting, scaled back.  colp, rowp, sc: r floats each.
+__device__ __forceinline__ void wide_invert(float* G, int ld, int r, float* colp, float* rowp, float* sc) {
+  const int tid = threadIdx.x;
+  if (tid < r) sc[tid] = rsqrtf(G[tid * ld + tid]);
+  __syncthreads();
+  for (int e = tid; e < r * r; e += kWideThreads) G[(e / r) * ld + e % r] *= sc[e / r] * sc[e % r];
+  __syncthreads();
+  for (int p = 0; p < r; ++p) {
+    if (tid < r) {
+      colp[tid] = G[tid * ld + p];
+      rowp[tid] = G[p * ld + tid];
+    }
+    __syncthreads();
+    const float piv = 1.0f / colp[p];
+    for (int e = tid; e < r * r; e += kWideThreads) {
+      const int i = e / r, j = e % r;
+      float v;
+      if (i == p)
+        v = j == p ? piv : rowp[j] * piv;
+      else if (j == p)
+        v = -colp[i] * piv;
+      else
+        v = fmaf(-colp[i] * piv, rowp[j], G[i * ld + j]);
+      G[i * ld + j] = v;
+    }
+    __syncthreads();
+  }
+  for (int e = tid; e < r * r; e += kWideThreads) G[(e / r) * ld + e % r] *= sc[e / r] * sc[e % r];
+  __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
+    const float* __restrict__ part, int S, const T* __restrict__ b_q, const T* __restrict__ b_k,
+    const T* __restrict__ q, const T* __restrict__ k_new, int hq, int hkv, int r, int d, int max_iter,
+    float* __restrict__ iter_out, float* __restrict__ deltas) {
+  extern __shared__ __align__(16) float wsm[];
+  const int ldb = d + 1, ldg = r + 1;
+  float* Bq = wsm;                 // [r][d + 1]
+  float* Bk = Bq + r * ldb;        // [r][d + 1]
+  float* GQ = Bk + r * ldb;        // [r][r + 1]
+  float* GK = GQ + r * ldg;        // [r][r + 1]
+  float* qv = GK + r * ldg;        // [d]
+  float* kv = qv + d;              // [d]
+  float* vec = kv + d;             // 10 vectors of kWideMaxR
+  float* rhs_q = vec, *kB = vec + 64, *hk0 = vec + 128, *yq0 = vec + 192, *hk = vec + 256, *hqv = vec + 320;
+  float* z = vec + 384, *y = vec + 448, *colp = vec + 512, *rowp = vec + 576;
+  float* sc = vec + 640;           // [kWideMaxR]
+  __shared__ float s_red[4];
+  const int tid = threadIdx.x;
+  const int h = blockIdx.x;
+  const int b = h / hq, kvh = (h % hq) / (hq / hkv);
+  const int ne = r * r + r;
+  for (int e = tid; e < r * d; e += kWideThreads) {
+    Bq[(e / d) * ldb + e % d] = ld_f32<T>(b_q, (int64_t)h * r * d + e);
+    Bk[(e / d) * ldb + e % d] = ld_f32<T>(b_k, (int64_t)h * r * d + e);
+  }
+  for (int c = tid; c < d; c += kWideThreads) {
+    qv[c] = ld_f32<T>(q, (int64_t)h * d + c);
+    kv[c] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
+  }
+  __syncthreads();
+  // G_K = B_K B_K^T, G_Q = B_Q B_Q^T + A^T A (partial sums added in split order)
+  const float* pin = part + (int64_t)h * S * ne;
+  for (int e = tid; e < r * r; e += kWideThreads) {
+    const int i = e / r, j = e % r;
+    float gq = 0.0f, gk = 0.0f;
+    for (int c = 0; c < d; ++c) {
+      gq = fmaf(Bq[i * ldb + c], Bq[j * ldb + c], gq);
+      gk = fmaf(Bk[i * ldb + c], Bk[j * ldb + c], gk);
+    }
+    float ga = 0.0f;
+    for (int s = 0; s < S; ++s) ga += pin[(int64_t)s * ne + e];
+    GQ[i * ldg + j] = gq + ga;
+    GK[i * ldg + j] = gk;
+  }
+  if (tid < r) {
+    float rq = 0.0f, kb = 0.0f, aw = 0.0f;
+    for (int c = 0; c < d; ++c) {
+      rq = fmaf(qv[c], Bq[tid * ldb + c], rq);
+      kb = fmaf(kv[c], Bk[tid * ldb + c], kb);
+    }
+    for (int s = 0; s < S; ++s) aw += pin[(int64_t)s * ne + r * r + tid];
+    rhs_q[tid] = rq + aw;   // q B_Q^T + (q K^T) A
+    kB[tid] = kb;           // k B_K^T
+  }
+  if (tid < kWave) {
+    float v = 0.0f;
+    for (int c = tid; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
+    v = wave_sum(v);
+    if (tid == 0) s_red[0] = v;  // q . k
+  }
+  __syncthreads();
+  wide_invert(GK, ldg, r, colp, rowp, sc);
+  wide_invert(GQ, ldg, r, colp, rowp, sc);
+  const float sqk = s_red[0];
+  // out[c] = sum_i in[i] G[i][c]
+  auto vecmat = [&](const float* in, const float* G, float* out) {
+    if (tid < r) {
+      float v = 0.0f;
+      for (int i = 0; i < r; ++i) v = fmaf(in[i], G[i * ldg + tid], v);
+      out[tid] = v;
+    }
+    __syncthreads();
+  };
+  // (a . b) over r elements, in every thread; s_red[1 + slot] is the scratch cell
+  auto dot = [&](const float* a, const float* bb, int slot) {
+    if (tid < kWave) {
+      float v = tid < r ? a[tid] * bb[tid] : 0.0f;
+      v = wave_sum(v);
+      if (tid == 0) s_red[1 + slot] = v;
+    }
+    __syncthreads();
+    const float v = s_red[1 + slot];
+    return v;
+  };
+  // x = b (G + v^T v)^-1 with b = b0 + s v, from G^-1 (Sherman-Morrison): z = v G^-1, y = y0 + s z,
+  // x = y - (y . v / (1 + z . v)) z
+  auto rank1 = [&](const float* y0, const float* v, const float* G, float* out) {
+    vecmat(v, G, z);
+    if (tid < r) y[tid] = fmaf(sqk, z[tid], y0[tid]);
+    __syncthreads();
+    const float yv = dot(y, v, 0);
+    const float zv = dot(z, v, 1);
+    const float alpha = yv / (1.0f + zv);
+    __syncthreads();  // (both cells read before the next call writes them)
+    if (tid < r) out[tid] = fmaf(-alpha, z[tid], y[tid]);
+    __syncthreads();
+  };
+  vecmat(kB, GK, hk0);      // k_hat_0 = kB G_K^-1
+  vecmat(rhs_q, GQ, yq0);   // rhs_q G_Q^-1
+  if (tid < r) hk[tid] = hk0[tid];
+  __syncthreads();
+  for (int it = 0; it < max_iter; ++it) {
+    rank1(yq0, hk, GQ, hqv);   // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
+    rank1(hk0, hqv, GK, y);    // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat   (y is free again: out may alias it)
+    float df = 0.0f;
+    if (tid < r) {
+      df = hk[tid] - y[tid];
+      df *= df;
+    }
+    if (tid < kWave) {
+      const float t = wave_sum(df);
+      if (tid == 0) deltas[(int64_t)h * max_iter + it] = t;
+    }
+    float* o = iter_out + ((int64_t)h * max_iter + it) * 2 * r;
+    if (tid < r) {
+      o[tid] = hqv[tid];
+      o[r + tid] = y[tid];
+    }
+    __syncthreads();
+    if (tid < r) hk[tid] = y[tid];
+    __syncthreads();
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kFinThreads) void als_finish_kernel(FinishArgs fa) {
   // workgroups [bh, 2 bh), if launched, encode the appended rows for the score index
@@ -598,6 +852,37 @@ __global__ __launch_bounds__(kFinThreads) void als_finish_kernel(FinishArgs fa) 
 }
 static inline unsigned finish_grid(const FinishArgs& fa) {
   return (unsigned)fa.bh * (fa.qa != nullptr && fa.append_row >= 0 ? 2u : 1u);
+}
+
+// The finish stage of a factor update whose iterates are in iter_out / deltas: launched, or handed to the step's
+// later launches.
+template <typename T>
+static int als_decode_finish(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, const void* q,
+                             const void* k_new, int bh, int hq, int hkv, int r, int d, int lpr_log2, int max_iter,
+                             float tol, void* q_hat, void* k_hat, int64_t append_row, float* iter_out, float* deltas,
+                             bool defer_finish, hipStream_t st) {
+  FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
+                head_stride, append_row, nullptr, nullptr, nullptr, 0};
+  if (ctx->sidx_enabled && ctx->sidx_a_k == a_k && ctx->sidx_bh == bh && ctx->sidx_r == r && append_row >= 0 &&
+      ctx->sidx_head_rows == head_stride / r && ctx->sidx_dtype == (sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16)) {
+    // the appended row also goes into the score index; rows stay contiguous as long as rows are appended in order
+    fa.qa = (uint8_t*)ctx->sidx_qa.p;
+    fa.qs = (uint16_t*)ctx->sidx_qs.p;
+    fa.qw = (const float*)ctx->sidx_wm.p;
+    fa.q_head_rows = ctx->sidx_head_rows;
+    if (append_row == ctx->sidx_valid) ctx->sidx_valid = append_row + 1;  // (a gap is indexed on demand later)
+  }
+  if (defer_finish) {
+    // the caller lets later launches of the step absorb the finish stage (flush_pending_finish otherwise)
+    ctx->fin = fa;
+    ctx->fin_dtype = sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16;
+    ctx->fin_pending = true;   // B update, outputs and the A_K row still to be done
+    ctx->qhat_pending = true;  // q_hat has not been written yet: consumers take the iterate from iter_out
+    return LRQK_OK;
+  }
+  hipLaunchKernelGGL((als_finish_kernel<T>), dim3(finish_grid(fa)), dim3(kFinThreads), 0, st, fa);
+  LRQK_HIP_CHECK(hipGetLastError());
+  return LRQK_OK;
 }
 
 template <typename T>
@@ -616,6 +901,37 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
                "head_dim %d unsupported (need a power of two in 8..256 with at least one 16-byte chunk)", d);
   LRQK_REQUIRE(((uintptr_t)b_q % 16 == 0) && ((uintptr_t)b_k % 16 == 0) && ((int64_t)r * d * sizeof(T)) % 16 == 0,
                LRQK_EINVAL, "b_q/b_k must be 16-byte aligned");
+  if (r > kAlsMaxR) {
+    // ranks beyond one matrix-core tile: the general kernels
+    const int S = std::min(32, std::max(1, (n + 255) / 256));
+    const int ne = r * r + r;
+    int rc = ctx->als_part.ensure((size_t)bh * S * ne * sizeof(float));
+    if (rc) return rc;
+    if ((rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float)))) return rc;
+    float* part = (float*)ctx->als_part.p;
+    float* iter_out = (float*)ctx->als_iter.p;
+    float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
+    const size_t smem_g = ((size_t)kWideTile * (r + 1) + kWideTile + d) * sizeof(float);
+    const size_t smem_s = ((size_t)2 * r * (d + 1) + (size_t)2 * r * (r + 1) + 2 * d + 11 * kWideMaxR) * sizeof(float);
+    LRQK_REQUIRE(smem_s <= (size_t)160 * 1024 - 256, LRQK_ELIMIT, "r=%d with rows of %d elements needs too much LDS", r, d);
+    static std::atomic<size_t> wide_allowed_dev[kMaxDeviceSlots];
+    std::atomic<size_t>& wide_allowed = wide_allowed_dev[per_device_slot()];
+    if (smem_s > std::max<size_t>(wide_allowed, 48 * 1024)) {
+      LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)als_solve_wide_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)smem_s));
+      wide_allowed = smem_s;
+    }
+    hipLaunchKernelGGL((als_gram_wide_kernel<T>), dim3((unsigned)S, (unsigned)bh), dim3(kWideThreads), smem_g, st,
+                       (const T*)a_k, head_stride, head_stride / r, active_idx, idx_stride, (T*)k_prev, kprev_slots, n,
+                       (const T*)q, r, d, part, S, ap);
+    LRQK_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL((als_solve_wide_kernel<T>), dim3((unsigned)bh), dim3(kWideThreads), smem_s, st, (const float*)part,
+                       S, (const T*)b_q, (const T*)b_k, (const T*)q, (const T*)k_new, hq, hkv, r, d, max_iter, iter_out,
+                       deltas);
+    LRQK_HIP_CHECK(hipGetLastError());
+    return als_decode_finish<T>(ctx, b_q, b_k, a_k, head_stride, q, k_new, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat,
+                                k_hat, append_row, iter_out, deltas, defer_finish, st);
+  }
   // one 32-token chunk per wave where possible: a workgroup then pays two memory latencies
   int S = (n + kGramWaves * kGramChunk - 1) / (kGramWaves * kGramChunk);
   if (S < 1) S = 1;
@@ -688,28 +1004,8 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
   }
 #undef LRQK_SOLVE_CASE
   LRQK_HIP_CHECK(hipGetLastError());
-  FinishArgs fa{b_q, b_k, q, k_new, iter_out, deltas, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat, k_hat, a_k,
-                head_stride, append_row, nullptr, nullptr, nullptr, 0};
-  if (ctx->sidx_enabled && ctx->sidx_a_k == a_k && ctx->sidx_bh == bh && ctx->sidx_r == r && append_row >= 0 &&
-      ctx->sidx_head_rows == head_stride / r && ctx->sidx_dtype == (sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16)) {
-    // the appended row also goes into the score index; rows stay contiguous as long as rows are appended in order
-    fa.qa = (uint8_t*)ctx->sidx_qa.p;
-    fa.qs = (uint16_t*)ctx->sidx_qs.p;
-    fa.qw = (const float*)ctx->sidx_wm.p;
-    fa.q_head_rows = ctx->sidx_head_rows;
-    if (append_row == ctx->sidx_valid) ctx->sidx_valid = append_row + 1;  // (a gap is indexed on demand later)
-  }
-  if (defer_finish) {
-    // the caller lets later launches of the step absorb the finish stage (flush_pending_finish otherwise)
-    ctx->fin = fa;
-    ctx->fin_dtype = sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16;
-    ctx->fin_pending = true;   // B update, outputs and the A_K row still to be done
-    ctx->qhat_pending = true;  // q_hat has not been written yet: consumers take the iterate from iter_out
-    return LRQK_OK;
-  }
-  hipLaunchKernelGGL((als_finish_kernel<T>), dim3(finish_grid(fa)), dim3(kFinThreads), 0, st, fa);
-  LRQK_HIP_CHECK(hipGetLastError());
-  return LRQK_OK;
+  return als_decode_finish<T>(ctx, b_q, b_k, a_k, head_stride, q, k_new, bh, hq, hkv, r, d, lpr_log2, max_iter, tol, q_hat,
+                              k_hat, append_row, iter_out, deltas, defer_finish, st);
 }
 
 static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride,
@@ -721,8 +1017,10 @@ static int als_decode_checked(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, in
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(b > 0 && hq > 0 && hkv > 0 && hq % hkv == 0 && (int64_t)b * hq <= 65535, LRQK_EINVAL,
                "bad heads b=%d hq=%d hkv=%d", b, hq, hkv);
-  LRQK_REQUIRE(r > 0 && r <= kAlsMaxR, LRQK_ELIMIT, "r=%d not in 1..%d (the factor update supports rank <= %d)", r,
-               kAlsMaxR, kAlsMaxR);
+  LRQK_REQUIRE(r > 0 && r <= kWideMaxR, LRQK_ELIMIT, "r=%d not in 1..%d (the factor update supports rank <= %d)", r,
+               kWideMaxR, kWideMaxR);
+  LRQK_REQUIRE((int64_t)r * d * (int64_t)elem_size(dtype) / 16 <= 2048, LRQK_ELIMIT,
+               "r=%d x d=%d: B_Q, B_K exceed the 32 KB each that the finish stage holds in registers", r, d);
   LRQK_REQUIRE(n > 0 && n <= kprev_slots, LRQK_EINVAL, "n=%d outside 1..%d", n, kprev_slots);
   LRQK_REQUIRE(!active_idx || idx_stride >= n, LRQK_EINVAL, "idx_stride < n");
   LRQK_REQUIRE(head_stride >= r && head_stride % r == 0, LRQK_EINVAL, "head_stride must be a multiple of r");

@@ -6,7 +6,8 @@
 
 namespace lrqk {
 
-constexpr int kAlsMaxR = 32;  // one 32x32 MFMA tile
+constexpr int kAlsMaxR = 32;  // one 32x32 MFMA tile (the tuned factor-update kernels)
+constexpr int kFinMaxR = 64;  // the finish stage itself takes the ranks of the general kernels too
 constexpr int kFinThreads = 256;
 
 // The stopping test of the decode iterations is batch-wide: iteration `it` stops the loop if the
@@ -126,7 +127,7 @@ __device__ __forceinline__ void als_finish_body(const FinishArgs& fa, int h) {
   const int64_t head_stride = fa.head_stride, append_row = fa.append_row;
   constexpr int VEC = Vec16<T>::N;
   constexpr int kMaxVec = 8;  // vectors per thread per matrix: r * d / VEC <= 2048
-  __shared__ float hat[2][kAlsMaxR];
+  __shared__ float hat[2][kFinMaxR];
   __shared__ float err[2][256];
   __shared__ float red[kFinThreads / kWave][2][256];
   __shared__ int s_it;

@@ -460,6 +460,26 @@ def test_long_run_with_wrapping_caches(lrqk, oracle):
     assert n > 0 and eng._A_K.capacity > 3200 and len(eng.KVcpu) == 3000 + 2 * 128
 
 
+def test_accuracy_focused_setting(lrqk, oracle):
+    """The reference's "accuracy-focused" setting (README.md:124-131: r 64, 4096 active tokens, 128 recent ones,
+    tol 1e-10, four iterations) at a reduced context: ranks beyond 32 run the general factor-update kernels, the
+    scan its rank-64 form with the score index."""
+    _say("accuracy-focused setting")
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=128, l=9000, r=64, k=4096, L=128, steps=16,
+                        dtype=torch.bfloat16, max_iter=(4, 4), tol=(1e-10, 1e-10), rho=96, capacity=16384, tag="r64",
+                        compare_every=4)
+    assert n > 0
+
+
+@pytest.mark.parametrize("r", [40, 48])
+def test_ranks_between_the_tuned_ones(lrqk, oracle, r):
+    """Ranks 40 and 48: the general factor-update kernels and the plain scan (the score index covers 16, 32, 64)."""
+    _say("rank", r)
+    _, _, n = _lockstep(lrqk, oracle, b=2, hq=4, hkv=2, d=128, l=1500, r=r, k=256, L=16, steps=20,
+                        dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=2 * r, capacity=2048, tag="r%d" % r)
+    assert n > 0
+
+
 def test_llama_shape_bf16_short(lrqk, oracle):
     """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, r 32, k 2048, L 64, bf16) at an
     8K context, long enough (70 steps) for the 64-token ring to be flushed to the host store once."""

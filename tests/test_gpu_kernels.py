@@ -549,7 +549,10 @@ def _als_inputs(g, b, hq, hkv, n, d, r, cap, dtype):
                                                 (torch.bfloat16, 32, 8, 2112, 128, 32), (torch.float32, 2, 2, 70, 8, 3),
                                                 # head widths 64 and 256 (bf16 rows that the d = 128 kernel does not take)
                                                 (torch.bfloat16, 8, 2, 300, 64, 16), (torch.bfloat16, 4, 1, 272, 256, 32),
-                                                (torch.float32, 4, 2, 150, 64, 8)])
+                                                (torch.float32, 4, 2, 150, 64, 8),
+                                                # ranks beyond 32 (the general kernels): 64, 48 and 40
+                                                (torch.bfloat16, 8, 2, 600, 128, 64), (torch.float32, 2, 1, 200, 64, 48),
+                                                (torch.bfloat16, 4, 4, 333, 128, 40)])
 @pytest.mark.parametrize("max_iter,tol", [(1, 0.0), (2, 0.0), (3, 1e30), (4, 1e-6)])
 def test_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol)
