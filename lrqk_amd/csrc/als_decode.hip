@@ -599,18 +599,24 @@ constexpr int kWideTile = 32;   // active rows per step
 constexpr int kWideMaxR = 64;
 
 // part per (head, split): r * r sums A^T A, then r sums A^T w.
+// A tile of 32 active rows at a time: their A_K rows (as 16-byte pieces, zero-padded to 64 columns) and K rows go
+// through LDS; thread (ti, tj) of a 16 x 16 grid keeps the 4 x 4 block (4 ti.., 4 tj..) of A^T A in registers.
+// Every load is unconditional (clamped index, masked value).  r % 8 == 0 and 16-byte aligned rows for the vector
+// loads of A_K (r = 40, 48, 56, 64 with bf16; multiples of 4 with fp32); other ranks take one element at a time.
 template <typename T>
 __global__ __launch_bounds__(kWideThreads) void als_gram_wide_kernel(
     const T* __restrict__ a_k, int64_t head_stride, int64_t a_rows, const int32_t* __restrict__ active_idx,
     int64_t idx_stride, T* k_prev, int kprev_slots, int n, const T* __restrict__ q, int r, int d,
     float* __restrict__ part, int S, GramAppend ap) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int lda = kWideMaxR + 4;           // floats per staged row of A (16-byte aligned rows, 4 banks apart)
   extern __shared__ __align__(16) float wsm[];
-  float* a_s = wsm;                            // [kWideTile][r + 1]
-  float* w_s = a_s + kWideTile * (r + 1);      // [kWideTile]
+  float* a_s = wsm;                            // [kWideTile][lda]
+  float* w_s = a_s + kWideTile * lda;          // [kWideTile]
   float* q_s = w_s + kWideTile;                // [d]
+  __shared__ int32_t tok_s[kWideTile];
   const int tid = threadIdx.x;
   const int h = blockIdx.y, s = blockIdx.x;
-  const int lda = r + 1;
   const T* A = a_k + (int64_t)h * head_stride;
   const T* Kp = k_prev + (int64_t)h * kprev_slots * d;
   const T* knew_h = Kp;
@@ -619,49 +625,79 @@ __global__ __launch_bounds__(kWideThreads) void als_gram_wide_kernel(
     knew_h = (const T*)ap.k_new + ((int64_t)bb * ap.hkv + kvh) * d;
   }
   for (int c = tid; c < d; c += kWideThreads) q_s[c] = ld_f32<T>(q, (int64_t)h * d + c);
+  const bool vec_a = r % VEC == 0 && ((uintptr_t)A % 16 == 0) && (head_stride * sizeof(T)) % 16 == 0;
   const int rows_per_split = (n + S - 1) / S;
   const int s0 = s * rows_per_split, s1 = min(n, s0 + rows_per_split);
-  constexpr int kPer = kWideMaxR * kWideMaxR / kWideThreads;  // 16 sums of A^T A per thread
-  float acc[kPer], racc = 0.0f;
+  const int ti = tid >> 4, tj = tid & 15;
+  float acc[4][4], racc = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) acc[i] = 0.0f;
-  __syncthreads();
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+  const int vpr = d / VEC;  // 16-byte pieces per K row (a power of two <= 64)
   for (int t0 = s0; t0 < s1; t0 += kWideTile) {
     const int rows = min(kWideTile, s1 - t0);
-    // the rows of A_K of the tile's tokens (zero where the slot holds no token or its row does not exist yet)
-    for (int e = tid; e < rows * r; e += kWideThreads) {
-      const int row = e / r, j = e % r;
-      const int t = t0 + row;
-      int32_t tok = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
-      if (t == ap.slot) tok = ap.token;
-      const bool ok = tok >= 0 && (int64_t)tok < a_rows;
-      a_s[row * lda + j] = ok ? ld_f32<T>(A, (int64_t)tok * r + j) : 0.0f;
-    }
-    // w = K q of the tile's rows: eight lanes per row
-    {
-      const int row = tid >> 3, sub = tid & 7;
-      float wv = 0.0f;
-      if (row < rows) {
-        const int t = t0 + row;
-        const T* kr = t == ap.slot ? knew_h : Kp + (int64_t)t * d;
-        for (int c = sub; c < d; c += 8) wv = fmaf(ld_f32<T>(kr, c), q_s[c], wv);
-      }
-      wv = group_sum(wv, 8);
-      if (sub == 0 && row < kWideTile) w_s[row] = row < rows ? wv : 0.0f;
+    if (tid < kWideTile) {
+      const int t = min(t0 + tid, n - 1);
+      const int32_t id = active_idx ? active_idx[(int64_t)h * idx_stride + t] : t;
+      tok_s[tid] = t == ap.slot ? ap.token : id;
     }
     __syncthreads();
+    // the rows of A_K of the tile's tokens (zero where the slot holds no token, and beyond column r)
+    if (vec_a) {
+      const int pieces = kWideMaxR / VEC;  // per staged row
+      for (int e = tid; e < kWideTile * pieces; e += kWideThreads) {
+        const int row = e / pieces, pc = e % pieces;
+        const int32_t tok = tok_s[row];
+        const bool ok = row < rows && tok >= 0 && (int64_t)tok < a_rows && pc * VEC < r;
+        const int64_t sr = min(max((int64_t)tok, (int64_t)0), a_rows - 1);
+        Vec16<T> v;
+        v.load(A + sr * r + min(pc * VEC, r - VEC));
+        float f[VEC];
+        v.unpack(f);
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-      const int e = tid + i * kWideThreads;
-      if (e < r * r) {
-        const int a = e / r, b2 = e % r;
-        float v = acc[i];
-        for (int row = 0; row < rows; ++row) v = fmaf(a_s[row * lda + a], a_s[row * lda + b2], v);
-        acc[i] = v;
+        for (int x = 0; x < VEC; ++x) a_s[row * lda + pc * VEC + x] = ok ? f[x] : 0.0f;
+      }
+    } else {
+      for (int e = tid; e < kWideTile * kWideMaxR; e += kWideThreads) {
+        const int row = e / kWideMaxR, j = e % kWideMaxR;
+        const int32_t tok = tok_s[row];
+        const bool ok = row < rows && tok >= 0 && (int64_t)tok < a_rows && j < r;
+        const int64_t sr = min(max((int64_t)tok, (int64_t)0), a_rows - 1);
+        const float v = ld_f32<T>(A, sr * r + min(j, r - 1));
+        a_s[row * lda + j] = ok ? v : 0.0f;
       }
     }
-    if (tid < r)
-      for (int row = 0; row < rows; ++row) racc = fmaf(w_s[row], a_s[row * lda + tid], racc);
+    // w = K q of the tile's rows: eight lanes per row, 16-byte pieces
+    {
+      const int row = tid >> 3, sub = tid & 7;
+      const int t = min(t0 + row, n - 1);
+      const T* kr = t == ap.slot ? knew_h : Kp + (int64_t)t * d;
+      float wv = 0.0f;
+      for (int pc = sub; pc < vpr; pc += 8) {
+        Vec16<T> v;
+        v.load(kr + pc * VEC);
+        float f[VEC];
+        v.unpack(f);
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) wv = fmaf(f[x], q_s[pc * VEC + x], wv);
+      }
+      wv = group_sum(wv, 8);
+      if (sub == 0) w_s[row] = row < rows ? wv : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int row = 0; row < kWideTile; ++row) {  // (rows beyond the tile are zero)
+      const float4 ai = *reinterpret_cast<const float4*>(a_s + row * lda + 4 * ti);
+      const float4 aj = *reinterpret_cast<const float4*>(a_s + row * lda + 4 * tj);
+      const float av[4] = {ai.x, ai.y, ai.z, ai.w}, bv[4] = {aj.x, aj.y, aj.z, aj.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    if (tid < kWideMaxR)
+      for (int row = 0; row < kWideTile; ++row) racc = fmaf(w_s[row], a_s[row * lda + tid], racc);
     __syncthreads();
   }
   if (ap.slot >= s0 && ap.slot < s1) {  // this workgroup owns the new token's slot: the ring append
@@ -678,10 +714,12 @@ __global__ __launch_bounds__(kWideThreads) void als_gram_wide_kernel(
   }
   float* pout = part + ((int64_t)h * S + s) * (r * r + r);
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    const int e = tid + i * kWideThreads;
-    if (e < r * r) pout[e] = acc[i];
-  }
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int a = 4 * ti + i, b2 = 4 * tj + j;
+      if (a < r && b2 < r) pout[a * r + b2] = acc[i][j];
+    }
   if (tid < r) pout[r * r + tid] = racc;
 }
 
@@ -748,8 +786,19 @@ __global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
     kv[c] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
   }
   __syncthreads();
-  // G_K = B_K B_K^T, G_Q = B_Q B_Q^T + A^T A (partial sums added in split order)
+  // G_K = B_K B_K^T, G_Q = B_Q B_Q^T + A^T A (partial sums added in split order, eight loads in flight)
   const float* pin = part + (int64_t)h * S * ne;
+  auto summed = [&](int e) {
+    float v = 0.0f;
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] = pin[(int64_t)min(s0 + u, S - 1) * ne + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v += s0 + u < S ? t[u] : 0.0f;
+    }
+    return v;
+  };
   for (int e = tid; e < r * r; e += kWideThreads) {
     const int i = e / r, j = e % r;
     float gq = 0.0f, gk = 0.0f;
@@ -757,9 +806,7 @@ __global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
       gq = fmaf(Bq[i * ldb + c], Bq[j * ldb + c], gq);
       gk = fmaf(Bk[i * ldb + c], Bk[j * ldb + c], gk);
     }
-    float ga = 0.0f;
-    for (int s = 0; s < S; ++s) ga += pin[(int64_t)s * ne + e];
-    GQ[i * ldg + j] = gq + ga;
+    GQ[i * ldg + j] = gq + summed(e);
     GK[i * ldg + j] = gk;
   }
   if (tid < r) {
@@ -768,7 +815,7 @@ __global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
       rq = fmaf(qv[c], Bq[tid * ldb + c], rq);
       kb = fmaf(kv[c], Bk[tid * ldb + c], kb);
     }
-    for (int s = 0; s < S; ++s) aw += pin[(int64_t)s * ne + r * r + tid];
+    aw = summed(r * r + tid);
     rhs_q[tid] = rq + aw;   // q B_Q^T + (q K^T) A
     kB[tid] = kb;           // k B_K^T
   }
@@ -911,7 +958,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
     float* part = (float*)ctx->als_part.p;
     float* iter_out = (float*)ctx->als_iter.p;
     float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
-    const size_t smem_g = ((size_t)kWideTile * (r + 1) + kWideTile + d) * sizeof(float);
+    const size_t smem_g = ((size_t)kWideTile * (kWideMaxR + 4) + kWideTile + d) * sizeof(float);
     const size_t smem_s = ((size_t)2 * r * (d + 1) + (size_t)2 * r * (r + 1) + 2 * d + 11 * kWideMaxR) * sizeof(float);
     LRQK_REQUIRE(smem_s <= (size_t)160 * 1024 - 256, LRQK_ELIMIT, "r=%d with rows of %d elements needs too much LDS", r, d);
     static std::atomic<size_t> wide_allowed_dev[kMaxDeviceSlots];
