@@ -30,7 +30,8 @@ extern "C" {
 #define LRQK_EHIP (-2)     /* a HIP runtime call failed */
 #define LRQK_ELIMIT (-3)   /* size beyond what the kernels support */
 
-#define LRQK_MAX_R 64          /* scan / select; the factor updates (lrqk_als_*) take r <= 32 */
+#define LRQK_MAX_R 64          /* every entry; the factor updates (lrqk_als_*) are tuned for r <= 32 and run
+                                * general kernels beyond (r (r + d) <= 12288 for the prefill) */
 #define LRQK_MAX_TOPK 8192
 #define LRQK_MAX_DECODE_ITERS 16
 
@@ -205,7 +206,8 @@ int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head
  * change of A_Q and A_K below tol) is evaluated on the device: once it fires the remaining
  * launches return at once, and the host never waits.  r <= 32: bf16 input with d <= 128 runs on
  * the bf16 matrix cores (fp32 operands as three bf16 pieces each, fp32 accumulation), fp32 input
- * or d = 256 on fp32 MFMA tiles, other shapes on a generic kernel.  Returns 0. */
+ * or d = 256 on fp32 MFMA tiles, other shapes -- and ranks up to 64 (README.md:124-131 of the reference
+ * names r = 64) -- on a general kernel, as long as r (r + d) <= 12288.  Returns 0. */
 int lrqk_als_prefill(lrqk_ctx* ctx, const void* q, const void* k, float* a_q, float* a_k, float* b_q,
                      float* b_k, int b, int hq, int hkv, int64_t l, int r, int d, int max_iter, float tol,
                      int dtype, void* stream);

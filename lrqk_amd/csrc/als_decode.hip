@@ -723,111 +723,194 @@ __global__ __launch_bounds__(kWideThreads) void als_gram_wide_kernel(
   if (tid < r) pout[r * r + tid] = racc;
 }
 
-// In-place inverse of the symmetric positive definite r x r matrix G (row stride ld) by the whole workgroup:
-// scaled to unit diagonal, Gauss-Jordan without pivoting, scaled back.  colp, rowp, sc: r floats each.
-__device__ __forceinline__ void wide_invert(float* G, int ld, int r, float* colp, float* rowp, float* sc) {
-  const int tid = threadIdx.x;
-  if (tid < r) sc[tid] = rsqrtf(G[tid * ld + tid]);
-  __syncthreads();
-  for (int e = tid; e < r * r; e += kWideThreads) G[(e / r) * ld + e % r] *= sc[e / r] * sc[e % r];
-  __syncthreads();
-  for (int p = 0; p < r; ++p) {
-    if (tid < r) {
-      colp[tid] = G[tid * ld + p];
-      rowp[tid] = G[p * ld + tid];
-    }
-    __syncthreads();
-    const float piv = 1.0f / colp[p];
-    for (int e = tid; e < r * r; e += kWideThreads) {
-      const int i = e / r, j = e % r;
-      float v;
-      if (i == p)
-        v = j == p ? piv : rowp[j] * piv;
-      else if (j == p)
-        v = -colp[i] * piv;
-      else
-        v = fmaf(-colp[i] * piv, rowp[j], G[i * ld + j]);
-      G[i * ld + j] = v;
-    }
-    __syncthreads();
-  }
-  for (int e = tid; e < r * r; e += kWideThreads) G[(e / r) * ld + e % r] *= sc[e / r] * sc[e % r];
-  __syncthreads();
-}
-
+// One workgroup per head.  Thread (ti, tj) of a 16 x 16 grid keeps the 4 x 4 block (4 ti.., 4 tj..) of G_K and of
+// G_Q in registers from the moment they are formed (B B^T from transposed copies of B_Q, B_K in LDS, plus the
+// partial sums of A^T A) until their inverses are complete: Gauss-Jordan without pivoting on the matrices scaled
+// to unit diagonal (symmetric positive definite), both at once, one barrier per pivot -- the owners of column p and
+// row p publish them in LDS (two buffers in turn), every thread updates its blocks.  Rows and columns beyond r are
+// an identity block.  Then the alternating rank-1 solves with the formulas of als_solve_kernel.
 template <typename T>
 __global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
     const float* __restrict__ part, int S, const T* __restrict__ b_q, const T* __restrict__ b_k,
     const T* __restrict__ q, const T* __restrict__ k_new, int hq, int hkv, int r, int d, int max_iter,
     float* __restrict__ iter_out, float* __restrict__ deltas) {
   extern __shared__ __align__(16) float wsm[];
-  const int ldb = d + 1, ldg = r + 1;
-  float* Bq = wsm;                 // [r][d + 1]
-  float* Bk = Bq + r * ldb;        // [r][d + 1]
-  float* GQ = Bk + r * ldb;        // [r][r + 1]
-  float* GK = GQ + r * ldg;        // [r][r + 1]
-  float* qv = GK + r * ldg;        // [d]
+  constexpr int R = kWideMaxR, ldt = R + 4, ldg = R + 1;
+  float* BtQ = wsm;                // [d][ldt]  B_Q transposed (columns beyond r zero)
+  float* BtK = BtQ + d * ldt;      // [d][ldt]
+  float* GQ = BtK + d * ldt;       // [R][ldg]  inverses
+  float* GK = GQ + R * ldg;        // [R][ldg]
+  float* qv = GK + R * ldg;        // [d]
   float* kv = qv + d;              // [d]
-  float* vec = kv + d;             // 10 vectors of kWideMaxR
-  float* rhs_q = vec, *kB = vec + 64, *hk0 = vec + 128, *yq0 = vec + 192, *hk = vec + 256, *hqv = vec + 320;
-  float* z = vec + 384, *y = vec + 448, *colp = vec + 512, *rowp = vec + 576;
-  float* sc = vec + 640;           // [kWideMaxR]
+  float* vec = kv + d;             // vectors of R
+  float* rhs_q = vec, *kB = vec + R, *hk0 = vec + 2 * R, *yq0 = vec + 3 * R, *hk = vec + 4 * R, *hqv = vec + 5 * R;
+  float* z = vec + 6 * R, *y = vec + 7 * R;
+  float* pub = vec + 8 * R;        // [2 buffers][colQ, rowQ, colK, rowK][R]
+  float* scq = pub + 8 * R, *sck = scq + R;
   __shared__ float s_red[4];
   const int tid = threadIdx.x;
+  const int ti = tid >> 4, tj = tid & 15;
   const int h = blockIdx.x;
   const int b = h / hq, kvh = (h % hq) / (hq / hkv);
   const int ne = r * r + r;
-  for (int e = tid; e < r * d; e += kWideThreads) {
-    Bq[(e / d) * ldb + e % d] = ld_f32<T>(b_q, (int64_t)h * r * d + e);
-    Bk[(e / d) * ldb + e % d] = ld_f32<T>(b_k, (int64_t)h * r * d + e);
+  for (int e = tid; e < R * d; e += kWideThreads) {
+    const int row = e / d, c = e % d;  // (d is a power of two)
+    const bool ok = row < r;
+    const int64_t src = (int64_t)h * r * d + (int64_t)min(row, r - 1) * d + c;
+    const float vq = ld_f32<T>(b_q, src), vk = ld_f32<T>(b_k, src);
+    BtQ[c * ldt + row] = ok ? vq : 0.0f;
+    BtK[c * ldt + row] = ok ? vk : 0.0f;
   }
   for (int c = tid; c < d; c += kWideThreads) {
     qv[c] = ld_f32<T>(q, (int64_t)h * d + c);
     kv[c] = ld_f32<T>(k_new, ((int64_t)b * hkv + kvh) * d + c);
   }
   __syncthreads();
-  // G_K = B_K B_K^T, G_Q = B_Q B_Q^T + A^T A (partial sums added in split order, eight loads in flight)
-  const float* pin = part + (int64_t)h * S * ne;
-  auto summed = [&](int e) {
-    float v = 0.0f;
-    for (int s0 = 0; s0 < S; s0 += 8) {
-      float t[8];
+  // ---- G_K = B_K B_K^T, G_Q = B_Q B_Q^T + A^T A
+  float gq[4][4], gk[4][4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) t[u] = pin[(int64_t)min(s0 + u, S - 1) * ne + e];
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v += s0 + u < S ? t[u] : 0.0f;
-    }
-    return v;
-  };
-  for (int e = tid; e < r * r; e += kWideThreads) {
-    const int i = e / r, j = e % r;
-    float gq = 0.0f, gk = 0.0f;
-    for (int c = 0; c < d; ++c) {
-      gq = fmaf(Bq[i * ldb + c], Bq[j * ldb + c], gq);
-      gk = fmaf(Bk[i * ldb + c], Bk[j * ldb + c], gk);
-    }
-    GQ[i * ldg + j] = gq + summed(e);
-    GK[i * ldg + j] = gk;
+    for (int j = 0; j < 4; ++j) gq[i][j] = gk[i][j] = 0.0f;
+#pragma unroll 4
+  for (int c = 0; c < d; ++c) {
+    const float4 qi = *reinterpret_cast<const float4*>(BtQ + c * ldt + 4 * ti);
+    const float4 qj = *reinterpret_cast<const float4*>(BtQ + c * ldt + 4 * tj);
+    const float4 ki = *reinterpret_cast<const float4*>(BtK + c * ldt + 4 * ti);
+    const float4 kj = *reinterpret_cast<const float4*>(BtK + c * ldt + 4 * tj);
+    const float a[4] = {qi.x, qi.y, qi.z, qi.w}, bb[4] = {qj.x, qj.y, qj.z, qj.w};
+    const float e[4] = {ki.x, ki.y, ki.z, ki.w}, f[4] = {kj.x, kj.y, kj.z, kj.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        gq[i][j] = fmaf(a[i], bb[j], gq[i][j]);
+        gk[i][j] = fmaf(e[i], f[j], gk[i][j]);
+      }
   }
+  const float* pin = part + (int64_t)h * S * ne;
+  for (int s = 0; s < S; ++s) {  // (split order; the block's sixteen loads of a split go out together)
+    float t[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        t[i][j] = pin[(int64_t)s * ne + min(4 * ti + i, r - 1) * r + min(4 * tj + j, r - 1)];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gq[i][j] += t[i][j];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = 4 * ti + i, col = 4 * tj + j;
+      if (row >= r || col >= r) gq[i][j] = gk[i][j] = row == col ? 1.0f : 0.0f;
+    }
   if (tid < r) {
     float rq = 0.0f, kb = 0.0f, aw = 0.0f;
     for (int c = 0; c < d; ++c) {
-      rq = fmaf(qv[c], Bq[tid * ldb + c], rq);
-      kb = fmaf(kv[c], Bk[tid * ldb + c], kb);
+      rq = fmaf(qv[c], BtQ[c * ldt + tid], rq);
+      kb = fmaf(kv[c], BtK[c * ldt + tid], kb);
     }
-    aw = summed(r * r + tid);
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] = pin[(int64_t)min(s0 + u, S - 1) * ne + r * r + tid];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) aw += s0 + u < S ? t[u] : 0.0f;
+    }
     rhs_q[tid] = rq + aw;   // q B_Q^T + (q K^T) A
     kB[tid] = kb;           // k B_K^T
   }
-  if (tid < kWave) {
+  if (tid >= kWideThreads - kWave) {  // (the last wave: the first is busy with the products above)
     float v = 0.0f;
-    for (int c = tid; c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
+    for (int c = tid - (kWideThreads - kWave); c < d; c += kWave) v = fmaf(qv[c], kv[c], v);
     v = wave_sum(v);
-    if (tid == 0) s_red[0] = v;  // q . k
+    if (tid == kWideThreads - kWave) s_red[0] = v;  // q . k
+  }
+  // ---- scale to unit diagonal
+  if (ti == tj) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      scq[4 * ti + i] = rsqrtf(gq[i][i]);
+      sck[4 * ti + i] = rsqrtf(gk[i][i]);
+    }
   }
   __syncthreads();
-  wide_invert(GK, ldg, r, colp, rowp, sc);
-  wide_invert(GQ, ldg, r, colp, rowp, sc);
+  float sqr[4], sqc[4], skr[4], skc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    sqr[i] = scq[4 * ti + i];
+    sqc[i] = scq[4 * tj + i];
+    skr[i] = sck[4 * ti + i];
+    skc[i] = sck[4 * tj + i];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      gq[i][j] *= sqr[i] * sqc[j];
+      gk[i][j] *= skr[i] * skc[j];
+    }
+  // ---- Gauss-Jordan, both matrices, one barrier per pivot
+  for (int p = 0; p < r; ++p) {
+    float* pb = pub + (p & 1) * 4 * R;
+    const int pt = p >> 2, pe = p & 3;
+    if (tj == pt) {  // this thread holds column p of rows 4 ti ..
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float cqv = gq[i][0], ckv = gk[i][0];
+#pragma unroll
+        for (int j = 1; j < 4; ++j) {
+          cqv = pe == j ? gq[i][j] : cqv;
+          ckv = pe == j ? gk[i][j] : ckv;
+        }
+        pb[4 * ti + i] = cqv;
+        pb[2 * R + 4 * ti + i] = ckv;
+      }
+    }
+    if (ti == pt) {  // row p of columns 4 tj ..
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float rqv = gq[0][j], rkv = gk[0][j];
+#pragma unroll
+        for (int i = 1; i < 4; ++i) {
+          rqv = pe == i ? gq[i][j] : rqv;
+          rkv = pe == i ? gk[i][j] : rkv;
+        }
+        pb[R + 4 * tj + j] = rqv;
+        pb[3 * R + 4 * tj + j] = rkv;
+      }
+    }
+    __syncthreads();
+    const float pq_ = 1.0f / pb[p], pk_ = 1.0f / pb[2 * R + p];
+    const float4 cq4 = *reinterpret_cast<const float4*>(pb + 4 * ti), rq4 = *reinterpret_cast<const float4*>(pb + R + 4 * tj);
+    const float4 ck4 = *reinterpret_cast<const float4*>(pb + 2 * R + 4 * ti), rk4 = *reinterpret_cast<const float4*>(pb + 3 * R + 4 * tj);
+    const float cq[4] = {cq4.x, cq4.y, cq4.z, cq4.w}, rq[4] = {rq4.x, rq4.y, rq4.z, rq4.w};
+    const float ck[4] = {ck4.x, ck4.y, ck4.z, ck4.w}, rk[4] = {rk4.x, rk4.y, rk4.z, rk4.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool rp = 4 * ti + i == p, cp = 4 * tj + j == p;
+        const float uq = fmaf(-cq[i] * pq_, rq[j], gq[i][j]), uk = fmaf(-ck[i] * pk_, rk[j], gk[i][j]);
+        const float vq = rp ? (cp ? pq_ : rq[j] * pq_) : (cp ? -cq[i] * pq_ : uq);
+        const float vk = rp ? (cp ? pk_ : rk[j] * pk_) : (cp ? -ck[i] * pk_ : uk);
+        gq[i][j] = vq;
+        gk[i][j] = vk;
+      }
+  }
+  // ---- scale back; the inverses go to LDS
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      GQ[(4 * ti + i) * ldg + 4 * tj + j] = gq[i][j] * sqr[i] * sqc[j];
+      GK[(4 * ti + i) * ldg + 4 * tj + j] = gk[i][j] * skr[i] * skc[j];
+    }
+  __syncthreads();
   const float sqk = s_red[0];
   // out[c] = sum_i in[i] G[i][c]
   auto vecmat = [&](const float* in, const float* G, float* out) {
@@ -868,7 +951,7 @@ __global__ __launch_bounds__(kWideThreads) void als_solve_wide_kernel(
   __syncthreads();
   for (int it = 0; it < max_iter; ++it) {
     rank1(yq0, hk, GQ, hqv);   // q_hat (G_Q + k_hat^T k_hat) = rhs_q + s k_hat
-    rank1(hk0, hqv, GK, y);    // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat   (y is free again: out may alias it)
+    rank1(hk0, hqv, GK, y);    // k_hat' (G_K + q_hat^T q_hat) = kB + s q_hat   (the result takes y's place)
     float df = 0.0f;
     if (tid < r) {
       df = hk[tid] - y[tid];
@@ -959,7 +1042,7 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
     float* iter_out = (float*)ctx->als_iter.p;
     float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
     const size_t smem_g = ((size_t)kWideTile * (kWideMaxR + 4) + kWideTile + d) * sizeof(float);
-    const size_t smem_s = ((size_t)2 * r * (d + 1) + (size_t)2 * r * (r + 1) + 2 * d + 11 * kWideMaxR) * sizeof(float);
+    const size_t smem_s = ((size_t)2 * d * (kWideMaxR + 4) + (size_t)2 * kWideMaxR * (kWideMaxR + 1) + 2 * d + 18 * kWideMaxR) * sizeof(float);
     LRQK_REQUIRE(smem_s <= (size_t)160 * 1024 - 256, LRQK_ELIMIT, "r=%d with rows of %d elements needs too much LDS", r, d);
     static std::atomic<size_t> wide_allowed_dev[kMaxDeviceSlots];
     std::atomic<size_t>& wide_allowed = wide_allowed_dev[per_device_slot()];
