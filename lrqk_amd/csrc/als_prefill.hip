@@ -25,23 +25,57 @@ constexpr int kPfThreads = 256;
 constexpr int kPfTile = 32;
 constexpr int kPfMaxPer = 48;  // accumulators per thread: r*(r+d) <= 256*48 (r = 64 with rows of 128 elements)
 
-// acc[e] += sum_rows a_s[row][j] * (c < r ? a_s[row][c] : x_s[row][c-r]),  e = j*(r+d)+c
+// Sums of a tile: out[j][c] += sum_rows a_s[row][j] * (c < r ? a_s[row][c] : x_s[row][c-r]),  0 <= j < r,
+// 0 <= c < r + d.  The 256 threads form a 16 x 16 grid; thread (tj, tc) owns rows j = tj + 16 i (i < I) and columns
+// c = tc + 16 k (k < 48 / I) and keeps them in acc[i * K + k]: I values of A and K of [A | X] per tile row feed
+// I * K products (a sixth of the LDS reads of one output at a time).  I = ceil(r / 16), which the limit
+// r (r + d) <= 12288 makes enough: 16 K >= r + d.
+template <int I>
+__device__ __forceinline__ void accumulate_gram_tile(const float* a_s, int lda, const float* x_s, int ldx, int rows, int r,
+                                                     int d, float* acc) {
+  constexpr int K = kPfMaxPer / I;
+  const int tj = threadIdx.x >> 4, tc = threadIdx.x & 15;
+  const float* cp[K];  // column c of a row: in the A tile or in the X tile
+  int cs[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int c = min(tc + 16 * k, r + d - 1);
+    cp[k] = c < r ? a_s + c : x_s + (c - r);
+    cs[k] = c < r ? lda : ldx;
+  }
+  for (int row = 0; row < rows; ++row) {
+    float av[I], cv[K];
+#pragma unroll
+    for (int i = 0; i < I; ++i) av[i] = a_s[row * lda + min(tj + 16 * i, r - 1)];
+#pragma unroll
+    for (int k = 0; k < K; ++k) cv[k] = cp[k][row * cs[k]];
+#pragma unroll
+    for (int i = 0; i < I; ++i)
+#pragma unroll
+      for (int k = 0; k < K; ++k) acc[i * K + k] = fmaf(av[i], cv[k], acc[i * K + k]);
+  }
+}
 __device__ __forceinline__ void accumulate_gram(const float* a_s, int lda, const float* x_s, int ldx, int rows, int r,
                                                 int d, float* acc) {
-  const int ne = r * (r + d);
+  if (r <= 16)
+    accumulate_gram_tile<1>(a_s, lda, x_s, ldx, rows, r, d, acc);
+  else if (r <= 32)
+    accumulate_gram_tile<2>(a_s, lda, x_s, ldx, rows, r, d, acc);
+  else if (r <= 48)
+    accumulate_gram_tile<3>(a_s, lda, x_s, ldx, rows, r, d, acc);
+  else
+    accumulate_gram_tile<4>(a_s, lda, x_s, ldx, rows, r, d, acc);
+}
+// The sums of accumulate_gram to `out` (packed [r][r + d]).
+__device__ __forceinline__ void store_gram(const float* acc, int r, int d, float* __restrict__ out) {
+  const int I = r <= 16 ? 1 : r <= 32 ? 2 : r <= 48 ? 3 : 4;
+  const int K = kPfMaxPer / I;
+  const int tj = threadIdx.x >> 4, tc = threadIdx.x & 15;
 #pragma unroll
-  for (int i = 0; i < kPfMaxPer; ++i) {
-    const int e = threadIdx.x + i * kPfThreads;
-    if (e < ne) {
-      const int j = e / (r + d), c = e % (r + d);
-      float v = acc[i];
-      if (c < r) {
-        for (int row = 0; row < rows; ++row) v = fmaf(a_s[row * lda + j], a_s[row * lda + c], v);
-      } else {
-        for (int row = 0; row < rows; ++row) v = fmaf(a_s[row * lda + j], x_s[row * ldx + c - r], v);
-      }
-      acc[i] = v;
-    }
+  for (int e = 0; e < kPfMaxPer; ++e) {
+    const int i = e / K, k = e % K;
+    const int j = tj + 16 * i, c = tc + 16 * k;
+    if (i < I && j < r && c < r + d) out[j * (r + d) + c] = acc[e];
   }
 }
 
@@ -84,15 +118,30 @@ __global__ __launch_bounds__(kPfThreads) void pf_pass_generic_kernel(const T* __
     }
     __syncthreads();
     if (apply) {
-      for (int e = tid; e < rows * r; e += kPfThreads) {
-        const int row = e / r, j = e % r;
-        float v = 0.0f;
-        for (int c = 0; c < d; ++c) v = fmaf(x_s[row * ldx + c], m_s[j * ldx + c], v);
-        const float old = Ah[t0 * r + e];
-        const float df = old - v;
-        dsum = fmaf(df, df, dsum);
-        Ah[t0 * r + e] = v;
-        a_s[row * lda + j] = v;
+      // thread -> (row of the tile, eight columns j = jg + 8 u of the new A): one element of X feeds eight products
+      static_assert(kPfTile == 32 && kPfThreads == 256, "32 rows x 8 column groups");
+      const int row = tid & (kPfTile - 1), jg = tid >> 5;
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = 0.0f;
+      const float* mrow[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) mrow[u] = m_s + min(jg + 8 * u, r - 1) * ldx;
+      for (int c = 0; c < d; ++c) {
+        const float x = x_s[row * ldx + c];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = fmaf(x, mrow[u][c], v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = jg + 8 * u;
+        if (row < rows && j < r) {
+          const float old = Ah[(t0 + row) * r + j];
+          const float df = old - v[u];
+          dsum = fmaf(df, df, dsum);
+          Ah[(t0 + row) * r + j] = v[u];
+          a_s[row * lda + j] = v[u];
+        }
       }
       __syncthreads();
     }
@@ -100,12 +149,7 @@ __global__ __launch_bounds__(kPfThreads) void pf_pass_generic_kernel(const T* __
     __syncthreads();
   }
   const int ne = r * (r + d);
-  float* out = part + ((int64_t)h * S + s) * ne;
-#pragma unroll
-  for (int i = 0; i < kPfMaxPer; ++i) {
-    const int e = tid + i * kPfThreads;
-    if (e < ne) out[e] = acc[i];
-  }
+  store_gram(acc, r, d, part + ((int64_t)h * S + s) * ne);
   if (apply) {
     dsum = wave_sum(dsum);
     if (lane_id() == 0) red[wave_id()] = dsum;
@@ -1017,6 +1061,9 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   const bool mfma = r <= 32 && d % VEC == 0 && d <= 256 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)k % 16 == 0);
   const bool small32 = r <= 32 && d <= kPfSmallThreads - 32 && d % 4 == 0;
   LRQK_REQUIRE(mfma || ne <= kPfThreads * kPfMaxPer, LRQK_ELIMIT, "r*(r+d)=%d exceeds %d", ne, kPfThreads * kPfMaxPer);
+  // (the general pass: a 16 x 16 thread grid with ceil(r / 16) rows and 48 / that many columns of the sums per thread)
+  LRQK_REQUIRE(mfma || (r <= 64 && 16 * (kPfMaxPer / ((r + 15) / 16)) >= r + d), LRQK_ELIMIT,
+               "r=%d with rows of %d elements exceeds the general kernel's tile", r, d);
   // splits of the long axis: about one workgroup per CU (a pass keeps one wave per SIMD busy), but
   // at least 128 rows per split
   int S = std::max(1, std::min(64, 256 / bh));
