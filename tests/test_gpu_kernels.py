@@ -552,7 +552,10 @@ def _als_inputs(g, b, hq, hkv, n, d, r, cap, dtype):
                                                 (torch.float32, 4, 2, 150, 64, 8),
                                                 # ranks beyond 32 (the general kernels): 64, 48 and 40
                                                 (torch.bfloat16, 8, 2, 600, 128, 64), (torch.float32, 2, 1, 200, 64, 48),
-                                                (torch.bfloat16, 4, 4, 333, 128, 40)])
+                                                (torch.bfloat16, 4, 4, 333, 128, 40),
+                                                # ... an odd one (A_K rows one element at a time), 56, 64 in fp32
+                                                (torch.float32, 2, 1, 100, 64, 33), (torch.bfloat16, 2, 2, 150, 128, 56),
+                                                (torch.float32, 4, 2, 272, 128, 64)])
 @pytest.mark.parametrize("max_iter,tol", [(1, 0.0), (2, 0.0), (3, 1e30), (4, 1e-6)])
 def test_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol):
     _check_als_decode(ops, ws, oracle, dtype, hq, hkv, n, d, r, max_iter, tol)
@@ -681,7 +684,8 @@ def test_als_prefill_long_sums(ops, ws, oracle):
                           (torch.bfloat16, 4, 1, 600, 128, 6, 2, 0.0),
                           # ranks beyond 32 (the general kernels): 64 with rows of 128 elements, 48, 40
                           (torch.bfloat16, 4, 2, 1500, 128, 64, 2, 0.0), (torch.float32, 2, 1, 700, 64, 48, 2, 0.0),
-                          (torch.bfloat16, 2, 1, 900, 128, 40, 3, 0.0)])
+                          (torch.bfloat16, 2, 1, 900, 128, 40, 3, 0.0), (torch.float32, 2, 1, 500, 64, 33, 2, 0.0),
+                          (torch.float32, 2, 2, 600, 128, 64, 2, 0.0)])
 def test_als_prefill(ops, ws, oracle, dtype, hq, hkv, l, d, r, iters, tol):
     _say("als_prefill", dtype, hq, l, d, r, iters, tol)
     from lrqk_amd import synth
