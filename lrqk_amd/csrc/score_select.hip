@@ -395,13 +395,13 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
   constexpr int QV = R / 16;  // 16-byte vectors per 8-bit row
   const int64_t base0 = (int64_t)blockIdx.x * tiles_per_wg * kFiltRows;
   uint4 pre[kPre][QV];
-  float pre_s[kPre];
+  uint16_t pre_s[kPre];  // (as stored: converting here would wait for the loads before the query is resolved)
 #pragma unroll
   for (int it = 0; it < kPre; ++it) {
     const int64_t i = min(base0 + it * kFiltThreads + tid, m - 1);
 #pragma unroll
     for (int c = 0; c < QV; ++c) pre[it][c] = reinterpret_cast<const uint4*>(QA + i * R)[c];
-    pre_s[it] = sidx_scale_from_bits(QS[i]);
+    pre_s[it] = QS[i];
   }
   if (pending) {
     const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
@@ -527,7 +527,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
       const int64_t i = base + it * kFiltThreads + tid;
       float ub;
       if (tile == 0 && it < kPre) {
-        ub = bound_of(pre[it < kPre ? it : 0], pre_s[it < kPre ? it : 0]);
+        ub = bound_of(pre[it < kPre ? it : 0], sidx_scale_from_bits(pre_s[it < kPre ? it : 0]));
       } else {
         const int64_t ic = min(i, m - 1);
         uint4 row[QV];
