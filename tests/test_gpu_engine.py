@@ -471,6 +471,15 @@ def test_accuracy_focused_setting(lrqk, oracle):
     assert n > 0
 
 
+def test_wide_rank_through_the_prefix_branch(lrqk, oracle):
+    """Rank 40 with a prompt shorter than k + lite: twenty steps of the growing-prefix branch (the factor update over
+    a plain prefix of the rows, no ring append in its first kernel), then the main branch."""
+    _say("rank 40, prefix branch")
+    _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=128, l=300, r=40, k=256, L=64, steps=40,
+                        dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=80, capacity=512, tag="r40prefix")
+    assert n > 0
+
+
 @pytest.mark.parametrize("r", [40, 48])
 def test_ranks_between_the_tuned_ones(lrqk, oracle, r):
     """Ranks 40 and 48: the general factor-update kernels and the plain scan (the score index covers 16, 32, 64)."""
