@@ -76,6 +76,9 @@ def parse():
     p.add_argument("--rank", type=int, default=0, help="decode mode: r instead of the workload's")
     p.add_argument("--topk", type=int, default=0, help="decode mode: active tokens k instead of the workload's")
     p.add_argument("--lite", type=int, default=0, help="decode mode: recent-token window instead of the workload's")
+    p.add_argument("--data-rank", type=int, default=0,
+                   help="decode mode: rank of the synthetic queries / keys before noise instead of the workload's 32 "
+                        "(a factorisation of rank r on data of lower rank has directions that hold only noise)")
     p.add_argument("--seqs", type=int, default=0,
                    help="decode mode: sequences stepped together (the batch of the layer-step; 0 = the workload's "
                         "own, 1 for the 128K configuration); value stays the time of one layer-step of the whole batch")
@@ -344,6 +347,9 @@ def main():
         import dataclasses
         w = dataclasses.replace(w, r=a.rank or w.r, num_active_tokens=a.topk or w.num_active_tokens,
                                 lite_tokens=a.lite or w.lite_tokens)
+    if a.data_rank:
+        import dataclasses
+        w = dataclasses.replace(w, rho=a.data_rank)
     l = a.context or w.context
     t_setup = time.perf_counter()
     # synthetic prompt, drawn on the GPU (128K x 48 heads x 128 would take minutes on the host)
