@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # the same runs).  The summary of those runs is kept under profiles/.
 # Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
 # 8-bit copy (34 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
-MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (79786.8 * 2.000 + 866.5 * 1.000) * 1024,
+MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (78844.6 * 2.000 + 867.2 * 1.000) * 1024,
                           ("llama8b_128k_bf16", False): (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
 
 
