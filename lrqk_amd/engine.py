@@ -237,6 +237,13 @@ class LightAttentionIndicesFactory:
             rem = seq_len - k
             self.lite_len = rem
             self.lite_indices = list(range(k, k + rem)) + [-1] * (L - rem)
+            if rem == L:
+                # A prompt of exactly k + L tokens fills the ring.  The reference leaves lite_len = L here
+                # (lrqk_attention.py:1449-1452) and its next _append indexes slot L (:1188): an IndexError.  The
+                # full ring is flushed instead, which is the state the reference is in when the same tokens
+                # have arrived one by one (:1192-1196).
+                self.KVcpu.append(key_states.narrow(2, k, L), value_states.narrow(2, k, L))
+                self.lite_len = 0
             self.Kgpu.narrow(2, 0, seq_len).copy_(repeat_kv(key_states, g))
             self.Vgpu.narrow(2, 0, seq_len).copy_(repeat_kv(value_states, g))
             self._active_idx[:, :, :seq_len] = torch.arange(seq_len, dtype=torch.int32, device=dev)

@@ -94,7 +94,8 @@ def _check_prefill_products(oracle, tag, Q, K, g, A_Q0, A_K0, r, max_iter, tol, 
 
 def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter, tol, rho, cls=None, capacity=64,
               seed=0, fp_tol=None, no_hit_miss=False, sigma=0.01, compare_factors=True, attn_in_step=True,
-              gpu_draw=False, oracle_heads=None, tag=None, configure=None, attn_tol=None, compare_every=1):
+              gpu_draw=False, oracle_heads=None, tag=None, configure=None, attn_tol=None, compare_every=1,
+              after_oracle_prefill=None):
     """One seeded prefill + decode trace on the GPU engine and on the oracle.
 
     compare_factors   compare the engine's stored factors with an fp64 oracle prefill element by element
@@ -103,6 +104,8 @@ def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter
     attn_in_step      the fused step computes the attention; False takes the path of a reference-style
                       caller (the step returns K, V and the caller runs the attention itself)
     gpu_draw          draw the inputs on the GPU (long contexts; a host draw would take minutes)
+    after_oracle_prefill   called with the oracle layer after its prefill (a test that covers a state the
+                      reference cannot continue from puts the oracle into the equivalent one)
     """
     from lrqk_amd import synth, ops
     tag = tag or f"b{b}h{hq}l{l}r{r}k{k}"
@@ -166,6 +169,8 @@ def _lockstep(lrqk, oracle, *, b, hq, hkv, d, l, r, k, L, steps, dtype, max_iter
     A_Q_full = torch.zeros((b, hq, l, r), dtype=dtype)
     A_Q_full[:, :, -1:] = gA_Qrow
     orc.prefill(Q, K, V, als_result=(A_Q_full, gB_Q, gA_K, gB_K))
+    if after_oracle_prefill:
+        after_oracle_prefill(orc)
     del A_Q_full, Qd, Kd, Vd
     _compare_state(eng, orc, k, "prefill")
 
@@ -277,6 +282,26 @@ def test_edge_branch_then_main(lrqk, oracle):
               max_iter=(2, 2), tol=(1e-8, 1e-8), rho=3, capacity=8)
 
 
+def test_prompt_that_exactly_fills_the_ring(lrqk, oracle):
+    """l == k + L.  The reference's prefill leaves a full ring unflushed (lite_len = L, lrqk_attention.py:1449-1452)
+    and its first decode step then fails with an IndexError (:1188); the engine flushes the ring at the prefill
+    instead.  The oracle is put into that state by its own primitives -- the flush of _append, :1192-1196 -- and
+    the trace must then stay in lock step through the switch to selection."""
+    _say("prompt of exactly k + L tokens")
+
+    def flush_full_ring(orc):
+        assert orc.lite_len == orc.L
+        orc._kv_append(orc._lite(orc.Kgpu), orc._lite(orc.Vgpu))
+        orc.lite_len = 0
+
+    for kw in (dict(b=1, hq=4, hkv=2, d=16, l=36, r=4, k=33, L=3, dtype=torch.float32, rho=8),
+               dict(b=2, hq=2, hkv=1, d=32, l=17, r=8, k=16, L=1, dtype=torch.bfloat16, rho=16),
+               dict(b=1, hq=8, hkv=2, d=64, l=258, r=16, k=256, L=2, dtype=torch.bfloat16, rho=24)):
+        _, _, n = _lockstep(lrqk, oracle, steps=24, max_iter=(2, 2), tol=(1e-8, 1e-8), capacity=8,
+                            compare_factors=False, after_oracle_prefill=flush_full_ring, **kw)
+        assert n > 0
+
+
 def test_staged_fetch_trace(lrqk, oracle):
     """The same lock-step trace with the misses moved by host gather + hipMemcpyAsync on the side
     stream (buffer growth included: the pinned store is reallocated during the run)."""
@@ -384,6 +409,65 @@ def _OffloadProbe(lrqk):
             assert self.Kgpu is None and self._A_K.data is None      # parked
             self._restore(q.device)
     return Probe
+
+
+def _random_trace_config(lrqk, i):
+    """Configuration ``i`` of the seeded family that test_random_small_traces runs."""
+    import random
+    rng = random.Random(7000 + i)
+    dtype = rng.choice([torch.float32, torch.bfloat16])
+    d = rng.choice([8, 16, 32, 64, 128] if dtype == torch.float32 else [16, 32, 64, 128])
+    hkv, g, b = rng.choice([1, 2, 4]), rng.choice([1, 2, 4]), rng.choice([1, 1, 2])
+    r = min(rng.choice([2, 3, 4, 5, 8, 12, 16, 16, 24, 32, 32]), d // 2)
+    if dtype == torch.bfloat16:
+        r = max(8, r // 8 * 8)          # 16-byte rows of A_K
+    k = rng.choice([4, 7, 16, 33, 64, 100, 128, 256, 300, 512, 1000])
+    L = rng.choice([1, 2, 3, 4, 8, 16])
+    kind = rng.random()
+    if kind < 0.15:
+        l = rng.randint(k, k + L)                      # growing-prefix branch first (k + L itself included)
+    elif kind < 0.3:
+        l = rng.randint(k + L + 1, k + L + 8)          # a handful of candidates beyond k
+    else:
+        l = rng.randint(k + L + 1, 2500 if rng.random() < 0.85 else 12000)
+    tol = rng.choice([(1e-8, 1e-8), (1e-2, 1e-2), (1e-4, 1e-3)])
+    variant = rng.choice(["plain"] * 5 + ["offload", "no_hit_miss", "staged"])
+    index_on, victim = rng.random() < 0.75, rng.choice([None, None, 0, 8, 32, 96])
+    cfg = dict(b=b, hq=hkv * g, hkv=hkv, d=d, l=l, r=r, k=k, L=L, steps=rng.choice([12, 24, 40]), dtype=dtype,
+               max_iter=rng.choice([(1, 1), (2, 2), (2, 4), (2, 8), (4, 4)]), tol=tol,
+               rho=min(r + rng.choice([4, 8, 16]), d), capacity=rng.choice([8, 64, 1024]), seed=i,
+               compare_factors=False, attn_in_step=rng.random() < 0.8,
+               # what is under test here are the integer stages (compared bit for bit whatever this limit is): with
+               # a loose stopping tolerance the two sides may stop one iteration apart, and the factor outputs of a
+               # random, small, badly conditioned trace scatter around the floors that the fixed traces hold
+               fp_tol=2e-2 if tol[0] > 1e-6 else 5e-3)
+    if variant == "offload":
+        cfg["cls"] = _OffloadProbe(lrqk)
+    elif variant == "no_hit_miss":
+        cfg["cls"], cfg["no_hit_miss"] = lrqk.LightAttentionIndicesNoHitMiss, True
+
+    def configure(e):
+        e.use_score_index, e.victim_rows = index_on, victim
+        if variant == "staged":
+            e.fetch_mode = "staged"
+    cfg["configure"] = configure
+    if l == k + L:
+        def flush_full_ring(orc):
+            orc._kv_append(orc._lite(orc.Kgpu), orc._lite(orc.Vgpu))
+            orc.lite_len = 0
+        cfg["after_oracle_prefill"] = flush_full_ring
+    return cfg, f"{variant} index={index_on} victim={victim}"
+
+
+def test_random_small_traces(lrqk, oracle):
+    """64 seeded random configurations (head counts and widths, ranks, k from 4 to 1000, rings of 1 to 16 tokens,
+    prompts from exactly k tokens to 12000, every engine variant, score index and victim cache on and off, buffer
+    capacities that force growth): ids, evicted slots, refetched rows, ring and host store bit for bit against the
+    oracle at every step, as in the fixed traces."""
+    for i in range(64):
+        cfg, what = _random_trace_config(lrqk, i)
+        _say("random trace", i, what, {k: v for k, v in cfg.items() if not callable(v)})
+        _lockstep(lrqk, oracle, tag=f"random{i}", **cfg)
 
 
 def test_overridden_stage_is_used(lrqk, oracle):
