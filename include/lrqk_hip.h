@@ -93,7 +93,7 @@ int lrqk_diff(const int32_t* new_idx, int64_t new_stride, int32_t* hit, int64_t 
               uint8_t* evict, int32_t* miss_slots, int32_t* miss_count, void* stream);
 
 /* py:1235-1273 + py:1275-1315 in one pass -- lrqk_score_select followed by lrqk_diff, with the
- * diff done by the select kernel while the selection is still on chip (m > topk required).
+ * diff done by the select kernel while the selection is still on chip (m >= topk required; with m == topk every row is selected).
  * new_idx: [bh][topk] receives the ascending selection; hit / evict / miss_slots / miss_count
  * as in lrqk_diff (evict may be NULL).  new_idx may be NULL: the caller then only gets what
  * changes (hit, evict, miss_slots, miss_count), and the selection is never put in order -- the

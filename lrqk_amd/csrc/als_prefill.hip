@@ -799,7 +799,6 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
         typedef short v4s __attribute__((ext_vector_type(4)));
         typedef v4s __attribute__((address_space(3))) * lds_v4s;
         const int s16 = lane & 15;
-<<<<<<< Updated upstream
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
           const uint16_t* p = &x_s[(16 * kb + 4 * half + (s16 >> 2)) * LDB + 32 * nb + (col & 16) + 4 * (s16 & 3)];
@@ -810,18 +809,6 @@ __global__ __launch_bounds__(NW * kWave) void pf_pass_bf16_kernel(const bf16_t* 
       } else {
         floatx16 xa;
 #pragma unroll
-=======
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          const uint16_t* p = &x_s[(16 * kb + 4 * half + (s16 >> 2)) * LDB + 32 * nb + (col & 16) + 4 * (s16 & 3)];
-          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)p);
-          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(p + 8 * LDB));
-          xb[kb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        }
-      } else {
-        floatx16 xa;
-#pragma unroll
->>>>>>> Stashed changes
         for (int v = 0; v < 16; ++v) xa[v] = 0.0f;
         xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb), ident[0], xa, 0, 0, 0);
         xa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_op(2 * nb + 1), ident[1], xa, 0, 0, 0);
@@ -1123,7 +1110,6 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   const dim3 grid((unsigned)S, (unsigned)bh), blk((unsigned)pass_threads), sblk(small32 ? kPfSmallThreads : kPfThreads);
   const T* Q = (const T*)q;
   const T* K = (const T*)k;
-<<<<<<< Updated upstream
   // bf16 rows of 128 elements: every iteration on the d x d Gram matrices (fp64), then one pass per side that
   // applies the last Mq, Mk; the Q side's sums over the given factors are formed together with Q^T Q (one
   // reading of Q), the K side's by the pass below (A_K has a head per query head, K per kv head)
@@ -1147,21 +1133,6 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
                        (float*)nullptr, (const int*)nullptr, S);
     LRQK_HIP_CHECK(hipGetLastError());
   }
-=======
-  PfPassFn<T> first = pass;  // the sums over the given initial factors
-  if constexpr (sizeof(T) == 2) {
-    if (mfma && d == 128) {
-      first = (PfPassFn<T>)pf_pass_bf16_kernel<4, 8, true, true>;
-      if (smem_pass > 48 * 1024)
-        LRQK_HIP_CHECK(hipFuncSetAttribute((const void*)first, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pass));
-    }
-  }
-  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, Q, hq, hq, l, r, d, (const float*)nullptr, a_q, partQ,
-                     (float*)nullptr, (const int*)nullptr, S);
-  hipLaunchKernelGGL(first, grid, blk, smem_pass, st, K, hkv, hq, l, r, d, (const float*)nullptr, a_k, partK,
-                     (float*)nullptr, (const int*)nullptr, S);
-  LRQK_HIP_CHECK(hipGetLastError());
->>>>>>> Stashed changes
   if constexpr (sizeof(T) == 2) {
     if (gram_domain) {
       float *mt_q = nullptr, *mt_k = nullptr;

@@ -50,15 +50,9 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
   const bf16_t* Xh = X + (int64_t)xh * l * kXtxD;
   const int nb1 = wave >> 1, nb2 = 2 * (wave & 1);
   constexpr int NL = kXtxRows * kXtxD / (kXtxThreads * 8);  // 16-byte loads per thread and step
-<<<<<<< Updated upstream
   // One step ahead is all that pays: with two steps of rows in flight per workgroup the kernel is slower
   // (65 against 54 us at 32 heads x 32K rows).
   uint4 pre_a[NL];
-=======
-  // two steps of rows are on their way while one is multiplied: a step is 32 KB per workgroup, and the memory
-  // system wants ~30 MB in flight over the GPU
-  uint4 pre[NL], pre2[NL];
->>>>>>> Stashed changes
   auto issue = [&](int64_t t0, uint4 (&dst)[NL]) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
@@ -70,7 +64,6 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
   gd_floatx16 acc0, acc1;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
-<<<<<<< Updated upstream
   // An operand of the 32x32x16 product, lane (col, half): rows row0 + 8 half .. + 7 of column 32 nb + col.  The
   // transposing LDS read hands a lane four successive rows of its column: within 16 lanes, lane s points at
   // row s / 4, columns 4 (s % 4) .. + 3, and lane t receives column t of the four rows.
@@ -87,11 +80,6 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
   const int64_t stride = (int64_t)S * kXtxRows;
   // one step: stage `cur` (the rows from t0 on), ask for the next step into `cur`, multiply
   auto step = [&](int64_t t0, uint4 (&cur)[NL]) {
-=======
-  if (r0 < r1) issue(r0, pre);
-  if (r0 + kXtxRows < r1) issue(r0 + kXtxRows, pre2);
-  for (int64_t t0 = r0; t0 < r1; t0 += kXtxRows) {
->>>>>>> Stashed changes
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       const int e = (i * kXtxThreads + tid) * 8;
@@ -99,27 +87,8 @@ __global__ __launch_bounds__(kXtxThreads) void pf_xtx_kernel(const bf16_t* __res
       *reinterpret_cast<uint4*>(&x_s[row * kXtxLd + e % kXtxD]) = t0 + row < l ? cur[i] : make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
-<<<<<<< Updated upstream
     if (t0 + stride < l) issue(t0 + stride, cur);
     const int tiles = (int)min((int64_t)4, (l - t0 + 31) / 32);
-=======
-#pragma unroll
-    for (int i = 0; i < NL; ++i) pre[i] = pre2[i];
-    if (t0 + 2 * kXtxRows < r1) issue(t0 + 2 * kXtxRows, pre2);
-    const int tiles = (int)min((int64_t)4, (r1 - t0 + 31) / 32);
-    // An operand of the 32x32x16 product, lane (col, half): rows row0 + 8 half .. + 7 of column 32 nb + col.  The
-    // transposing LDS read hands a lane four successive rows of its column: within 16 lanes, lane s points at
-    // row s / 4, columns 4 (s % 4) .. + 3, and lane t receives column t of the four rows.
-    auto operand = [&](int row0, int nb) {
-      const int s16 = lane & 15;
-      const uint16_t* p = &x_s[(row0 + 8 * half + (s16 >> 2)) * kXtxLd + 32 * nb + (col & 16) + 4 * (s16 & 3)];
-      typedef short gd_v4s __attribute__((ext_vector_type(4)));
-      typedef gd_v4s __attribute__((address_space(3))) * gd_lds_v4s;
-      const gd_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)p);
-      const gd_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gd_lds_v4s)(p + 4 * kXtxLd));
-      return __builtin_bit_cast(gd_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    };
->>>>>>> Stashed changes
     for (int tile = 0; tile < tiles; ++tile) {
       gd_floatx16 t0a, t1a;
 #pragma unroll

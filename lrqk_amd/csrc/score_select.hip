@@ -1773,7 +1773,8 @@ extern "C" int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t he
   }
   LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
   LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_EINVAL, "r=%d", r);
-  LRQK_REQUIRE(m > topk, LRQK_EINVAL, "m=%lld must exceed topk=%d (no diff happens in the prefix branch)",
+  // (m == topk is the first step after the growing-prefix branch, py:1560-1562: every row is selected)
+  LRQK_REQUIRE(m >= topk, LRQK_EINVAL, "m=%lld is below topk=%d (no diff happens in the prefix branch)",
                (long long)m, topk);
   LRQK_REQUIRE(head_stride >= m * r && hit_stride >= topk, LRQK_EINVAL, "stride too small");
   int rc = score_select_diff(ctx, a_k, head_stride, q_hat, bh, m, r, topk, dtype, round_bf16, new_idx, hit, hit_stride,

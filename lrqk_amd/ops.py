@@ -160,12 +160,12 @@ def score_select(ws: Workspace, a_k: torch.Tensor, q_hat: torch.Tensor, m: int, 
 
 def score_select_diff(ws: Workspace, a_k: torch.Tensor, q_hat: torch.Tensor, m: int, topk: int, hit: torch.Tensor,
                       round_to_storage: bool = True, want_new: bool = True):
-    """score_select + diff in one pass (m > topk).  hit int32 [b,H,>=topk] is updated in place.
+    """score_select + diff in one pass (m >= topk).  hit int32 [b,H,>=topk] is updated in place.
     Returns (new_idx int32 [b,H,topk], evict u8 [b,H,topk], miss_slots int32 [b,H,topk], miss_count int32 [b,H]).
     want_new=False: only what changes is produced (new_idx is None), as inside the decode step."""
     _need_cuda(a_k, q_hat, hit)
     b, H, cap, r = a_k.shape
-    assert a_k.is_contiguous() and hit.is_contiguous() and hit.dtype == torch.int32 and topk < m <= cap
+    assert a_k.is_contiguous() and hit.is_contiguous() and hit.dtype == torch.int32 and topk <= m <= cap
     qh = q_hat.reshape(b * H, r).contiguous()
     dev = a_k.device
     new = torch.empty((b, H, topk), dtype=torch.int32, device=dev) if want_new else None

@@ -282,10 +282,12 @@ def _check_diff(ops, oracle, now, new):
 @pytest.mark.parametrize("m,cap,k,H,dtype", [(5000, 5008, 512, 3, torch.float32), (40000, 40000, 2048, 2, torch.bfloat16),
                                              (300000, 300032, 2048, 2, torch.bfloat16),
                                              (270000, 270000, 4096, 1, torch.bfloat16),
-                                             (20000, 20000, 4100, 1, torch.float32)])
+                                             (20000, 20000, 4100, 1, torch.float32),
+                                             (2048, 2056, 2048, 2, torch.bfloat16), (7, 16, 7, 3, torch.float32)])
 def test_score_select_diff_fused(ops, oracle, m, cap, k, H, dtype):
     """Selection and hit/miss diff in one pass against the oracle's two stages: one bitmap chunk
-    (m <= 262144), several chunks, the largest fused k, and a k beyond it (separate diff launch).
+    (m <= 262144), several chunks, the largest fused k, a k beyond it (separate diff launch), and m == k (the first
+    step after the growing-prefix branch: every row is selected).
     Second round on the same workspace goes through the filtered path."""
     _say("score_select_diff", m, k, H, dtype)
     ws = ops.Workspace()
