@@ -748,6 +748,48 @@ def test_als_prefill_benchmark_configuration(ops, ws, oracle):
     assert abs(res_g - res_o) < 1e-4 and abs(resq_g - resq_o) < 1e-4
 
 
+def test_random_kernel_shapes(ops, ws, oracle):
+    """160 seeded random shapes through the checks above (factor update incl. the general-rank kernels, attention,
+    hit/miss diff, selection with tied and quantised scores): sizes next to the powers of two and split boundaries
+    that the fixed cases are built around, not on them."""
+    import random
+    for i in range(160):
+        rng = random.Random(4200 + i)
+        kind = rng.choice(["als", "als", "attention", "diff", "select"])
+        dtype = rng.choice([torch.float32, torch.bfloat16])
+        if kind == "als":
+            d = rng.choice([8, 16, 32, 64, 128, 256] if dtype == torch.float32 else [16, 32, 64, 128, 256])
+            hkv = rng.choice([1, 2, 3])
+            r = min(rng.choice([2, 3, 4, 8, 16, 24, 32, 33, 40, 48, 64]), d // 2)
+            if dtype == torch.bfloat16:
+                r = max(8, r // 8 * 8)                       # 16-byte rows of A_K
+            if r > 32 and d == 256:
+                r = 32                                       # (refused: ranks above 32 take rows of at most 128 elements)
+            n = max(rng.choice([r + 1, 2 * r + 3, 70, 129, 300, 544, 1000, 2112, 3000, 4160]), r + 1)
+            max_iter, tol = rng.choice([(1, 0.0), (2, 0.0), (3, 1e30), (4, 1e-6), (8, 1e-8)])
+            _check_als_decode(ops, ws, oracle, dtype, hkv * rng.choice([1, 2, 4]), hkv, n, d, r, max_iter, tol)
+        elif kind == "attention":
+            d = rng.choice([8, 16, 32, 64, 128, 256] if dtype == torch.float32 else [16, 32, 64, 128, 256])
+            test_attention(ops, ws, oracle, dtype, d,
+                           rng.choice([1, 2, 12, 63, 64, 65, 100, 255, 256, 257, 544, 1000, 2112, 4224, 9000]))
+        elif kind == "diff":
+            k = rng.choice([1, 2, 8, 100, 512, 1000, 2048, 2500, 4096, 5000, 8192])
+            test_diff_random(ops, oracle, k, k + rng.choice([1, 5, k, 10 * k]))
+        else:
+            m = rng.choice([9, 100, 1000, 5000, 40000, 70000])
+            k = rng.choice([1, 8, 64, 512, 2048, 4096, 8192])
+            g = torch.Generator().manual_seed(i)
+            s = torch.randn((2, 3, m), generator=g)
+            mode = rng.choice(["plain", "few values", "bf16 values"])
+            s = (s * 2).round() / 2 if mode == "few values" else (s.bfloat16().float() if mode == "bf16 values" else s)
+            _say("select", m, k, mode)
+            if m <= k:
+                got = ops.select_from_scores(ws, s.to(DEV), k).cpu()
+                assert torch.equal(got, torch.arange(m, dtype=torch.int32).expand(2, 3, m))
+            else:
+                _check_select(ops, ws, oracle, s, k)
+
+
 def test_measurement_probes(ops):
     """The plain read / copy kernels and the event-pair calibration that the bench line carries: the copy
     really copies, the rates and the bracket are finite and of a plausible order of magnitude."""
