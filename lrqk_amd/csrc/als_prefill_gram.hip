@@ -439,8 +439,9 @@ constexpr int kGdLg = 33;         // doubles per row of an r x r matrix in LDS
 // 16 rt + l / 16 + 4 v, column 16 u + l % 16 of tile (rt, u)): each of the four waves holds W itself (every wave
 // eliminates its own copy: no wave waits for another, the solve has no barrier) and 32 columns of RHS.
 // Step m, with P the pivot columns 4 m .. 4 m + 3 (32 x 4) and D its rows 4 m .. 4 m + 3:
-//     X <- X - ((P - E) D^-1) X[4 m .. 4 m + 3, :]        (E: the identity in the pivot rows)
-// which leaves D^-1 X[pivot rows] in the pivot rows and clears the pivot columns elsewhere.  The right-hand
+//     X <- X - (P D^-1) X[4 m .. 4 m + 3, :] outside the pivot rows,   X[pivot rows] <- D^-1 X[pivot rows]
+// (one product: the pivot rows' accumulators are cleared and their left operand is D^-1 itself), which clears the
+// pivot columns elsewhere.  The right-hand
 // operand, four rows of X, is element m % 4 of the lane's own tile in row tile m / 4: no data moves for it.  The
 // left operand needs P by rows: the lanes that hold the pivot columns put them into the wave's own LDS slot, the
 // two pivot blocks are inverted side by side in the two halves of the wave (by 2 x 2 blocks, no pivoting) and
@@ -551,9 +552,12 @@ __device__ __forceinline__ void gd_solve_pair(GdSys (&s)[2], double* __restrict_
         const int row = 16 * rt + li;
         const double2 lo = *reinterpret_cast<const double2*>(&P[row * 4]);
         const double2 hi = *reinterpret_cast<const double2*>(&P[row * 4 + 2]);
-        const double m0 = lo.x - (row == 4 * m ? 1.0 : 0.0), m1 = lo.y - (row == 4 * m + 1 ? 1.0 : 0.0);
-        const double m2 = hi.x - (row == 4 * m + 2 ? 1.0 : 0.0), m3 = hi.y - (row == 4 * m + 3 ? 1.0 : 0.0);
-        aop[sy][rt] = -fma(m0, ic[0], fma(m1, ic[1], fma(m2, ic[2], m3 * ic[3])));
+        // pivot rows: the rows of D^-1 themselves (their accumulators are cleared below, so they come out as
+        // D^-1 X and not as X - (I - D^-1) X, which cancels in its leading digits when D is far from unit size:
+        // with a diagonal of 1e12 solutions were off by 5e-3 where the conditioning allowed 1e-11)
+        const double own = xch[sy * 16 + (row & 3) * 4 + lk];
+        const double oth = -fma(lo.x, ic[0], fma(lo.y, ic[1], fma(hi.x, ic[2], hi.y * ic[3])));
+        aop[sy][rt] = (row >> 2) == m ? own : oth;
       }
     }
     gd_wave_sync();  // (the reads of the slot precede the next step's writes)
@@ -564,6 +568,7 @@ __device__ __forceinline__ void gd_solve_pair(GdSys (&s)[2], double* __restrict_
       for (int u = 0; u < 2; ++u) {
         if (u < tp) continue;
         const double bop = s[sy].w[tp][u][vp];
+        s[sy].w[tp][u][vp] = 0.0;
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt)
           s[sy].w[rt][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(aop[sy][rt], bop, s[sy].w[rt][u], 0, 0, 0);
@@ -573,6 +578,7 @@ __device__ __forceinline__ void gd_solve_pair(GdSys (&s)[2], double* __restrict_
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const double bop = s[sy].x[tp][u][vp];
+        s[sy].x[tp][u][vp] = 0.0;
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt)
           s[sy].x[rt][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(aop[sy][rt], bop, s[sy].x[rt][u], 0, 0, 0);
