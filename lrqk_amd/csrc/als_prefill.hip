@@ -179,9 +179,15 @@ __device__ __forceinline__ void solve_multi(float* Mx, int ldm, int r, int nrhs)
 
 __device__ __forceinline__ void reduce_part(const float* part, int S, int ne, float* dst) {
   for (int e = threadIdx.x; e < ne; e += kPfThreads) {
+    // (more than 16 partial sums -- long prompts -- are added in fp64)
     float v = 0.0f;
-    for (int s = 0; s < S; ++s) v += part[(int64_t)s * ne + e];
-    dst[e] = v;
+    double w = 0.0;
+    for (int s = 0; s < S; ++s) {
+      const float x = part[(int64_t)s * ne + e];
+      v += x;
+      w += (double)x;
+    }
+    dst[e] = S > 16 ? (float)w : v;
   }
 }
 
@@ -237,8 +243,13 @@ __global__ __launch_bounds__(kPfThreads) void pf_small_generic_kernel(int stage,
   // sum over the splits of element e of a head's packed [G | C] block, in split order
   auto summed = [&](const float* part, int e) {
     float v = 0.0f;
-    for (int s = 0; s < S; ++s) v += part[(int64_t)s * ne + e];
-    return v;
+    double w = 0.0;
+    for (int s = 0; s < S; ++s) {
+      const float x = part[(int64_t)s * ne + e];
+      v += x;
+      w += (double)x;
+    }
+    return S > 16 ? (float)w : v;
   };
   if (stage == 0 || stage == 2) {
     reduce_part(pk, S, ne, G2);
@@ -905,8 +916,12 @@ __device__ __forceinline__ void pf_reduce_part(const float* __restrict__ part, i
   constexpr int EB = 16;
   for (int e0 = threadIdx.x; e0 < ne; e0 += EB * kPfSmallThreads) {
     float v[EB];
+    double w[EB];  // (more than 16 partial sums -- long prompts -- are added in fp64)
 #pragma unroll
-    for (int q = 0; q < EB; ++q) v[q] = 0.0f;
+    for (int q = 0; q < EB; ++q) {
+      v[q] = 0.0f;
+      w[q] = 0.0;
+    }
     for (int s0 = 0; s0 < S; s0 += 8) {
       float x[EB][8];
 #pragma unroll
@@ -918,11 +933,14 @@ __device__ __forceinline__ void pf_reduce_part(const float* __restrict__ part, i
       for (int q = 0; q < EB; ++q)
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-          if (s0 + u < S) v[q] += x[q][u];
+          if (s0 + u < S) {
+            v[q] += x[q][u];
+            w[q] += (double)x[q][u];
+          }
     }
 #pragma unroll
     for (int q = 0; q < EB; ++q)
-      if (e0 + q * kPfSmallThreads < ne) dst[e0 + q * kPfSmallThreads] = v[q];
+      if (e0 + q * kPfSmallThreads < ne) dst[e0 + q * kPfSmallThreads] = S > 16 ? (float)w[q] : v[q];
   }
 }
 
@@ -1067,6 +1085,11 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   // splits of the long axis: about one workgroup per CU (a pass keeps one wave per SIMD busy), but
   // at least 128 rows per split
   int S = std::max(1, std::min(64, 256 / bh));
+  // The row-by-row formulation solves its r x r systems from these sums in fp32, and a split adds its rows up in
+  // fp32: at most 2048 rows per split there (the partial sums are added in fp64), however few splits fill the GPU.
+  // (The iteration on Gram matrices takes only its first sums from here, where the systems are well conditioned.)
+  const bool gram_path = sizeof(T) == 2 && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
+  if (!gram_path) S = (int)std::min<int64_t>(64, std::max<int64_t>(S, (l + 2047) / 2048));
   S = (int)std::max<int64_t>(1, std::min<int64_t>(S, (l + 127) / 128));
   const int iters = max_iter > 0 ? max_iter : 0;
   // workspace: partQ, partK, Mt, deltas[iters][2][bh][S], flags[iters+1]
