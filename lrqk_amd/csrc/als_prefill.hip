@@ -1088,8 +1088,10 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   // The row-by-row formulation solves its r x r systems from these sums in fp32, and a split adds its rows up in
   // fp32: at most 2048 rows per split there (the partial sums are added in fp64), however few splits fill the GPU.
   // (The iteration on Gram matrices takes only its first sums from here, where the systems are well conditioned.)
-  const bool gram_path = sizeof(T) == 2 && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
-  if (!gram_path) S = (int)std::min<int64_t>(64, std::max<int64_t>(S, (l + 2047) / 2048));
+  // (At most 64 splits per head: beyond 128K rows a split of the row-by-row formulation adds up l / 64 rows.)
+  // bf16 rows of 128 elements, 16-byte aligned: every iteration runs on the d x d Gram matrices (fp64)
+  const bool gram_domain = sizeof(T) == 2 && mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
+  if (!gram_domain) S = (int)std::min<int64_t>(64, std::max<int64_t>(S, (l + 2047) / 2048));
   S = (int)std::max<int64_t>(1, std::min<int64_t>(S, (l + 127) / 128));
   const int iters = max_iter > 0 ? max_iter : 0;
   // workspace: partQ, partK, Mt, deltas[iters][2][bh][S], flags[iters+1]
@@ -1136,7 +1138,6 @@ static int prefill_impl(lrqk_ctx* ctx, const void* q, const void* k, float* a_q,
   // bf16 rows of 128 elements: every iteration on the d x d Gram matrices (fp64), then one pass per side that
   // applies the last Mq, Mk; the Q side's sums over the given factors are formed together with Q^T Q (one
   // reading of Q), the K side's by the pass below (A_K has a head per query head, K per kv head)
-  const bool gram_domain = sizeof(T) == 2 && mfma && d == 128 && r <= 32 && !getenv("LRQK_PREFILL_ROWWISE");
   const bool fused_sums = gram_domain && !getenv("LRQK_PREFILL_SEPARATE_SUMS");  // (the Q side's, with Q^T Q)
   // (the iteration on Gram matrices writes every stopping flag before it reads it)
   if (!gram_domain) LRQK_HIP_CHECK(hipMemsetAsync(flags, 0, (size_t)(iters + 1) * sizeof(int), st));

@@ -1765,14 +1765,16 @@ extern "C" int lrqk_score_select_diff(lrqk_ctx* ctx, const void* a_k, int64_t he
                                       int32_t* hit, int64_t hit_stride, uint8_t* evict, int32_t* miss_slots,
                                       int32_t* miss_count, void* stream) {
   LRQK_REQUIRE(ctx && a_k && q_hat && hit && miss_slots && miss_count, LRQK_EINVAL, "null pointer");
+  LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
+  LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_EINVAL, "r=%d", r);
+  LRQK_REQUIRE(bh > 0 && bh <= 65535, LRQK_EINVAL, "bh=%d out of range", bh);
+  LRQK_REQUIRE(topk > 0 && topk <= LRQK_MAX_TOPK, LRQK_ELIMIT, "topk=%d not in 1..%d", topk, LRQK_MAX_TOPK);
   const bool want_new = new_idx != nullptr;
   if (!want_new) {  // the caller only wants what changes: the selection is never put in order
     int rce = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t));
     if (rce) return rce;
     new_idx = (int32_t*)ctx->new_idx.p;
   }
-  LRQK_REQUIRE(dtype == LRQK_F32 || dtype == LRQK_BF16, LRQK_EINVAL, "dtype=%d", dtype);
-  LRQK_REQUIRE(r > 0 && r <= LRQK_MAX_R, LRQK_EINVAL, "r=%d", r);
   // (m == topk is the first step after the growing-prefix branch, py:1560-1562: every row is selected)
   LRQK_REQUIRE(m >= topk, LRQK_EINVAL, "m=%lld is below topk=%d (no diff happens in the prefix branch)",
                (long long)m, topk);
@@ -1819,6 +1821,9 @@ extern "C" int lrqk_scan_stats(lrqk_ctx* ctx, int64_t* rows_scanned, int64_t* ro
   *rows_scanned = *rows_rescored = 0;
   if (!ctx->cand_cnt.p || ctx->sel_bh <= 0 || ctx->scan_wgs <= 0) return LRQK_OK;
   std::vector<int> v((size_t)ctx->scan_wgs);
+  // the counters belong to the last scan, which may still be running on a stream that does not wait for the
+  // null stream's copy
+  LRQK_HIP_CHECK(hipDeviceSynchronize());
   LRQK_HIP_CHECK(hipMemcpy(v.data(), (int*)ctx->cand_cnt.p + 6 * ctx->sel_bh + 3, v.size() * sizeof(int),
                            hipMemcpyDeviceToHost));
   int64_t t = 0;
@@ -1834,6 +1839,7 @@ extern "C" int lrqk_select_stats(lrqk_ctx* ctx, int* fast_heads, int* full_heads
   if (!ctx->cand_cnt.p || ctx->sel_bh <= 0) return LRQK_OK;
   int* stats = (int*)ctx->cand_cnt.p + 6 * ctx->sel_bh;
   int v[3];
+  LRQK_HIP_CHECK(hipDeviceSynchronize());
   LRQK_HIP_CHECK(hipMemcpy(v, stats, sizeof(v), hipMemcpyDeviceToHost));
   *fast_heads = v[0];
   *full_heads = v[1] + v[2];
