@@ -59,6 +59,9 @@ def parse():
                    help="miss fetch: the kernel reads the pinned store itself, or host gather + hipMemcpyAsync")
     p.add_argument("--no-score-index", action="store_true",
                    help="scan the bf16 A_K rows directly instead of their 8-bit score index")
+    p.add_argument("--factor-state", action="store_true",
+                   help="run every step's factor update in fp64 from the state kept between steps instead of over the "
+                        "active rows in fp32 (adds a launch per step that brings the state up to date)")
     p.add_argument("--victim-rows", type=int, default=-1,
                    help="rows per head of the device-side cache of evicted K/V rows (-1: 4 k, 0: off)")
     p.add_argument("--mode", default="decode", choices=["decode", "prefill_als", "decoder"],
@@ -363,6 +366,7 @@ def main():
         e_.attn_in_step = not a.no_attn
         e_.fetch_mode = a.fetch
         e_.use_score_index = not a.no_score_index
+        e_.use_factor_state = a.factor_state
         if a.victim_rows >= 0:
             e_.victim_rows = a.victim_rows
         return e_

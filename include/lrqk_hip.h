@@ -154,6 +154,26 @@ int lrqk_ctx_victim_cache(lrqk_ctx* ctx, int rows_per_head);
  * rows came from the victim cache).  Synchronises.  Counts only while the victim cache is on. */
 int lrqk_victim_stats(lrqk_ctx* ctx, int64_t* host_rows, int reset);
 
+/* Kept state of the factor update inside lrqk_decode_step (no counterpart in the reference; a new ctx has it
+ * off).  In py:555-609 everything but a few products with the step's q and k -- B_Q B_Q^T + A^T A, B_K B_K^T, their
+ * inverses and K__^T A over the active slots -- depends only on what the previous step left, because the new
+ * token's A_K row is zero while its update runs (py:888, 1560).  The ctx keeps those per head in fp64 and brings
+ * them up to date after each step's fetch from the rows that the step replaced (one more launch at the end of the
+ * step), so a step's update is one small launch in fp64: its iterates agree with an fp64 evaluation of py:555-609
+ * to rounding, where the update over the active rows in fp32 is cond(G) * 2^-24 away (ranks <= 32, head widths 32,
+ * 64, 128 or 256, at most 8 iterations; other shapes and every other entry point run the update over the active
+ * rows in fp32).  The state describes the buffers that
+ * the last lrqk_decode_step call was given, as its next call will find them: call this (any value) after changing
+ * B_Q, B_K, the active ids, A_K rows or K rows of the active set in any other way, and the next step forms the
+ * state from scratch.  0 switches the kept state off. */
+int lrqk_ctx_factor_state(lrqk_ctx* ctx, int enable);
+/* The iterates of the last lrqk_decode_step that ran from kept state, in fp64 as computed (before they are
+ * rounded): out [bh][max_iter][2 r] = (q_hat, k_hat) of every iteration.  bh, max_iter, r receive the sizes and
+ * token the id of the token whose step it was (-1: none yet); out may be NULL to ask for them.  Synchronises.
+ * Test hook; no counterpart in the reference. */
+int lrqk_last_iterates(lrqk_ctx* ctx, double* out, int64_t n_doubles, int* bh, int* max_iter, int* r,
+                       int64_t* token);
+
 /* py:1339-1351 fetch_by_hit (same-device branch) -- k_act[bh][j][:] = src[b][h/groups][idx[bh][j]][:]
  * for j < count, src: [b][hkv][src_len][d] on the device. */
 int lrqk_gather_rows(const void* src, int64_t src_len, const int32_t* idx, int64_t idx_stride, int count,
@@ -182,7 +202,8 @@ int lrqk_attention(lrqk_ctx* ctx, const void* q, const void* k_act, const void* 
  * Limit: bh * min(64, ceil(n_valid / 64)) * (d + 2) <= 1048576, else LRQK_ELIMIT.  All calls on one
  * GPU share that block: calls that overlap on one GPU (different streams or threads) race; calls on
  * one stream are ordered.  The block needs no clearing between calls (every entry that is read was
- * written by the same call). */
+ * written by the same call).  The first call on a device looks up the block's address (and lets the
+ * runtime load the kernels): make it outside a graph capture. */
 int lrqk_attention_static(const void* q, const void* k_act, const void* v_act, int n_slots, int n_valid,
                           void* out, int bh, int d, int dtype, void* stream);
 

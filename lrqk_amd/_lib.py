@@ -55,6 +55,8 @@ def _sig(lib):
         "lrqk_ctx_score_index": ([vp, i32], i32),
         "lrqk_ctx_victim_cache": ([vp, i32], i32),
         "lrqk_victim_stats": ([vp, c.POINTER(c.c_int64), i32], i32),
+        "lrqk_ctx_factor_state": ([vp, i32], i32),
+        "lrqk_last_iterates": ([vp, vp, i64, c.POINTER(i32), c.POINTER(i32), c.POINTER(i32), c.POINTER(i64)], i32),
         "lrqk_gather_rows": ([vp, i64, vp, i64, i32, vp, i32, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_append_token": ([vp, vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, i32, i32, i32, vp], i32),
         "lrqk_flush_ring": ([vp, vp, i32, i32, i32, vp, i64, i64, i32, i32, i32, i32, i32, vp], i32),

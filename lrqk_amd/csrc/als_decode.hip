@@ -1182,6 +1182,19 @@ int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t he
                             hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, defer_finish, dtype, st);
 }
 
+int als_defer_finish(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, const void* q,
+                     const void* k_new, int bh, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
+                     void* k_hat, int64_t append_row, float* iter_out, float* deltas, int dtype) {
+  const int vec = dtype == LRQK_F32 ? 4 : 8;
+  int lpr_log2 = 0;
+  while ((1 << lpr_log2) < d / vec) ++lpr_log2;
+  if (dtype == LRQK_F32)
+    return als_decode_finish<float>(ctx, b_q, b_k, a_k, head_stride, q, k_new, bh, hq, hkv, r, d, lpr_log2, max_iter, tol,
+                                    q_hat, k_hat, append_row, iter_out, deltas, true, nullptr);
+  return als_decode_finish<bf16_t>(ctx, b_q, b_k, a_k, head_stride, q, k_new, bh, hq, hkv, r, d, lpr_log2, max_iter, tol,
+                                   q_hat, k_hat, append_row, iter_out, deltas, true, nullptr);
+}
+
 // Runs a deferred finish stage as its own launch (when no later launch of the step took it over).
 int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st) {
   if (!ctx->fin_pending) return LRQK_OK;
@@ -1205,6 +1218,7 @@ extern "C" int lrqk_als_decode(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, i
                                int max_iter, float tol, void* q_hat, void* k_hat, int64_t append_row, int dtype,
                                void* stream) {
   GramAppend ap{nullptr, nullptr, nullptr, nullptr, -1, 0, hq, hkv};
+  if (ctx) ctx->fs_valid = false;  // B_Q, B_K change behind the kept state of the decode step
   return als_decode_checked(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, k_prev, kprev_slots, n, q, k_new, b,
                             hq, hkv, r, d, max_iter, tol, q_hat, k_hat, append_row, ap, false, dtype, (hipStream_t)stream);
 }

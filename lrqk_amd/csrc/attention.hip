@@ -264,7 +264,8 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
                                                      int k, int h, int blk, int nblk, const T* __restrict__ q, int d,
                                                      float scale_log2e, float* __restrict__ pout,
                                                      const int32_t* __restrict__ miss_old, const VictimView& vic,
-                                                     const int32_t* __restrict__ miss_new) {
+                                                     const int32_t* __restrict__ miss_new, uint4* __restrict__ evk,
+                                                     int evk_rows) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float accs[8][256 + 2];               // [row group][m, l, acc[d]] (at most 8 groups are merged at a time)
   const int tid = threadIdx.x, lane = lane_id();
@@ -381,9 +382,25 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
         }
         if (ok[u] && c == 0 && !from_fifo[u]) atomicAdd(&vic.host_rows[h], 1);
       }
+      // the K rows that leave their slots, in the order of the miss list, for the kept sums of the factor update
+      if (evk) {
+#pragma unroll
+        for (int u = 0; u < kFR; ++u)
+          if (ok[u] && is_k && j[u] < evk_rows) evk[((int64_t)h * evk_rows + j[u]) * cpr + c] = old_val[u];
+      }
     } else {
+      uint4 old_val[kFR];
+      if (evk) {  // (uniform)
+#pragma unroll
+        for (int u = 0; u < kFR; ++u) old_val[u] = *own[u];
+      }
 #pragma unroll
       for (int u = 0; u < kFR; ++u) val[u] = *(ok[u] ? host_src[u] : own[u]);
+      if (evk) {
+#pragma unroll
+        for (int u = 0; u < kFR; ++u)
+          if (ok[u] && is_k && j[u] < evk_rows) evk[((int64_t)h * evk_rows + j[u]) * cpr + c] = old_val[u];
+      }
     }
 #pragma unroll
     for (int u = 0; u < kFR; ++u) {
@@ -463,14 +480,16 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
 // launch depends on, and after it one that encodes the appended row for the score index (if there
 // is one).  The copy is bound by the host link, so the other roles ride along.
 template <typename T>
-__global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
+__global__ __launch_bounds__(kAttnThreads, 4) void fetch_attn_partial_kernel(
     const uint4* __restrict__ store, int64_t cap, int32_t* __restrict__ hit, int64_t hit_stride,
     const int32_t* __restrict__ miss_slots, const int32_t* __restrict__ miss_count, const uint8_t* __restrict__ evict,
     int hq, int hkv, int cpr, int k, int n_fetch, const T* __restrict__ q, T* __restrict__ K, T* __restrict__ V,
     int n_slots, int d, int lpr_log2, float scale_log2e, float* __restrict__ part, int S, int with_finish,
     FinishArgs fa, const int32_t* __restrict__ miss_old, VictimView vic, const int32_t* __restrict__ miss_new,
-    const float* __restrict__ kq) {
+    const float* __restrict__ kq, uint4* __restrict__ evk, int evk_rows, int32_t* __restrict__ count_copy) {
   const int h = blockIdx.y;
+  // (the caller's copy of the miss counts, when the kernels keep them in the library's own block)
+  if (count_copy && blockIdx.x == 0 && threadIdx.x == 0) count_copy[h] = miss_count[h];
   if (with_finish && (int)blockIdx.x >= n_fetch + S) {
     if ((int)blockIdx.x == n_fetch + S)
       als_finish_body<T>(fa, h);
@@ -481,7 +500,8 @@ __global__ __launch_bounds__(kAttnThreads) void fetch_attn_partial_kernel(
   if ((int)blockIdx.x < n_fetch) {
     fetch_rows_attn_body<T>(store, cap, (uint4*)K, (uint4*)V, n_slots, hit, hit_stride, miss_slots, miss_count, hq, hkv,
                             cpr, k, h, blockIdx.x, n_fetch, q, d, scale_log2e,
-                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic, miss_new);
+                            part + ((int64_t)h * (S + n_fetch) + S + blockIdx.x) * (d + 2), miss_old, vic, miss_new, evk,
+                            evk_rows);
     return;
   }
   // (eight row groups in flight per wave: the launch has few attention workgroups)
@@ -647,7 +667,8 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
                                 int n_slots, int32_t* hit, int64_t hit_stride, const int32_t* miss_slots,
                                 const int32_t* miss_count, const uint8_t* evict, int b, int hq, int hkv, int d, int k,
                                 const void* q, void* out, hipStream_t st, const int32_t* miss_old,
-                                const VictimView* vicp, const int32_t* miss_new) {
+                                const VictimView* vicp, const int32_t* miss_new, void* evk, int evk_rows,
+                                int32_t* count_copy) {
   const int bh = b * hq;
   VictimView vic{};
   if (vicp && miss_old && vicp->nv > 0) vic = *vicp;
@@ -698,7 +719,8 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
   hipLaunchKernelGGL((fetch_attn_partial_kernel<T>), dim3((unsigned)(n_fetch + S + with_finish + index_role), (unsigned)bh),
                      dim3(kAttnThreads), 0, st, (const uint4*)dev_store, cap, hit, hit_stride, miss_slots, miss_count,
                      evict, hq, hkv, cpr, k, n_fetch, (const T*)q, (T*)k_act, (T*)v_act, n_slots, d, lpr_log2,
-                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new, kq);
+                     scale_log2e, (float*)ctx->attn_part.p, S, with_finish, ctx->fin, miss_old, vic, miss_new, kq,
+                     (uint4*)evk, evk_rows, count_copy);
   LRQK_HIP_CHECK(hipGetLastError());
   if (out) {
     hipLaunchKernelGGL((attn_combine_kernel<T>), dim3((unsigned)bh), dim3(kCombThreads), 0, st,
@@ -715,7 +737,8 @@ static int fetch_attention_impl(lrqk_ctx* ctx, const void* dev_store, int64_t ca
 int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_act, void* v_act, int n_slots,
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
-                    hipStream_t st, const int32_t* miss_old, const VictimView* vic, const int32_t* miss_new) {
+                    hipStream_t st, const int32_t* miss_old, const VictimView* vic, const int32_t* miss_new, void* evk,
+                    int evk_rows, int32_t* count_copy) {
   const void* dev_store = nullptr;
   int rc = resolve_store(kv_store, &dev_store);
   if (rc) return rc;
@@ -724,9 +747,11 @@ int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_ac
                LRQK_EINVAL, "pointers must be 16-byte aligned");
   if (dtype == LRQK_F32)
     return fetch_attention_impl<float>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                       miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new);
+                                       miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new, evk,
+                                       evk_rows, count_copy);
   return fetch_attention_impl<bf16_t>(ctx, dev_store, cap, k_act, v_act, n_slots, hit, hit_stride, miss_slots,
-                                      miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new);
+                                      miss_count, evict, b, hq, hkv, d, k, q, out, st, miss_old, vic, miss_new, evk,
+                                      evk_rows, count_copy);
 }
 
 }  // namespace lrqk

@@ -50,6 +50,9 @@ extern "C" int lrqk_ctx_destroy(lrqk_ctx* ctx) {
   ctx->als_pre.release();
   ctx->als_kq.release();
   ctx->als_iter.release();
+  ctx->als_iter64.release();
+  ctx->fstate.release();
+  ctx->evk.release();
   ctx->prefill_ws.release();
   ctx->prefill_gd.release();
   ctx->new_idx.release();

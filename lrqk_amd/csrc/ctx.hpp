@@ -58,6 +58,20 @@ struct lrqk_ctx {
   int kq_bh = 0, kq_n = 0;
   lrqk::DevBuf als_pre;     // f32 [bh][4*1024 + 65]: what the solve needs from B_Q, B_K, q, k (formed beside the Gram pass)
   lrqk::DevBuf als_iter;    // f32 [bh][MAX_IT][2r] + deltas
+  lrqk::DevBuf als_iter64;  // f64 [bh][MAX_IT][2r]: the same iterates before rounding to fp32 (kept-state update only)
+  int iter64_bh = 0, iter64_r = 0, iter64_iters = 0;
+  int64_t iter64_token = -1;  // token whose step left them
+  // Kept state of the decode step's factor update (als_state.hip): per head, fp64, the sums over the active slots
+  // and the inverses / projections that the next step starts from.
+  lrqk::DevBuf fstate;      // f64 [bh][3 d 32 + 3 * 1024]
+  lrqk::DevBuf evk;         // storage dtype [bh][evk_rows][d]: K rows that the step's misses replaced
+  int evk_rows = 0;
+  bool fs_enabled = false;  // lrqk_ctx_factor_state
+  bool fs_valid = false;    // fstate describes the buffers below as the next step (fs_next_*) will find them
+  const void *fs_bq = nullptr, *fs_bk = nullptr, *fs_ak = nullptr, *fs_kact = nullptr, *fs_idx = nullptr;
+  int64_t fs_head_stride = 0;
+  int fs_bh = 0, fs_r = 0, fs_d = 0, fs_dtype = -1, fs_topk = 0, fs_n = 0, fs_next_slot = -1;
+  int32_t fs_next_token = -1;
   lrqk::DevBuf prefill_ws;  // prefill ALS accumulators
   lrqk::DevBuf prefill_gd;  // prefill ALS on Gram matrices: X^T X sums, fp64 state
   lrqk::DevBuf new_idx;     // i32 [bh][k] selection result of the fused step
@@ -131,6 +145,26 @@ int als_decode_append(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t he
                       const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
                       void* k_hat, int64_t append_row, int slot, int32_t token, bool defer_finish, int dtype,
                       hipStream_t st);
+// Leaves the finish stage of a factor update whose iterates are in iter_out / deltas pending in the ctx (the
+// step's later launches absorb it, flush_pending_finish otherwise).
+int als_defer_finish(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, const void* q,
+                     const void* k_new, int bh, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
+                     void* k_hat, int64_t append_row, float* iter_out, float* deltas, int dtype);
+// The factor update from kept state (als_state.hip).
+constexpr int kStepFusedDiffMaxK = 4096;  // the select kernel's in-kernel diff (it lists the replaced tokens)
+bool factor_state_supported(int r, int d, int dtype, int max_iter);
+int factor_state_rebuild(lrqk_ctx* ctx, const void* b_q, const void* b_k, const void* a_k, int64_t head_stride,
+                         const int32_t* active_idx, int64_t idx_stride, const void* k_act, int n_slots, int bh, int r,
+                         int d, int topk, int skip_slot, int dtype, hipStream_t st);
+int factor_state_advance(lrqk_ctx* ctx, const void* b_q, const void* b_k, const void* a_k, int64_t head_stride,
+                         const int32_t* active_idx, int64_t idx_stride, const void* k_act, int n_slots,
+                         const int32_t* miss_slots, const int32_t* miss_old, const int32_t* miss_new,
+                         const int32_t* miss_count, int64_t cap, int bh, int r, int d, int topk, int ring_slot,
+                         int32_t ring_token, int skip_slot, int dtype, hipStream_t st);
+int factor_state_quick(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64_t head_stride, int32_t* active_idx,
+                       int64_t idx_stride, void* k_act, void* v_act, int n_slots, const void* q, const void* k_new,
+                       const void* v_new, int b, int hq, int hkv, int r, int d, int max_iter, float tol, void* q_hat,
+                       void* k_hat, int64_t append_row, int slot, int32_t token, int dtype, hipStream_t st);
 // Runs a deferred finish stage as its own launch (no-op if none is pending).
 int flush_pending_finish(lrqk_ctx* ctx, hipStream_t st);
 // Miss fetch overlapped with the attention over the slots that stay resident (one launch), then
@@ -139,7 +173,8 @@ int fetch_attention(lrqk_ctx* ctx, const void* kv_store, int64_t cap, void* k_ac
                     int32_t* hit, int64_t hit_stride, const int32_t* miss_slots, const int32_t* miss_count,
                     const uint8_t* evict, int b, int hq, int hkv, int d, int k, const void* q, void* out, int dtype,
                     hipStream_t st, const int32_t* miss_old = nullptr, const VictimView* vic = nullptr,
-                    const int32_t* miss_new = nullptr);
+                    const int32_t* miss_new = nullptr, void* evk = nullptr, int evk_rows = 0,
+                    int32_t* count_copy = nullptr);
 // Makes the score index cover rows [0, m) of a_k (building or extending it as needed).  Returns 1 and
 // fills `view` if the scan may use it, 0 if the index is off or does not apply, negative on error.
 int score_index_prepare(lrqk_ctx* ctx, const void* a_k, int64_t head_stride, int bh, int64_t m, int r, int dtype,

@@ -2,6 +2,8 @@
 // update, proxy-score scan + top-k, hit/miss diff, miss fetch and (optionally) the exact
 // attention over the active set.  Only launches; never synchronises.
 #include "common.hpp"
+#include <algorithm>
+
 #include "ctx.hpp"
 
 using namespace lrqk;
@@ -28,7 +30,10 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   if ((rc = ctx->misc.ensure((size_t)bh * topk * 13 + (size_t)bh * 4 + 64))) return rc;
   int32_t* new_idx = (int32_t*)ctx->new_idx.p;
   int32_t* miss_slots = (int32_t*)ctx->misc.p;
-  int32_t* mcount = miss_count ? miss_count : miss_slots + (size_t)bh * topk;
+  // (the counts stay in the library's own block: a launch that reads them may run after the caller has let go
+  // of its buffer; the caller's copy is written by the step's last launch, or the kernels use its buffer directly)
+  int32_t* mcount_own = miss_slots + (size_t)bh * topk;
+  int32_t* mcount = miss_count ? miss_count : mcount_own;
   int32_t* miss_old = miss_slots + (size_t)bh * topk + bh;
   int32_t* miss_new = miss_old + (size_t)bh * topk;
   uint8_t* ev = evict ? evict : (uint8_t*)(miss_new + (size_t)bh * topk);
@@ -40,12 +45,41 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   // (without attn_out the same launch runs with its fetch, finish and index roles only)
   const bool fused_tail = !no_hit_miss && ctx->fetch_mode == 0 && 2 * (size_t)d * elem_size(dtype) / 16 <= (size_t)kWave;
   const bool defer_finish = fused_tail;
-  // ring append folded into the first kernel of the factor update; the flush of a full ring
-  // (which reads the slot just written) follows it
-  if ((rc = als_decode_append(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq, hkv,
-                              r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, defer_finish,
-                              dtype, (hipStream_t)stream)))
-    return rc;
+  // The factor update from kept state (als_state.hip, if the ctx has it switched on): one small launch before the
+  // scan, and after the fetch one launch that brings the state up to date.  It needs the replaced tokens listed
+  // (the select kernel's own diff) and the fused tail; every other path runs the update over the active rows, and
+  // leaves the kept state invalid.
+  const bool quick = fused_tail && ctx->fs_enabled && m > topk && topk <= kStepFusedDiffMaxK &&
+                     factor_state_supported(r, d, dtype, max_iter) && (int64_t)b * hq <= 65535;
+  if (quick) {
+    mcount = mcount_own;
+    const bool valid = ctx->fs_valid && ctx->fstate.p && ctx->fs_bq == b_q && ctx->fs_bk == b_k && ctx->fs_ak == a_k &&
+                       ctx->fs_kact == k_act && ctx->fs_idx == active_idx && ctx->fs_head_stride == head_stride &&
+                       ctx->fs_bh == bh && ctx->fs_r == r && ctx->fs_d == d && ctx->fs_dtype == dtype &&
+                       ctx->fs_topk == topk && ctx->fs_n == n && ctx->fs_next_slot == topk + ring_slot &&
+                       ctx->fs_next_token == token;
+    ctx->fs_valid = false;  // until this step has brought it up to date
+    const int evk_rows = std::min(topk, std::max(256, topk / 2));
+    if ((rc = ctx->evk.ensure((size_t)bh * evk_rows * d * elem_size(dtype)))) return rc;
+    ctx->evk_rows = evk_rows;
+    if (!valid) {
+      if ((rc = factor_state_rebuild(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, n, bh, r, d, topk,
+                                     topk + ring_slot, dtype, (hipStream_t)stream)))
+        return rc;
+    }
+    if ((rc = factor_state_quick(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq,
+                                 hkv, r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, dtype,
+                                 (hipStream_t)stream)))
+      return rc;
+  } else {
+    ctx->fs_valid = false;
+    // ring append folded into the first kernel of the factor update; the flush of a full ring
+    // (which reads the slot just written) follows it
+    if ((rc = als_decode_append(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, v_act, n, q, k_new, v_new, b, hq,
+                                hkv, r, d, max_iter, tol, q_hat, k_hat, token, topk + ring_slot, token, defer_finish,
+                                dtype, (hipStream_t)stream)))
+      return rc;
+  }
   if (flush_row0 >= 0) {
     if ((rc = lrqk_flush_ring(k_act, v_act, n, topk, lite, kv_store, cap, flush_row0, b, hq, hkv, d, dtype, stream)))
       return rc;
@@ -86,9 +120,36 @@ extern "C" int lrqk_decode_step(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, 
   }
   if (fused_tail) {
     // the fetch is bound by the host link: the attention over the resident slots runs beside it
-    return fetch_attention(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, ev, b, hq, hkv, d,
-                           topk, q, attn_out, dtype, (hipStream_t)stream, miss_old, vic_active ? vic : nullptr,
-                           fused_diff ? miss_new : nullptr);
+    const bool keep_state = quick && fused_diff;
+    if ((rc = fetch_attention(ctx, kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, ev, b, hq, hkv, d,
+                              topk, q, attn_out, dtype, (hipStream_t)stream, miss_old, vic_active ? vic : nullptr,
+                              fused_diff ? miss_new : nullptr, keep_state ? ctx->evk.p : nullptr, ctx->evk_rows,
+                              miss_count && mcount != miss_count ? miss_count : nullptr)))
+      return rc;
+    if (keep_state) {
+      if ((rc = flush_pending_finish(ctx, (hipStream_t)stream))) return rc;  // (the fetch launch carried it, normally)
+      const int next_slot = topk + (ring_slot + 1) % lite;
+      if ((rc = factor_state_advance(ctx, b_q, b_k, a_k, head_stride, active_idx, n, k_act, n, miss_slots, miss_old,
+                                     miss_new, mcount, cap, bh, r, d, topk, topk + ring_slot, token, next_slot, dtype,
+                                     (hipStream_t)stream)))
+        return rc;
+      ctx->fs_bq = b_q;
+      ctx->fs_bk = b_k;
+      ctx->fs_ak = a_k;
+      ctx->fs_kact = k_act;
+      ctx->fs_idx = active_idx;
+      ctx->fs_head_stride = head_stride;
+      ctx->fs_bh = bh;
+      ctx->fs_r = r;
+      ctx->fs_d = d;
+      ctx->fs_dtype = dtype;
+      ctx->fs_topk = topk;
+      ctx->fs_n = n;
+      ctx->fs_next_slot = next_slot;
+      ctx->fs_next_token = token + 1;
+      ctx->fs_valid = true;
+    }
+    return LRQK_OK;
   }
   if ((rc = lrqk_fetch_rows(kv_store, cap, k_act, v_act, n, active_idx, n, miss_slots, mcount, b, hq, hkv, d, topk, dtype,
                             stream)))

@@ -82,6 +82,9 @@ class LightAttentionIndicesFactory:
         self.victim_rows: Optional[int] = None
         # 8-bit copy of the A_K rows read by the scan (bounds + exact rescoring of the rows that may pass)
         self.use_score_index = True
+        # True: the decode step's factor update runs in fp64 from state kept between steps (iterates equal to an
+        # fp64 evaluation to rounding; one more launch per step); False: over the active rows in fp32
+        self.use_factor_state = False
 
     # ------------------------------------------------------------------ small accessors
     @property
@@ -138,6 +141,7 @@ class LightAttentionIndicesFactory:
         v = value.reshape(value.shape[0], value.shape[1], -1)
         self._hit_len = v.shape[2]
         self._active_idx[:, :, :self._hit_len] = v.to(torch.int32)
+        self.ws.factor_state(self.use_factor_state)   # the kept sums describe the old ids
 
     @property
     def A_K_hitted(self):
@@ -162,6 +166,7 @@ class LightAttentionIndicesFactory:
         self.B_K = B_K
         # rows of A_K were written behind the library's back: whatever the scan had indexed is dropped
         self.ws.score_index(self.use_score_index)
+        self.ws.factor_state(self.use_factor_state)
         return self
 
     def _is_overridden(self, name: str) -> bool:
@@ -189,7 +194,9 @@ class LightAttentionIndicesFactory:
     def fetch_by_hit(self, dst: torch.Tensor, src: torch.Tensor, hit_indices: torch.Tensor,
                      dst_mask: Optional[torch.Tensor] = None):
         """lrqk_attention.py:1317-1383.  dst [b,Hq,<=k,d] must be the topk area of Kgpu or Vgpu
-        (a narrow view); src [b,Hkv,seq,d] on the GPU, or the pinned [K|V] store with dst_mask."""
+        (a narrow view); src [b,Hkv,seq,d] on the GPU or in pinned host memory: a K or a V source whose rows
+        are as wide as dst's (not the 2d-wide [K|V] store: such a source is refused); with dst_mask only the
+        slots it marks are written."""
         b, H = hit_indices.shape[:2]
         idx = hit_indices.reshape(b, H, -1).to(device=dst.device, dtype=torch.int32)
         count = idx.shape[2]
@@ -203,6 +210,7 @@ class LightAttentionIndicesFactory:
             if dst_mask is not None:
                 idx = torch.where(dst_mask.reshape(b, H, -1).to(dst.device), idx, torch.full_like(idx, -1))
         ops.gather_rows(src if not src.is_cuda else src.contiguous(), idx.contiguous(), full, count)
+        self.ws.factor_state(self.use_factor_state)   # rows of the active set changed
         return dst if count >= self.attn_topk else dst.narrow(2, 0, count)
 
     # ------------------------------------------------------------------ prefill
@@ -317,6 +325,7 @@ class LightAttentionIndicesFactory:
 
         if self.current_len <= self.gpu_capacity:
             # growing-prefix branch (lrqk_attention.py:1526-1545): no selection yet
+            self.ws.factor_state(self.use_factor_state)
             ops.append_token(kn, vn, self.Kgpu, self.Vgpu, k + slot, self._active_idx, token)
             if flush_row0 >= 0:
                 ops.flush_ring(self.Kgpu, self.Vgpu, k, L, self.KVcpu.data, flush_row0, hkv)
@@ -348,6 +357,7 @@ class LightAttentionIndicesFactory:
         k, L = self.attn_topk, self.num_lite_tokens
         hkv = kn.shape[1]
         a_k = self._A_K.data
+        self.ws.factor_state(self.use_factor_state)   # this step changes the active set stage by stage
         ops.append_token(kn, vn, self.Kgpu, self.Vgpu, k + slot, self._active_idx, token)
         if flush_row0 >= 0:
             ops.flush_ring(self.Kgpu, self.Vgpu, k, L, self.KVcpu.data, flush_row0, hkv)

@@ -60,6 +60,25 @@ class Workspace:
         """Size (and empty) the victim cache of the fused decode step; 0 switches it off."""
         check(_lib.load().lrqk_ctx_victim_cache(self.handle, int(rows_per_head)))
 
+    def factor_state(self, enable: bool = True):
+        """Switch the kept state of the decode step's factor update on or off; either way what is kept is
+        dropped (call it after changing B_Q, B_K, the active ids or rows behind the library's back)."""
+        check(_lib.load().lrqk_ctx_factor_state(self.handle, 1 if enable else 0))
+
+    def last_iterates(self, token: Optional[int] = None) -> Optional[torch.Tensor]:
+        """fp64 [bh, max_iter, 2, r]: (q_hat, k_hat) of every iteration of the last decode step that ran from
+        kept state, before any rounding; None if no such step ran (with ``token``: if that token's step did not)."""
+        bh, it, r, tok = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int64()
+        lib = _lib.load()
+        check(lib.lrqk_last_iterates(self.handle, None, 0, ctypes.byref(bh), ctypes.byref(it), ctypes.byref(r),
+                                     ctypes.byref(tok)))
+        if bh.value * it.value * r.value == 0 or (token is not None and tok.value != token):
+            return None
+        out = torch.empty((bh.value, it.value, 2, r.value), dtype=torch.float64)
+        check(lib.lrqk_last_iterates(self.handle, out.data_ptr(), out.numel(), ctypes.byref(bh), ctypes.byref(it),
+                                     ctypes.byref(r), ctypes.byref(tok)))
+        return out
+
     def victim_stats(self, reset: bool = True) -> int:
         """Rows the fused decode step fetched over the host link since the last reset."""
         n = ctypes.c_int64()
@@ -249,6 +268,13 @@ def gather_rows(src: torch.Tensor, idx: torch.Tensor, dst: torch.Tensor, count: 
         raise ValueError("a host source must be pinned memory")
     b, hkv, l, d = src.shape
     _, hq, n, _ = dst.shape
+    # the kernel takes the row width and the element type from src alone: a source whose rows are wider than
+    # the destination's (the [K|V] store, 2d wide) would be written past the end of dst
+    if src.shape[-1] != dst.shape[-1] or src.dtype != dst.dtype or src.shape[0] != dst.shape[0]:
+        raise ValueError(f"source rows {tuple(src.shape)} {src.dtype} do not match the destination "
+                         f"{tuple(dst.shape)} {dst.dtype}: pass a K or a V source whose rows are as wide as dst")
+    if hq % hkv != 0 or tuple(idx.shape[:2]) != (b, hq) or not 0 <= count <= min(idx.shape[2], n):
+        raise ValueError("idx must be [b,Hq,>=count] with count slots inside dst")
     assert src.is_contiguous() and dst.is_contiguous() and idx.is_contiguous() and idx.dtype == torch.int32
     check(_lib.load().lrqk_gather_rows(src.data_ptr(), l, idx.data_ptr(), idx.shape[2], count, dst.data_ptr(), n, b, hq,
                                        hkv, d, _dt(src), _stream(dst)))
