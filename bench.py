@@ -33,8 +33,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # the same runs).  The summary of those runs is kept under profiles/.
 # Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
 # 8-bit copy (34 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
-MEASURED_TRAFFIC_BYTES = {("llama8b_128k_bf16", True): (78844.6 * 2.000 + 867.2 * 1.000) * 1024,
-                          ("llama8b_128k_bf16", False): (131110.0 * 2.000 + 1060.2 * 1.000) * 1024}
+MEASURED_TRAFFIC = {
+    ("llama8b_128k_bf16", True): {"bytes": (78844.6 * 2.000 + 867.2 * 1.000) * 1024, "rows_rescored_in_that_run": 171000,
+                                  "profile": "profiles/score_filter_llama8b_128k_hbm_traffic.md"},
+    ("llama8b_128k_bf16", False): {"bytes": (131110.0 * 2.000 + 1060.2 * 1.000) * 1024, "rows_rescored_in_that_run": 0,
+                                   "profile": "profiles/score_filter_llama8b_128k_hbm_traffic.md"}}
 
 
 def parse():
@@ -48,11 +51,24 @@ def parse():
     p.add_argument("--cpu-steps", type=int, default=160,
                    help="decode mode: oracle steps timed for cpu_baseline (about 12 s of host work at the 128K "
                         "configuration); the other modes only ask whether it is 0 (= no cpu_baseline)")
-    p.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, os.cpu_count())")
-    p.add_argument("--event-every", type=int, default=0,
-                   help="bracket every n-th proxy-score launch of the timed region with HIP events (each pair "
-                        "of event packets delays its step by ~10 us, so every launch would inflate the step time); "
-                        "0 = every 8th, or more often so that at least 32 launches are bracketed")
+    p.add_argument("--cpu-threads", type=int, default=0,
+                   help="0 = every core this process may use (affinity mask, OMP_NUM_THREADS where the host is shared)")
+    p.add_argument("--min-timed", type=int, default=512,
+                   help="decode mode: when --steps is smaller than this, `value` is timed over this many steps in a "
+                        "second region (the region of exactly --steps steps is reported beside it)")
+    p.add_argument("--event-steps", type=int, default=64,
+                   help="decode mode: steps of the pass after the timed regions in which every proxy-score launch of "
+                        "the first copy sits between two HIP events (no timed region has an event inside a step)")
+    p.add_argument("--also", default="auto", choices=["auto", "on", "off"],
+                   help="decode mode: add compact results of the other configurations (32K decode, four sequences, "
+                        "prefill factorisation, full decoder) under the `also` key; auto = for the default workload "
+                        "with no overrides")
+    p.add_argument("--no-also-decoder", dest="also_decoder", action="store_false",
+                   help="leave the full decoder out of `also`")
+    p.add_argument("--also-budget-s", type=float, default=150.0,
+                   help="the full decoder of `also` is skipped when the run has already taken this long")
+    p.add_argument("--no-probe-sweep", action="store_true",
+                   help="skip the sweep over the variants of the plain read kernel")
     p.add_argument("--no-attn", action="store_true", help="leave the attention kernel out of the step")
     p.add_argument("--variant", default="default", choices=["default", "no_hit_miss"])
     p.add_argument("--fetch", default="direct", choices=["direct", "staged"],
@@ -101,8 +117,9 @@ def parse():
     p.add_argument("--warm-steps", type=int, default=128,
                    help="decode mode: after the timed region, step the first copy alone this many times and report "
                         "that (cache-warm) time per step as a secondary figure; 0 = skip")
-    p.add_argument("--probe-mb", type=int, default=1024,
-                   help="decode mode: size of the plain read / copy kernels whose rates are reported beside the scan's")
+    p.add_argument("--probe-mb", type=int, default=2048,
+                   help="decode mode: size of the buffer the sweep of plain read kernels runs over (the default read / "
+                        "copy pair runs over at most 1024 MiB); 0 = no probes")
     p.add_argument("--calib-copy-mb", type=int, default=0,
                    help="after the timed region, run one plain device copy of this many MiB (a known-size "
                         "kernel to scale hardware counters by)")
@@ -171,7 +188,7 @@ def prefill_als(a):
     if a.cpu_steps > 0:
         # the oracle's fp32 run of the same factorisation on a few heads, scaled to all heads
         from oracle import lrqk_oracle as orc
-        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        threads, host = host_threads(a)
         torch.set_num_threads(threads)
         hs = list(range(0, w.num_heads, max(1, w.num_heads // 4)))[:4]
         Qc = Q[:, hs].float().cpu()
@@ -184,6 +201,7 @@ def prefill_als(a):
         cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": threads, "kind": "port",
                "sample": f"fp32 torch-CPU factorisation of {len(hs)} of the {w.num_heads} heads at the full length "
                          f"on {threads} threads, scaled to all heads"}
+        cpu.update(host)
     # one pass = apply (2 l d r) + Grams (2 l r (r + d)); 2 initial Gram passes + 2 passes per iteration
     flops = bh * (2 * 2.0 * l * r * (r + d) + iters * 2 * (2.0 * l * d * r + 2.0 * l * r * (r + d)))
     e = 2 if w.dtype == torch.bfloat16 else 4
@@ -237,7 +255,7 @@ def prefill_als(a):
            "rel_residual_K": round((num_k / den_k) ** 0.5, 6), "rel_residual_Q": round((num_q / den_q) ** 0.5, 6),
            "roofline": roof,
            "cpu_baseline": cpu}
-    print(json.dumps(out))
+    return out
 
 
 def decoder(a):
@@ -283,7 +301,7 @@ def decoder(a):
         # and context, continued from layer 0's state with stand-in q, k, v; everything else a decoded position
         # needs (projections, MLP, lm_head, the other layers) is not in this figure
         import types
-        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        threads, host = host_threads(a)
         torch.set_num_threads(threads)
         eng0 = cache.lwattn[0]
         wl = types.SimpleNamespace(lite_tokens=64, num_active_tokens=2048, groups=cfg.heads // cfg.kv_heads, r=32,
@@ -301,6 +319,7 @@ def decoder(a):
         cpu = {"value": round(cpu_s * 1e6, 1), "unit": "us/layer-step (cache path only)", "cores": threads, "kind": "port",
                "sample": f"one decode step of layer 0's cache path at batch {a.batch} continued from the GPU state "
                          f"(stand-in q, k, v); compare with cache_path_us_per_layer_step"}
+        cpu.update(host)
     out = {"metric": "lrqk_decoder_tokens_per_s", "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1,
            "steps": n_dec, "warmup": 0, "ms_per_step": round(t_decode / n_dec * 1e3, 3), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -316,42 +335,41 @@ def decoder(a):
            "cache_path_us_per_layer_step": round(path_us, 1),
            "other_us_per_layer_step": round(t_extra / cfg.layers * 1e6 - path_us, 1),
            "roofline": None, "cpu_baseline": cpu}
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    a = parse()
-    if a.gpus != 1:
-        print("bench.py measures one GPU: the LRQK cache path has no multi-GPU part (heads shard trivially); "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
+def host_threads(a):
+    """Threads for the CPU legs: every core this process may use (its affinity mask, and the share of the host that
+    OMP_NUM_THREADS names where the machine is shared between jobs), with the counts it was chosen from."""
+    n_all = os.cpu_count() or 1
+    try:
+        n_aff = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n_aff = n_all
+    try:
+        share = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        share = 0
+    n = a.cpu_threads or max(1, min(n_aff, share or n_aff))
+    return n, {"host_cpu_count": n_all, "cpus_in_affinity_mask": n_aff, "omp_num_threads_env": share or None}
+
+
+def decode_bench(a, compact=False):
+    """One decode-mode measurement; returns the result line as a dict (compact: the few keys of a sub-result)."""
     from lrqk_amd import synth
     import lrqk_amd
-    from lrqk_amd import _lib
     from lrqk_amd import ops as ops_mod
-    _lib.load()  # fail loudly if the HIP library is missing
-    if a.mode == "prefill_als":
-        return prefill_als(a)
-    if a.mode == "decoder":
-        return decoder(a)
-
+    import dataclasses
     dev = torch.device("cuda:0")
     w = synth.WORKLOADS[a.workload]
     if a.seqs > 0 and a.seqs != w.batch:
-        import dataclasses
         w = dataclasses.replace(w, batch=a.seqs)
     if a.max_iter > 0:
-        import dataclasses
         w = dataclasses.replace(w, max_iter=(a.max_iter, a.max_iter), tol=(a.tol, a.tol))
     if a.rank or a.topk or a.lite:
-        import dataclasses
         w = dataclasses.replace(w, r=a.rank or w.r, num_active_tokens=a.topk or w.num_active_tokens,
                                 lite_tokens=a.lite or w.lite_tokens)
     if a.data_rank:
-        import dataclasses
         w = dataclasses.replace(w, rho=a.data_rank)
     l = a.context or w.context
     t_setup = time.perf_counter()
@@ -359,6 +377,7 @@ def main():
     Q, K, V, bases, gen = synth.prompt_qkv(w, a.seed, l, device=dev)
     A0 = synth.init_factors(w, l, a.seed + 1, device=dev)
     cls = lrqk_amd.LightAttentionIndicesNoHitMiss if a.variant == "no_hit_miss" else lrqk_amd.LightAttentionIndicesFactory
+
     def make_engine():
         e_ = cls(num_lite_tokens=w.lite_tokens, attn_topk=w.num_active_tokens, num_key_value_groups=w.groups, r=w.r,
                  max_iter=w.max_iter, tol=w.tol, capacity=4096)
@@ -383,11 +402,14 @@ def main():
         others.append(o_)
     del A0
     stream = synth.DecodeStream(w, Q[:, :, -1:], bases, gen)
-    a.warmup_asked = a.warmup
-    a.warmup += max(0, a.settle)  # all untimed alike; the line reports both numbers
+    n_warm = a.warmup + max(0, a.settle)  # all untimed alike; the line reports both numbers
     copies = 1 + len(others)
+    # the timed regions, in this order: exactly --steps steps; a longer one (at least --min-timed steps) when --steps
+    # is short; a few steps with every scan launch between events; the first copy alone, back to back
+    long_steps = a.min_timed if a.steps < a.min_timed else 0
+    ev_steps = max(0, a.event_steps)
     warm_steps = max(0, a.warm_steps) if copies > 1 else 0
-    total = a.warmup + a.steps + warm_steps
+    total = n_warm + a.steps + long_steps + ev_steps + warm_steps
     qs, ks, vs = [], [], []
     for _ in range(total):
         q, k, v = stream.next()
@@ -401,7 +423,7 @@ def main():
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
 
-    for i in range(a.warmup):
+    for i in range(n_warm):
         eng.decode(qs[i], ks[i], vs[i])
         for o_ in others:
             o_.decode(qs[i], ks[i], vs[i])
@@ -409,16 +431,7 @@ def main():
             torch.cuda.synchronize()  # (untimed: keeps the launch queue short)
     torch.cuda.synchronize()
     cap_before = (eng._A_K.capacity, eng.KVcpu.capacity)
-    m_first = eng.lite_indices[eng.lite_len] - 1
 
-    # at least 32 bracketed launches (when there are that many steps), at most every 8th
-    every = a.event_every if a.event_every > 0 else max(1, min(8, a.steps // 32))
-    eng.ws.timing_enable(a.steps, every=every)
-    eng.ws.select_stats(reset=True)
-    eng.ws.victim_stats(reset=True)
-    counts = []
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
     # The host enqueues a step in less than half the time the GPU needs for it.  Left alone it runs thousands
     # of launches ahead, and once the runtime's launch queue is full (at about 2000 launches here) every
     # further launch waits in a way that leaves gaps on the GPU.  So the host stays at most 128 layer-steps
@@ -426,9 +439,13 @@ def main():
     # runs dry.  The same marks (one per 32 layer-steps) give the spread of the step time.
     mark_every = max(1, 32 // copies)   # engine iterations between marks
     ahead = max(2, 128 // (mark_every * copies))
-    marks = []
 
     def timed_loop(first, count, engines):
+        """count steps of every engine in turn, with no event inside a step: (seconds per layer-step, sorted
+        microseconds per layer-step of every mark interval, miss counts of the first engine)."""
+        marks, counts = [], []
+        torch.cuda.synchronize()
+        t_ = time.perf_counter()
         for i in range(first, first + count):
             if (i - first) % mark_every == 0:
                 marks.append(torch.cuda.Event(enable_timing=True))
@@ -441,56 +458,89 @@ def main():
                     counts.append(e_.last_miss_count)
         marks.append(torch.cuda.Event(enable_timing=True))
         marks[-1].record()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t_) / (count * len(engines))
+        spans = []
+        for j in range(len(marks) - 1):
+            n_it = min(mark_every, count - j * mark_every)
+            if n_it > 0:
+                spans.append(marks[j].elapsed_time(marks[j + 1]) * 1e3 / (n_it * len(engines)))
+        return sec, sorted(spans), counts
 
-    timed_loop(a.warmup, a.steps, [eng] + others)
-    torch.cuda.synchronize()
-    elapsed = (time.perf_counter() - t0) / copies
-    kern_ms, launches = eng.ws.timing_read()
-    eng.ws.timing_enable(0)
-    # per-mark-interval time per layer-step (the last interval may be shorter)
-    spans = []
-    for j in range(len(marks) - 1):
-        n_it = min(mark_every, a.steps - j * mark_every)
-        if n_it > 0:
-            spans.append(marks[j].elapsed_time(marks[j + 1]) * 1e3 / (n_it * copies))
-    spans.sort()
+    engines = [eng] + others
+    pos = n_warm
+    eng.ws.select_stats(reset=True)
+    eng.ws.victim_stats(reset=True)
+    m_first = eng.lite_indices[eng.lite_len] - 1
+    sec_k, spans_k, counts_k = timed_loop(pos, a.steps, engines)
+    pos += a.steps
+    sec_v, spans, counts, n_value = sec_k, spans_k, counts_k, a.steps
+    if long_steps:
+        eng.ws.select_stats(reset=True)
+        eng.ws.victim_stats(reset=True)
+        m_first = eng.lite_indices[eng.lite_len] - 1
+        sec_v, spans, counts = timed_loop(pos, long_steps, engines)
+        pos += long_steps
+        n_value = long_steps
+    # statistics of the region that `value` comes from
+    sel_fast, sel_full = eng.ws.select_stats()
+    sel_short, sel_over = eng.ws.select_stats_detail()
+    host_rows = eng.ws.victim_stats()
+    m_last = eng.lite_indices[eng.lite_len] - 1
+    grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
 
     def pct(p_):
         return round(spans[min(len(spans) - 1, int(p_ * len(spans)))], 2) if spans else None
 
-    sel_fast, sel_full = eng.ws.select_stats()
-    sel_short, sel_over = eng.ws.select_stats_detail()
-    host_rows = eng.ws.victim_stats()
+    # Kernel time of the scan: a separate pass after the timed regions, every launch of the first copy between two
+    # HIP events (a pair delays its step by several microseconds, so none is inside a timed region).
+    kern_ms, launches = 0.0, 0
+    if ev_steps:
+        eng.ws.timing_enable(ev_steps, every=1)
+        timed_loop(pos, ev_steps, engines)
+        kern_ms, launches = eng.ws.timing_read()
+        eng.ws.timing_enable(0)
+        pos += ev_steps
     rows_scanned, rows_rescored = eng.ws.scan_stats()
     vic_on = eng.victim_rows_effective > 0 and a.fetch == "direct" and a.variant == "default"
-    grew = cap_before != (eng._A_K.capacity, eng.KVcpu.capacity)
-    m_last = eng.lite_indices[eng.lite_len] - 1
-    n_timed = len(counts)
 
     # the same state stepped back to back: its score index largely stays in the last-level cache
     warm_us = None
     if warm_steps:
-        marks.clear()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        timed_loop(a.warmup + a.steps, warm_steps, [eng])
-        torch.cuda.synchronize()
-        warm_us = (time.perf_counter() - t1) / warm_steps * 1e6
-    counts = counts[:n_timed]
+        warm_us = timed_loop(pos, warm_steps, [eng])[0] * 1e6
+        pos += warm_steps
 
     n_miss = int(torch.stack(counts).sum())
     n_sel = len(counts) * w.batch * w.num_heads * w.num_active_tokens
     e = 2 if w.dtype == torch.bfloat16 else 4
     row_bytes = 2 * w.head_dim * e
-    us_step = elapsed / a.steps * 1e6
+    us_step = sec_v * 1e6
     m_avg = (m_first + m_last) / 2.0
     bh = w.batch * w.num_heads
     scan_bytes = bh * m_avg * w.r * e            # what the reference's scan reads: r values per cached token and head
-    kern_us = kern_ms * 1e3 / max(launches, 1)
     n_act = w.num_active_tokens + w.lite_tokens
     step_bytes = (scan_bytes + (0 if a.no_attn else 2 * bh * n_act * w.head_dim * e) + bh * n_act * w.head_dim * e
                   + bh * n_act * w.r * e + 4 * bh * w.r * w.head_dim * e + 3 * bh * w.num_active_tokens * 4
-                  + n_miss / a.steps * row_bytes)
+                  + n_miss / n_value * row_bytes)
+
+    read_gbs = copy_gbs = pair_us = pair2_us = None
+    sweep = None
+    if a.probe_mb > 0:
+        read_gbs, copy_gbs = ops_mod.probe_bandwidth(min(a.probe_mb, 1024) << 20, 10, dev)
+        # what the same event bracket reads around one and around two kernels that do nothing
+        pair_us = ops_mod.probe_event_pair(64, dev)
+        pair2_us = ops_mod.probe_event_pair(64, dev, kernels=2)
+        if not a.no_probe_sweep:
+            table, _ = ops_mod.probe_read_sweep(a.probe_mb << 20, 5, dev)
+            best = max(table, key=table.get)
+            sweep = {"bytes": a.probe_mb << 20, "best_gbs": round(table[best], 1),
+                     "best": {"vectors_in_flight": best[0], "nontemporal": bool(best[1]), "workgroups_per_cu": best[2]},
+                     "gbs_by_in_flight_nontemporal_wg_per_cu": {f"{k[0]}/{k[1]}/{k[2]}": round(v, 0)
+                                                                for k, v in sorted(table.items())}}
+    # (between events: the profiler's duration of the same kernel is 2 to 3 us shorter; an empty kernel reads
+    # pair_us between the same events, and a second one adds as much again, so the share of the bracket that is
+    # not the kernel cannot be taken off by such a calibration)
+    kern_us = kern_ms * 1e3 / max(launches, 1)
 
     sidx_on = (not a.no_score_index) and w.r in (16, 32, 64)
     # Bytes one launch of the scan has to move.  Without the score index: the A_K rows.  With it: the 8-bit copy
@@ -501,15 +551,9 @@ def main():
     else:
         must_move = scan_bytes
     achieved = must_move / (kern_us * 1e-6) / 1e9 if launches else 0.0
-    traffic = MEASURED_TRAFFIC_BYTES.get((w.name, sidx_on)) \
+    tr = MEASURED_TRAFFIC.get((w.name, sidx_on)) \
         if a.context is None and a.variant == "default" and w.batch == 1 else None
-
-    read_gbs = copy_gbs = pair_us = None
-    if a.probe_mb > 0:
-        read_gbs, copy_gbs = ops_mod.probe_bandwidth(a.probe_mb << 20, 10, dev)
-        # what the same event bracket reads around a kernel that does nothing: the share of kernel_us that
-        # is the two event packets and the launch itself (a profiler's kernel duration has neither)
-        pair_us = ops_mod.probe_event_pair(64, dev)
+    traffic = tr["bytes"] if tr else None
 
     if a.calib_copy_mb > 0:
         src = torch.empty(a.calib_copy_mb << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -521,7 +565,7 @@ def main():
 
     cpu = None
     if a.cpu_steps > 0:
-        threads = a.cpu_threads or min(16, os.cpu_count() or 1)
+        threads, host = host_threads(a)
         torch.set_num_threads(threads)
         o, orc = oracle_from_engine(eng, w, threads)
         extra = [stream.next() for _ in range(a.cpu_steps + 1)]
@@ -538,52 +582,177 @@ def main():
         cpu = {"value": round(cpu_s * 1e6, 1), "unit": "us/layer-step", "cores": threads, "kind": "port",
                "sample": f"{a.cpu_steps} decode steps of the same workload continued from the GPU state "
                          f"(fp32 torch-CPU factor update + C scan/sort/diff/gather per head on {threads} threads)"}
+        cpu.update(host)
+
+    hit_rate = round(1.0 - n_miss / max(n_sel, 1), 4)
+    served = round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0
+    step_frac = round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+    # achieved = bytes the scan kernel has to move per launch (see must_move above) over its duration, so
+    # frac is a fraction of the HBM peak; algorithmic_equiv_gbs prices the same duration at the bytes the
+    # reference's scan reads (r values of the storage type per cached token and head), which the score
+    # index undercuts; traffic = HBM bytes per launch read from hardware counters (profiles/).
+    roof = {"bound": "hbm", "kernel": "score_prefilter_kernel" if sidx_on else "score_filter_kernel",
+            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": round(traffic) if traffic else None,
+            "traffic_gbs": round(traffic / (kern_us * 1e-6) / 1e9, 1) if traffic and launches else None,
+            "traffic_from": {k_: v_ for k_, v_ in tr.items() if k_ != "bytes"} if tr else None,
+            "kernel_us": round(kern_us, 2), "launches": launches,
+            "launches_timed_in": "a pass of %d steps after the timed regions" % ev_steps,
+            "bytes_per_launch": round(must_move),
+            "event_pair_around_empty_kernel_us": round(pair_us, 2) if pair_us is not None else None,
+            "event_pair_around_two_empty_kernels_us": round(pair2_us, 2) if pair2_us is not None else None,
+            "rows_rescored_per_launch": rows_rescored,
+            "algorithmic_bytes_per_launch": round(scan_bytes),
+            "algorithmic_equiv_gbs": round(scan_bytes / (kern_us * 1e-6) / 1e9, 1) if launches else None,
+            "measured_read_gbs": round(max(read_gbs or 0.0, sweep["best_gbs"] if sweep else 0.0), 1) or None,
+            "measured_read_gbs_default_probe": round(read_gbs, 1) if read_gbs else None,
+            "measured_copy_gbs": round(copy_gbs, 1) if copy_gbs else None,
+            "read_probe_sweep": sweep}
+    if compact:
+        for k_ in ("traffic_from", "read_probe_sweep", "measured_read_gbs", "measured_read_gbs_default_probe",
+                   "measured_copy_gbs", "event_pair_around_empty_kernel_us", "event_pair_around_two_empty_kernels_us",
+                   "traffic", "traffic_gbs", "launches_timed_in"):
+            roof.pop(k_, None)
+        return {"workload": f"{w.name}@{l}", "batch": w.batch, "layer_copies": copies, "steps": n_value,
+                "us_per_layer_step": round(us_step, 2), "us_per_sequence_layer_step": round(us_step / w.batch, 2),
+                "tokens_per_s_32_layers": round(w.batch * 1e6 / (32 * us_step), 2),
+                "step_algorithmic_bytes": round(step_bytes), "step_hbm_frac": step_frac,
+                "hit_rate": hit_rate, "victim_cache_served": served,
+                "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / n_value * row_bytes),
+                "roofline": roof, "cpu_baseline": cpu}
 
     out = {
         "metric": "lrqk_decode_us_per_layer_step", "value": round(us_step, 2), "unit": "us",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup_asked, "settle_steps": max(0, a.settle),
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_steps": max(0, a.settle),
         "ms_per_step": round(us_step / 1e3, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": f"{w.name}@{l}", "batch": w.batch, "heads": [w.num_heads, w.num_kv_heads],
                    "head_dim": w.head_dim, "r": w.r, "k": w.num_active_tokens, "lite": w.lite_tokens, "max_iter": list(w.max_iter),
                    "variant": a.variant, "fetch": a.fetch, "score_index": sidx_on, "attention_in_step": not a.no_attn, "candidates_m": [m_first, m_last],
+                   "factor_update": "fp64 from kept state" if a.factor_state else "fp32 over the active rows",
                    "layer_copies": copies,
                    "cache": "cold: %d copies of the layer state take turns, as the layers of a decoder do" % copies
                    if copies > 1 else "warm: one copy stepped back to back"},
+        # `value` is timed over value_timed_steps steps of every copy (at least --min-timed: a region of --steps 20
+        # lasts 7 ms); the region of exactly --steps steps ran first and is reported beside it
+        "value_timed_steps": n_value, "value_timed_layer_steps": n_value * copies,
+        "us_per_step_over_exactly_steps": round(sec_k * 1e6, 2),
         "us_per_step_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
         "us_per_step_one_copy_back_to_back": round(warm_us, 2) if warm_us else None,
         "us_per_sequence_layer_step": round(us_step / w.batch, 2),
         "tokens_per_s_32_layers": round(w.batch * 1e6 / (32 * us_step), 2),
-        "hit_rate": round(1.0 - n_miss / max(n_sel, 1), 4),
-        "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / a.steps * row_bytes),
-        "missed_bytes_per_step": round(n_miss / a.steps * row_bytes),
+        "hit_rate": hit_rate,
+        "h2d_bytes_per_step": round((host_rows if vic_on else n_miss) / n_value * row_bytes),
+        "missed_bytes_per_step": round(n_miss / n_value * row_bytes),
         "victim_cache": {"rows_per_head": eng.victim_rows_effective
                          if vic_on else 0,
-                         "served": round(1.0 - host_rows / max(n_miss, 1), 4) if vic_on else 0.0},
+                         "served": served},
         "step_algorithmic_bytes": round(step_bytes),
-        "step_hbm_frac": round(step_bytes / (us_step * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-        # achieved = bytes the scan kernel has to move per launch (see must_move above) over its duration, so
-        # frac is a fraction of the HBM peak; algorithmic_equiv_gbs prices the same duration at the bytes the
-        # reference's scan reads (r values of the storage type per cached token and head), which the score
-        # index undercuts; traffic = HBM bytes per launch read from hardware counters (profiles/).
-        "roofline": {"bound": "hbm", "kernel": "score_prefilter_kernel" if sidx_on else "score_filter_kernel",
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": round(traffic) if traffic else None,
-                     "traffic_gbs": round(traffic / (kern_us * 1e-6) / 1e9, 1) if traffic and launches else None,
-                     "kernel_us": round(kern_us, 2), "launches": launches, "bytes_per_launch": round(must_move),
-                     "event_pair_around_empty_kernel_us": round(pair_us, 2) if pair_us is not None else None,
-                     "rows_rescored_per_launch": rows_rescored,
-                     "algorithmic_bytes_per_launch": round(scan_bytes),
-                     "algorithmic_equiv_gbs": round(scan_bytes / (kern_us * 1e-6) / 1e9, 1) if launches else None,
-                     "measured_read_gbs": round(read_gbs, 1) if read_gbs else None,
-                     "measured_copy_gbs": round(copy_gbs, 1) if copy_gbs else None},
+        "step_hbm_frac": step_frac,
+        "roofline": roof,
         "selector_heads": {"from_candidate_list": sel_fast, "rescanned": sel_full, "list_short": sel_short,
                            "list_overflow": sel_over},
         "cpu_baseline": cpu,
         "prefill_s": round(prefill_s, 3), "setup_s": round(setup_s, 2), "buffers_grew_in_timed_region": grew,
     }
+    return out
+
+
+def also_results(a, t_start):
+    """The other configurations, compact, for the `also` key of the default line: 32K decode, four sequences stepped
+    together at 128K, the prefill factorisation, the full decoder.  Each runs after the one before it has freed its
+    buffers; one that fails leaves its error text in place of a result."""
+    import copy
+    import gc
+
+    def run(name, fn):
+        gc.collect()
+        torch.cuda.empty_cache()
+        if hasattr(torch._C, "_host_emptyCache"):
+            torch._C._host_emptyCache()  # pinned blocks of the earlier stores (the allocator keeps them otherwise)
+        free_b, total_b = torch.cuda.mem_get_info()
+        print(f"also.{name}: starts with {free_b / 2**30:.1f} of {total_b / 2**30:.1f} GiB of device memory free",
+              file=sys.stderr, flush=True)
+        t0 = time.perf_counter()
+        try:
+            res = fn()
+        except Exception as ex:  # the main line is still worth printing
+            import traceback
+            where = [f"{f.name}:{f.lineno}" for f in traceback.extract_tb(ex.__traceback__)[-4:]]
+            res = {"error": f"{type(ex).__name__}: {str(ex).splitlines()[0] if str(ex) else ''}", "at": where}
+        res["wall_s"] = round(time.perf_counter() - t0, 1)
+        print(f"also.{name}: {res['wall_s']} s", file=sys.stderr, flush=True)
+        return res
+
+    def sub(**kw):
+        b = copy.copy(a)
+        b.context, b.seqs, b.probe_mb, b.calib_copy_mb, b.warm_steps = None, 0, 0, 0, 0
+        for k_, v_ in kw.items():
+            setattr(b, k_, v_)
+        return b
+
+    out = {}
+    # 32K: eight copies take turns (four copies of its 36 MB index would all stay in the 256 MB last-level cache)
+    out["ctx32k"] = run("ctx32k", lambda: decode_bench(
+        sub(workload="llama8b_32k_bf16", steps=256, min_timed=256, warmup=16, settle=64, rotate=8, event_steps=32,
+            cpu_steps=min(a.cpu_steps, 32)), compact=True))
+    out["seqs4"] = run("seqs4", lambda: decode_bench(
+        sub(workload="llama8b_128k_bf16", seqs=4, steps=128, min_timed=128, warmup=16, settle=64, rotate=2,
+            event_steps=32, cpu_steps=min(a.cpu_steps, 8)), compact=True))
+
+    def pf():
+        r_ = prefill_als(sub(workload="llama8b_32k_prefill_als", steps=8, warmup=2, cpu_steps=min(a.cpu_steps, 1)))
+        roof = r_["roofline"]
+        return {"workload": r_["config"]["workload"], "ms": r_["value"], "rel_residual_K": r_["rel_residual_K"],
+                "rel_residual_Q": r_["rel_residual_Q"], "max_iter": r_["config"]["max_iter"],
+                "roofline": {k_: roof.get(k_) for k_ in ("bound", "achieved", "peak", "unit", "frac", "hbm_bytes_per_call",
+                                                          "executed_bf16_mfma_tflops", "executed_bf16_mfma_frac",
+                                                          "readings_of_the_long_axis")},
+                "cpu_baseline": r_["cpu_baseline"]}
+    out["prefill_als"] = run("prefill_als", pf)
+
+    if a.also_decoder and time.perf_counter() - t_start < a.also_budget_s:
+        def dec():
+            r_ = decoder(sub(layers=32, batch=4, prompt=65536, new_tokens=128, context_scale=5.0,
+                             cpu_steps=min(a.cpu_steps, 1)))
+            keep = ("value", "unit", "prefill_s", "decode_s", "us_per_layer_step", "last_step_hit_rate",
+                    "cache_path_us_per_layer_step", "other_us_per_layer_step", "cpu_baseline")
+            res = {k_: r_[k_] for k_ in keep}
+            res["workload"] = r_["config"]["workload"] + " x 4 sequences, 32 layers, 128 new tokens, context_scale 5"
+            return res
+        out["decoder"] = run("decoder", dec)
+    else:
+        out["decoder"] = {"skipped": "off (--no-also-decoder)" if not a.also_decoder else
+                          "the run had already taken %.0f s" % (time.perf_counter() - t_start)}
+    return out
+
+
+def main():
+    t_start = time.perf_counter()
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: the LRQK cache path has no multi-GPU part (heads shard trivially); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from lrqk_amd import _lib
+    _lib.load()  # fail loudly if the HIP library is missing
+    if a.mode == "prefill_als":
+        print(json.dumps(prefill_als(a)))
+        return
+    if a.mode == "decoder":
+        print(json.dumps(decoder(a)))
+        return
+    out = decode_bench(a)
+    plain = (a.workload == "llama8b_128k_bf16" and a.context is None and a.variant == "default" and not a.seqs
+             and not (a.rank or a.topk or a.lite or a.max_iter or a.data_rank) and not a.no_attn)
+    if a.also == "on" or (a.also == "auto" and plain):
+        out["also"] = also_results(a, t_start)
+    out["wall_s"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(out))
 
 

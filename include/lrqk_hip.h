@@ -269,10 +269,17 @@ int lrqk_timing_read(lrqk_ctx* ctx, double* total_ms, int* launches);
  * src, dst: device memory, 16-byte aligned, bytes a multiple of 16. */
 int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, int reps, double* read_ms, double* copy_ms,
                          void* stream);
-/* No counterpart in the reference.  What a pair of HIP events reads around a kernel that does nothing (average
- * microseconds over `reps` <= 256 pairs on the caller's stream, each pair between two other launches; waits for the
- * stream): the part of an event-bracketed kernel time (lrqk_timing_read) that is not the kernel. */
-int lrqk_probe_event_pair(int reps, double* pair_us, void* stream);
+/* Measurement helper (no counterpart in the reference): one variant of the plain read -- in_flight (4, 8 or 16)
+ * 16-byte vectors per thread, plain or non-temporal loads, grid_per_cu workgroups of 256 threads per CU -- for a
+ * sweep that looks for the best read rate of the GPU at hand.  sink: a few KB of device memory (never written in
+ * practice).  Waits for the stream. */
+int lrqk_probe_read_variant(const void* src, void* sink, int64_t bytes, int reps, int in_flight, int nontemporal,
+                            int grid_per_cu, double* read_ms, void* stream);
+/* No counterpart in the reference.  What a pair of HIP events reads around `kernels` (1..16) launches that do nothing
+ * (average microseconds over `reps` <= 256 pairs on the caller's stream, each pair between two other launches; waits
+ * for the stream).  The reading with one launch less the difference between two launches and one is the part of an
+ * event-bracketed kernel time (lrqk_timing_read) that is not the kernel. */
+int lrqk_probe_event_pair(int reps, int kernels, double* pair_us, void* stream);
 
 /* Host-side row gathers with the reference's native signatures (the staged fetch path
  * and API parity); multi-threaded memcpy.

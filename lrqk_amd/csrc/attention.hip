@@ -380,7 +380,12 @@ __device__ __forceinline__ void fetch_rows_attn_body(const uint4* __restrict__ s
             vic.pos[(int64_t)h * vic.cap + old[u]] = (int16_t)p_ins[u];
           }
         }
-        if (ok[u] && c == 0 && !from_fifo[u]) atomicAdd(&vic.host_rows[h], 1);
+      }
+      {  // statistics: rows taken from the host store (one addition per wave: additions to one line are served in turn)
+        int n_host = 0;
+#pragma unroll
+        for (int u = 0; u < kFR; ++u) n_host += __popcll(__ballot(ok[u] && c == 0 && !from_fifo[u]));
+        if (n_host && lane_id() == 0) atomicAdd(&vic.host_rows[h], n_host);
       }
       // the K rows that leave their slots, in the order of the miss list, for the kept sums of the factor update
       if (evk) {

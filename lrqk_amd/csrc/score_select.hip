@@ -153,12 +153,17 @@ __global__ __launch_bounds__(256) void arange_kernel(int32_t* out, int64_t out_s
 
 // Per-head selector state: t_low (key that had rank ~1.5k at the previous call), q_norm (|q_hat|
 // of that call), t_used / q_cur (bound and norm the filter of the current call used).
+// The per-head counters of the candidate lists take atomic additions from every workgroup of a scan: each sits in a
+// 128-byte line of its own (additions to one line are served one after the other, about 11 ns each, whichever
+// word of the line they name).
+constexpr int kCountStride = 32;
+
 struct SelState {
   uint32_t* t_low;
   float* q_norm;
   uint32_t* t_used;
   float* q_cur;
-  int* cand_count;
+  int* cand_count;   // [bh * kCountStride], element h * kCountStride
   int* level;        // slack of the carried bound per head (see bound_rank): level | calm calls << 8
   int* stats;
   int* rescored;     // per workgroup of the last index scan: rows whose bound passed (rescored exactly)
@@ -172,7 +177,7 @@ __global__ void init_select_state_kernel(SelState st, int bh) {
     st.q_norm[i] = 0.0f;
     st.t_used[i] = 0xffffffffu;
     st.q_cur[i] = 0.0f;
-    st.cand_count[i] = 0;
+    st.cand_count[i * kCountStride] = 0;
     st.level[i] = 0;
   }
   if (i < 3) st.stats[i] = 0;
@@ -204,7 +209,6 @@ constexpr int kFiltRPT = LRQK_FILT_RPT;  // rows per thread and tile
 #endif
 constexpr int kFiltTiles = LRQK_FILT_TILES;  // tiles per workgroup: one global list reservation for all of them
 constexpr int kFiltRows = kFiltThreads * kFiltRPT;
-constexpr int kPreCap = 2048;   // exact hits a prefilter workgroup can hold
 constexpr int kFiltMaxIt = 8;  // most iterations of the factor update whose pending iterate the filter can pick itself
 
 // Proxy query taken straight from the iterates of the factor update whose finish stage has not
@@ -320,7 +324,7 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
   __syncthreads();
   const int n = l_count;
   if (n == 0) return;
-  if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n);
+  if (tid == 0) g_base = atomicAdd(&st.cand_count[h * kCountStride], n);
   __syncthreads();
   const int gb = g_base;
   for (int j = tid; j < n; j += kFiltThreads) {
@@ -330,37 +334,69 @@ __global__ __launch_bounds__(kFiltThreads) void score_filter_kernel(const T* __r
 }
 
 // --------------------------------------------------------------------------- score + filter through the score index
-// Same output as score_filter_kernel (the candidate list of all rows with key >= bound), read from
+// Same output as score_filter_kernel (the candidate list of all rows with key >= bound, as a set), read from
 // the 8-bit copy of A_K in whitened coordinates: 34 bytes per row instead of 64.  Every wave solves
 // W q' = q (back substitution, lane i holds row i of W; q' ends up in scalar registers); for every
 // row an upper bound of its (rounded) score follows from the copy:
 //   |score - s~| <= D = scale * |q'|_1 * kSidxDFactor,   s~ = scale * sum_j (u_j - 128) q'_j
 //   round_bf16(score) <= s~ + D + (|s~| + D) / 256       (half a bf16 ulp)
 // Rows whose bound reaches the threshold (or is not a number) are rescored exactly from A_K; only
-// those that really pass enter the list.  Two LDS lists: "maybe" row ids, then the (key, id) pairs.
+// those that really pass enter the list.  Laid out for the memory system:
+//  * consecutive lanes read consecutive 16-byte vectors of the copy (a row of R bytes is shared by R / 16 lanes, which
+//    each keep the 16 elements of q' they need and add their partial sums across lanes), with non-temporal loads;
+//  * a wave works on steps of kScanU vectors per lane and requests the next step's vectors before it evaluates the
+//    current ones, so its loads never drain;
+//  * nothing is done per workgroup: every wave keeps its own list of rows to rescore and its own list of exact hits
+//    in LDS, rescoring 64 rows at a time while its next vectors are in flight, so that there is no barrier and
+//    no common phase in which every workgroup of the launch has stopped reading.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kScanU = 4;
+constexpr int kScanWaves = kFiltThreads / kWave;
+
 template <typename T, int R>
-__global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* __restrict__ a_k, int64_t head_stride,
-                                                                       const T* __restrict__ q_hat, int64_t m, int r,
-                                                                       int round_bf16, SelState st,
-                                                                       uint2* __restrict__ cand, int cand_cap,
-                                                                       FilterQ fq, ScoreIndexView six, int tiles_per_wg) {
+__global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(
+    const T* __restrict__ a_k, int64_t head_stride, const T* __restrict__ q_hat, int64_t m, int r, int round_bf16,
+    SelState st, uint2* __restrict__ cand, int cand_cap, FilterQ fq, ScoreIndexView six) {
   static_assert(R == 16 || R == 32 || R == 64, "the score index covers ranks 16, 32, 64");
-  // `maybe` takes the rows whose bound passes, `lc` the exact hits among them; both are emptied in
-  // between if a workgroup collects more than they hold.
-  __shared__ uint2 lc[kPreCap];
-  __shared__ uint32_t maybe[kFiltTiles * kFiltRows];
-  __shared__ int l_count, m_count, g_base;
+  constexpr int QV = R / 16;                  // lanes per row
+  constexpr int kRowsPerLoad = kWave / QV;    // rows that one load of a wave covers
+  constexpr int kStepRows = kRowsPerLoad * kScanU;
+  constexpr int kMaybeCap = kWave + kStepRows;
+  constexpr int kHitCap = 2 * kWave;
+  __shared__ uint32_t maybe_s[kScanWaves][kMaybeCap];
+  __shared__ uint2 hits_s[kScanWaves][kHitCap];
+  __shared__ __align__(16) float qx_s[kScanWaves][R];  // the proxy query as the exact score uses it (a copy per wave)
+  __shared__ int resc_s;
   const int h = blockIdx.y;
-  const int tid = threadIdx.x, lane = lane_id();
+  const int tid = threadIdx.x, lane = lane_id(), w = wave_id();
   const T* A = a_k + (int64_t)h * head_stride;
   const uint8_t* QA = six.qa + (int64_t)h * six.head_rows * R;
   const uint16_t* QS = six.qs + (int64_t)h * six.head_rows;
-  RowScorer<T, R> rs;
-  if (tid == 0) {
-    l_count = 0;
-    m_count = 0;
+  uint32_t* maybe = maybe_s[w];
+  uint2* hits = hits_s[w];
+  if (tid == 0) resc_s = 0;
+  const int sub = lane % QV;        // which 16 bytes of its row this lane reads
+  const int lrow = lane / QV;       // row of this lane within a load
+  const int64_t n_steps = (m + kStepRows - 1) / kStepRows;
+  const int64_t s_stride = (int64_t)gridDim.x * kScanWaves;
+  int64_t s_cur = (int64_t)blockIdx.x * kScanWaves + w;
+  const bool has_work = s_cur < n_steps;  // (wave-uniform)
+
+  u32x4_t buf[2][kScanU];
+  uint16_t scb[2][kScanU];
+  auto request = [&](int b, int64_t s) {
+#pragma unroll
+    for (int u = 0; u < kScanU; ++u) {
+      const int64_t row = min(s * kStepRows + u * kRowsPerLoad + lrow, m - 1);
+      buf[b][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(QA + row * R) + sub);
+      scb[b][u] = __builtin_nontemporal_load(QS + row);
+    }
+  };
+  if (has_work) {  // two steps are on their way while the proxy query is resolved
+    request(0, s_cur);
+    if (s_cur + s_stride < n_steps) request(1, s_cur + s_stride);
   }
-  __syncthreads();
+
   const uint32_t t_prev = st.t_low[h];
   const float qn_prev = st.q_norm[h];
   const bool pending = fq.iter_out != nullptr;
@@ -370,13 +406,13 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
 #pragma unroll
     for (int it = 0; it < kFiltMaxIt; ++it)
       oit[it] = fq.iter_out[((int64_t)h * fq.max_iter + min(it, fq.max_iter - 1)) * 2 * r + min(lane, r - 1)];
-  } else {
-    rs.init(q_hat + (int64_t)h * r, r, round_bf16);
   }
   // row `lane` of W and 1 / W_ll (lanes >= R repeat the last row; their results are never read)
   const float* Wm = six.wm + (int64_t)h * (R * R + R);
-  float wrow[R];
+  float qh[16];  // the 16 elements of q' that meet this lane's bytes
+  float qsum = 0.0f, ql1 = 0.0f, ql2 = 0.0f;
   {
+    float wrow[R];
     const float4* wp = reinterpret_cast<const float4*>(Wm + min(lane, R - 1) * R);
 #pragma unroll
     for (int c = 0; c < R / 4; ++c) {
@@ -386,36 +422,20 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
       wrow[4 * c + 2] = w4.z;
       wrow[4 * c + 3] = w4.w;
     }
-  }
-  const float dinv = Wm[R * R + min(lane, R - 1)];
-  float q_lane = 0.0f;  // element `lane` of the proxy query as the exact score uses it
-  if (!pending) q_lane = ld_f32<T>(q_hat, (int64_t)h * r + min(lane, R - 1));
-  // the first rows of the copy are requested before the proxy query is resolved
-  constexpr int kPre = 2;
-  constexpr int QV = R / 16;  // 16-byte vectors per 8-bit row
-  const int64_t base0 = (int64_t)blockIdx.x * tiles_per_wg * kFiltRows;
-  uint4 pre[kPre][QV];
-  uint16_t pre_s[kPre];  // (as stored: converting here would wait for the loads before the query is resolved)
+    const float dinv = Wm[R * R + min(lane, R - 1)];
+    float q_lane = 0.0f;  // element `lane` of the proxy query as the exact score uses it
+    if (!pending) q_lane = ld_f32<T>(q_hat, (int64_t)h * r + min(lane, R - 1));
+    if (pending) {
+      const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
+      float qv = oit[0];
 #pragma unroll
-  for (int it = 0; it < kPre; ++it) {
-    const int64_t i = min(base0 + it * kFiltThreads + tid, m - 1);
-#pragma unroll
-    for (int c = 0; c < QV; ++c) pre[it][c] = reinterpret_cast<const uint4*>(QA + i * R)[c];
-    pre_s[it] = QS[i];
-  }
-  if (pending) {
-    const int chosen = als_decide<kFiltMaxIt>(sacc, fq.bh, fq.max_iter, r, fq.tol);
-    float qv = oit[0];
-#pragma unroll
-    for (int it = 1; it < kFiltMaxIt; ++it) qv = chosen == it ? oit[it] : qv;
-    if (blockIdx.x == 0 && tid < r) st_f32<T>((T*)fq.q_hat_out, (int64_t)h * r + tid, qv);
-    rs.init_from_lanes(qv, r, round_bf16);
-    q_lane = sizeof(T) == 2 ? round_to_bf16_f32(qv) : qv;
-  }
-  // q' from W q' = q, last unknown first; lane i keeps the residual of equation i
-  float qc[R];
-  float qsum = 0.0f, ql1 = 0.0f, ql2 = 0.0f;
-  {
+      for (int it = 1; it < kFiltMaxIt; ++it) qv = chosen == it ? oit[it] : qv;
+      if (blockIdx.x == 0 && tid < r) st_f32<T>((T*)fq.q_hat_out, (int64_t)h * r + tid, qv);
+      q_lane = sizeof(T) == 2 ? round_to_bf16_f32(qv) : qv;
+    }
+    if (lane < R) qx_s[w][lane] = lane < r ? q_lane : 0.0f;
+    // q' from W q' = q, last unknown first; lane i keeps the residual of equation i
+    float qc[R];
     float resid = q_lane;
 #pragma unroll
     for (int j = R - 1; j >= 0; --j) {
@@ -429,10 +449,14 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
       ql1 += fabsf(qc[j]);
       ql2 = fmaf(qc[j], qc[j], ql2);
     }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      float x = qc[e];
+#pragma unroll
+      for (int c = 1; c < QV; ++c) x = sub == c ? qc[c * 16 + e] : x;
+      qh[e] = x;
+    }
   }
-  // The rows are white in the index's coordinates, so the scores of a head spread like |q'|, whatever
-  // the direction of the proxy query: the carried bound follows that norm (the plain scan, which has
-  // no transform, follows |q_hat|).
   const float qn = sqrtf(ql2);
   const uint32_t tl = rescaled_bound(t_prev, qn_prev, qn, round_bf16);
   if (tid == 0 && blockIdx.x == 0) {
@@ -440,123 +464,124 @@ __global__ __launch_bounds__(kFiltThreads) void score_prefilter_kernel(const T* 
     st.q_cur[h] = qn;
   }
   const float dfac = ql1 * kSidxDFactor;
-  // float threshold; an unset bound (no key passes) keeps the list empty exactly like the plain filter
   const bool any = tl != 0xffffffffu;
   const float thr = key_score(tl);
   const float thr_lo = thr - fabsf(thr) * 1e-6f;
-  auto bound_of = [&](const uint4 (&row)[QV], float scale) {
-    float t = 0.0f;
-#pragma unroll
-    for (int c = 0; c < QV; ++c) {
-      const uint32_t w[4] = {row[c].x, row[c].y, row[c].z, row[c].w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        t = fmaf((float)((w[e] >> 0) & 0xffu), qc[c * 16 + e * 4 + 0], t);
-        t = fmaf((float)((w[e] >> 8) & 0xffu), qc[c * 16 + e * 4 + 1], t);
-        t = fmaf((float)((w[e] >> 16) & 0xffu), qc[c * 16 + e * 4 + 2], t);
-        t = fmaf((float)((w[e] >> 24) & 0xffu), qc[c * 16 + e * 4 + 3], t);
-      }
-    }
-    const float sa = scale * (t - 128.0f * qsum);
-    const float dd = scale * dfac;
-    return sa + dd + (fabsf(sa) + dd) * (1.0f / 256.0f);
+  __syncthreads();  // (resc_s is zero)
+
+  int n_maybe = 0, n_hits = 0, n_resc = 0;  // (wave-uniform)
+  auto lds_wave_sync = [&]() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
-  // the exact hits collected in lc go to the head's list (one reservation per call)
-  auto flush_hits = [&](bool last) {
-    const int n = l_count;  // (uniform: a barrier precedes every call)
-    if (n == 0) return;
-    if (tid == 0) g_base = atomicAdd(&st.cand_count[h], n);
-    __syncthreads();
-    const int gb = g_base;
-    for (int j = tid; j < n; j += kFiltThreads) {
+  // this wave's exact hits go to the head's list
+  auto flush_hits = [&]() {
+    if (n_hits == 0) return;
+    int gb = 0;
+    if (lane == 0) gb = atomicAdd(&st.cand_count[h * kCountStride], n_hits);
+    gb = __builtin_amdgcn_readfirstlane(gb);
+    lds_wave_sync();
+    for (int j = lane; j < n_hits; j += kWave) {
       const int p = gb + j;
-      if (p < cand_cap) cand[(int64_t)h * cand_cap + p] = lc[j];  // (beyond the capacity the count alone tells the select kernel)
+      if (p < cand_cap) cand[(int64_t)h * cand_cap + p] = hits[j];  // (beyond the capacity the count alone tells the select kernel)
     }
-    if (!last) {
-      __syncthreads();
-      if (tid == 0) l_count = 0;
-      __syncthreads();
-    }
+    lds_wave_sync();
+    n_hits = 0;
   };
-  // exact scores of the collected rows; the ones that really pass go to lc, which is emptied
-  // whenever kPreCap rows have been looked at (so it cannot overflow)
+  // exact scores of the last (up to) 64 rows of this wave's list
   auto rescore = [&]() {
-    const int nm = m_count;
-    for (int j0 = 0; j0 < nm; j0 += kFiltThreads) {
-      if (j0 > 0 && j0 % kPreCap == 0) {  // (uniform)
-        __syncthreads();
-        flush_hits(false);
-      }
-      const int j = j0 + tid;
-      const uint32_t i = maybe[min(j, nm - 1)];
-      const uint32_t key = score_key(rs.score(A, (int64_t)i));  // unconditional load (clamped), masked below
-      const bool hit = j < nm && key >= tl;
-      int wt;
-      const int rk = wave_rank(hit, wt);
-      if (wt) {
-        int wbase = 0;
-        if (lane == 0) wbase = atomicAdd(&l_count, wt);
-        wbase = __shfl(wbase, 0, kWave);
-        if (hit) lc[wbase + rk] = make_uint2(key, i);
+    const int take = min(n_maybe, kWave);
+    const int first = n_maybe - take;
+    lds_wave_sync();
+    const uint32_t i = maybe[first + min(lane, take - 1)];
+    // the exact score of row i: the chain of RowScorer::score, with the query read from LDS (unconditional load,
+    // masked below)
+    constexpr int VEC = Vec16<T>::N;
+    Vec16<T> xv[R / VEC];
+#pragma unroll
+    for (int c = 0; c < R / VEC; ++c) xv[c].load(A + (int64_t)i * R + c * VEC);
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < R / VEC; ++c) {
+      float f[VEC];
+      xv[c].unpack(f);
+#pragma unroll
+      for (int e4 = 0; e4 < VEC / 4; ++e4) {
+        const float4 q4 = reinterpret_cast<const float4*>(qx_s[w])[(c * VEC) / 4 + e4];
+        acc = __builtin_fmaf(f[4 * e4 + 0], q4.x, acc);
+        acc = __builtin_fmaf(f[4 * e4 + 1], q4.y, acc);
+        acc = __builtin_fmaf(f[4 * e4 + 2], q4.z, acc);
+        acc = __builtin_fmaf(f[4 * e4 + 3], q4.w, acc);
       }
     }
-    __syncthreads();
+    if (round_bf16) acc = round_to_bf16_f32(acc);
+    if (acc == 0.0f) acc = 0.0f;
+    const uint32_t key = score_key(acc);
+    const bool hit = lane < take && key >= tl;
+    int wt;
+    const int rk = wave_rank(hit, wt);
+    if (hit) hits[n_hits + rk] = make_uint2(key, i);
+    n_hits += wt;
+    n_maybe = first;
+    n_resc += take;
+    if (n_hits > kHitCap - kWave) flush_hits();
   };
-  // A workgroup takes tiles_per_wg consecutive tiles (2 unless the context is so long that the launch
-  // would otherwise hold more workgroups than the GPU does at a time).
-  int resc_total = 0;  // (thread 0) rows handed to the exact rescoring so far
-#pragma unroll 1
-  for (int tile = 0; tile < tiles_per_wg; ++tile) {
-    const int64_t base = base0 + (int64_t)tile * kFiltRows;
-    if (base >= m) break;
-    if (tile >= kFiltTiles) {  // (uniform) long contexts only: make room in the list if the next tile might not fit
-      __syncthreads();
-      if (m_count > kFiltTiles * kFiltRows - kFiltRows) {
-        rescore();
-        flush_hits(false);
-        if (tid == 0) {
-          resc_total += m_count;
-          m_count = 0;
-        }
-        __syncthreads();
-      }
-    }
+  auto evaluate = [&](int b, int64_t s) {
     uint32_t mask = 0;
 #pragma unroll
-    for (int it = 0; it < kFiltRPT; ++it) {
-      const int64_t i = base + it * kFiltThreads + tid;
-      float ub;
-      if (tile == 0 && it < kPre) {
-        ub = bound_of(pre[it < kPre ? it : 0], sidx_scale_from_bits(pre_s[it < kPre ? it : 0]));
-      } else {
-        const int64_t ic = min(i, m - 1);
-        uint4 row[QV];
+    for (int u = 0; u < kScanU; ++u) {
+      const uint32_t wv[4] = {buf[b][u].x, buf[b][u].y, buf[b][u].z, buf[b][u].w};
+      float t = 0.0f;
 #pragma unroll
-        for (int c = 0; c < QV; ++c) row[c] = reinterpret_cast<const uint4*>(QA + ic * R)[c];
-        ub = bound_of(row, sidx_scale_from_bits(QS[ic]));
+      for (int e = 0; e < 4; ++e) {
+        t = fmaf((float)((wv[e] >> 0) & 0xffu), qh[e * 4 + 0], t);
+        t = fmaf((float)((wv[e] >> 8) & 0xffu), qh[e * 4 + 1], t);
+        t = fmaf((float)((wv[e] >> 16) & 0xffu), qh[e * 4 + 2], t);
+        t = fmaf((float)((wv[e] >> 24) & 0xffu), qh[e * 4 + 3], t);
       }
-      if (any && i < m && !(ub < thr_lo)) mask |= 1u << it;
+      t = group_sum(t, QV);
+      const float scale = sidx_scale_from_bits(scb[b][u]);
+      const float sa = scale * (t - 128.0f * qsum);
+      const float dd = scale * dfac;
+      const float ub = sa + dd + (fabsf(sa) + dd) * (1.0f / 256.0f);
+      const int64_t row = s * kStepRows + u * kRowsPerLoad + lrow;
+      if (any && sub == 0 && row < m && !(ub < thr_lo)) mask |= 1u << u;
     }
     const int cnt = __popc(mask);
     const int incl = wave_inclusive_sum(cnt);
-    const int wtot = __shfl(incl, kWave - 1, kWave);
+    const int wtot = __builtin_amdgcn_readlane(incl, kWave - 1);
     if (wtot) {
-      int wbase = 0;
-      if (lane == kWave - 1) wbase = atomicAdd(&m_count, wtot);
-      wbase = __shfl(wbase, kWave - 1, kWave);
-      int pos = wbase + incl - cnt;
+      int pos = n_maybe + incl - cnt;
 #pragma unroll
-      for (int it = 0; it < kFiltRPT; ++it)
-        if ((mask >> it) & 1u) maybe[pos++] = (uint32_t)(base + it * kFiltThreads + tid);
+      for (int u = 0; u < kScanU; ++u)
+        if ((mask >> u) & 1u) maybe[pos++] = (uint32_t)(s * kStepRows + u * kRowsPerLoad + lrow);
+      n_maybe += wtot;
     }
+  };
+  if (has_work) {
+    // evaluate a step, ask for the step after the next into the registers it leaves, then rescore what has gathered
+    while (true) {
+      evaluate(0, s_cur);
+      if (s_cur + 2 * s_stride < n_steps) request(0, s_cur + 2 * s_stride);
+      while (n_maybe >= kWave) rescore();
+      s_cur += s_stride;
+      if (s_cur >= n_steps) break;
+      evaluate(1, s_cur);
+      if (s_cur + 2 * s_stride < n_steps) request(1, s_cur + 2 * s_stride);
+      while (n_maybe >= kWave) rescore();
+      s_cur += s_stride;
+      if (s_cur >= n_steps) break;
+    }
+    if (n_maybe > 0) rescore();
+    flush_hits();
+    if (lane == 0 && n_resc) atomicAdd(&resc_s, n_resc);
   }
   __syncthreads();
   if (tid == 0) {
     const int slot = h * (int)gridDim.x + (int)blockIdx.x;
-    if (slot < st.rescored_cap) st.rescored[slot] = resc_total + m_count;
+    if (slot < st.rescored_cap) st.rescored[slot] = resc_s;
   }
-  rescore();
-  flush_hits(true);
 }
 
 // --------------------------------------------------------------------------- select (+ diff)
@@ -751,9 +776,9 @@ __device__ __forceinline__ void select_generic(const SelLds& L, int mode, const 
   int64_t N = m;
   uint32_t lo = 0;
   if (mode == 0) {
-    if (tid == 0 && n_list < 0) s_n = st.cand_count[h];
+    if (tid == 0 && n_list < 0) s_n = st.cand_count[h * kCountStride];
     __syncthreads();
-    if (tid == 0) st.cand_count[h] = 0;  // re-arm for the next call (every thread has read the count by now)
+    if (tid == 0) st.cand_count[h * kCountStride] = 0;  // re-arm for the next call (every thread has read the count by now)
     const int n = n_list < 0 ? s_n : n_list;
     fast = n >= k && n <= cand_cap;
     if (fast) {
@@ -1436,7 +1461,7 @@ __device__ __forceinline__ void select_step_fast(const SelLds& L, const uint2* _
       df.vic_ptr[h] = (base + min(n_pair, df.vic_nv)) % df.vic_nv;
     }
     if (df.miss_count) df.miss_count[h] = n_pair;
-    st.cand_count[h] = 0;  // re-arm for the next call
+    st.cand_count[h * kCountStride] = 0;  // re-arm for the next call
   }
 }
 
@@ -1458,7 +1483,7 @@ __global__ __launch_bounds__(kSelThreads) void select_step_kernel(const uint2* _
                                                                   DiffArgs df) {
   LRQK_SEL_LDS(L);
   const int h = blockIdx.x;
-  const int n = __builtin_amdgcn_readfirstlane(st.cand_count[h]);
+  const int n = __builtin_amdgcn_readfirstlane(st.cand_count[h * kCountStride]);
   const int lvl = __builtin_amdgcn_readfirstlane(st.level[h]);
   const bool fast = n >= k && n <= cand_cap && n <= 16 * kSelThreads;
   int level = lvl & 0xff, calm = lvl >> 8;
@@ -1534,17 +1559,19 @@ static int prepare_select(lrqk_ctx* ctx, int bh, int64_t m, int topk, hipStream_
   sb->cand_cap = 8 * topk < 4096 ? 4096 : 8 * topk;  // (the register-resident paths take up to 8192 and 16384 entries)
   if ((rc = ctx->cand.ensure((size_t)bh * sb->cand_cap * sizeof(uint2)))) return rc;
   sb->cand = (uint2*)ctx->cand.p;
-  // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | cand_count i32 [bh] | level i32 [bh] |
-  // stats i32 [3]: served from the list, rescans because the list was too short, because it overflowed
+  // layout: t_low u32 [bh] | q_norm f32 [bh] | t_used u32 [bh] | q_cur f32 [bh] | (unused) [bh] | level i32 [bh] |
+  // stats i32 [3]: served from the list, rescans because the list was too short, because it overflowed |
+  // rescored i32 [bh + kRescSlots] | cand_count i32 [bh * kCountStride] on a 128-byte boundary
   void* before = ctx->cand_cnt.p;
   constexpr int kRescSlots = 8192;  // workgroups of one index scan (never more than the GPU holds at a time)
-  if ((rc = ctx->cand_cnt.ensure((size_t)(6 * bh + 3 + bh + kRescSlots) * 4))) return rc;
+  const size_t count_at = ((size_t)(6 * bh + 3 + bh + kRescSlots) + 31) & ~(size_t)31;  // (in words)
+  if ((rc = ctx->cand_cnt.ensure((count_at + (size_t)bh * kCountStride) * 4))) return rc;
   uint32_t* base = (uint32_t*)ctx->cand_cnt.p;
   sb->st.t_low = base;
   sb->st.q_norm = (float*)(base + bh);
   sb->st.t_used = base + 2 * bh;
   sb->st.q_cur = (float*)(base + 3 * bh);
-  sb->st.cand_count = (int*)(base + 4 * bh);
+  sb->st.cand_count = (int*)(base + count_at);
   sb->st.level = (int*)(base + 5 * bh);
   sb->st.stats = (int*)(base + 6 * bh);
   sb->st.rescored = (int*)(base + 6 * bh + 3);
@@ -1613,27 +1640,29 @@ static int launch_filter_select(lrqk_ctx* ctx, const SelectBufs& sb, const void*
     const int ri = score_index_prepare(ctx, a_k, head_stride, bh, m, r, sizeof(T) == 4 ? LRQK_F32 : LRQK_BF16, st, &six);
     if (ri < 0) return ri;
     if (ri == 1) {
-      // no more workgroups than the GPU holds at a time: beyond that a workgroup takes more tiles
+      // As many workgroups as the GPU holds at a time, shared out over the heads: every wave then runs once, from
+      // the first row to the last (a second round of workgroups would pay the solve for q' and the final
+      // rescoring again, with the memory idle meanwhile).
       static std::atomic<int> slots_dev[kMaxDeviceSlots];
       std::atomic<int>& slots_a = slots_dev[per_device_slot()];
       int slots = slots_a;
       if (slots == 0) {
         int per_cu = 0, dev = 0, n_cu = 0;
-        LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, score_prefilter_kernel<T, R>, kFiltThreads, 0));
+        LRQK_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, score_prefilter_kernel<T, R>,
+                                                                    kFiltThreads, 0));
         LRQK_HIP_CHECK(hipGetDevice(&dev));
         LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
         slots = std::max(1, per_cu * n_cu);
         slots_a = slots;
       }
-      const int64_t tiles = (m + kFiltRows - 1) / kFiltRows;
-      const int64_t wgs = std::max<int64_t>(1, std::min<int64_t>((tiles + kFiltTiles - 1) / kFiltTiles, slots / bh));
-      const int tiles_per_wg = (int)std::max<int64_t>(kFiltTiles, (tiles + wgs - 1) / wgs);
-      dim3 grid_ix((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)bh);
-      hipLaunchKernelGGL((score_prefilter_kernel<T, R>), grid_ix, dim3(kFiltThreads), 0, st, (const T*)a_k,
-                         head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six,
-                         tiles_per_wg);
+      constexpr int kStepRowsWg = (kWave / (R / 16)) * kScanU * kScanWaves;  // rows one step of a workgroup's waves covers
+      const int64_t need = (m + kStepRowsWg - 1) / kStepRowsWg;
+      const int64_t wgs = std::max<int64_t>(1, std::min<int64_t>(need, slots / bh));
+      dim3 grid_st((unsigned)wgs, (unsigned)bh);
+      hipLaunchKernelGGL((score_prefilter_kernel<T, R>), grid_st, dim3(kFiltThreads), 0, st, (const T*)a_k,
+                         head_stride, (const T*)q_hat, m, r, round_bf16, sb.st, sb.cand, sb.cand_cap, fq, six);
       via_index = true;
-      ctx->scan_wgs = (int)std::min<int64_t>((int64_t)grid_ix.x * bh, sb.st.rescored_cap);
+      ctx->scan_wgs = (int)std::min<int64_t>((int64_t)grid_st.x * bh, sb.st.rescored_cap);
       ctx->scan_rows = (int64_t)bh * m;
     }
   }

@@ -395,11 +395,29 @@ def probe_bandwidth(nbytes: int, reps: int = 10, device="cuda:0"):
     return nbytes / (r_ms.value * 1e-3) / 1e9, 2 * nbytes / (c_ms.value * 1e-3) / 1e9
 
 
-def probe_event_pair(reps: int = 64, device="cuda:0") -> float:
-    """Microseconds that a pair of HIP events reads around a kernel that does nothing (average of ``reps`` pairs)."""
+def probe_read_sweep(nbytes: int, reps: int = 5, device="cuda:0"):
+    """The plain read over ``nbytes`` in every variant (4 / 8 / 16 vectors in flight, plain / non-temporal loads,
+    1 .. 8 workgroups per CU): ({(in_flight, nontemporal, grid_per_cu): GB/s}, best GB/s)."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device=device).fill_(1)
+    sink = torch.zeros(1 << 16, dtype=torch.uint8, device=device)
+    table = {}
+    ms = ctypes.c_double()
+    for nt in (0, 1):
+        for fl in (4, 8, 16):
+            for per_cu in (1, 2, 4, 8):
+                check(_lib.load().lrqk_probe_read_variant(src.data_ptr(), sink.data_ptr(), nbytes, reps, fl, nt, per_cu,
+                                                          ctypes.byref(ms), _stream(src)))
+                table[(fl, nt, per_cu)] = nbytes / (ms.value * 1e-3) / 1e9
+    return table, max(table.values())
+
+
+def probe_event_pair(reps: int = 64, device="cuda:0", kernels: int = 1) -> float:
+    """Microseconds that a pair of HIP events reads around ``kernels`` launches that do nothing (average of ``reps``
+    pairs)."""
     us = ctypes.c_double()
     with torch.cuda.device(device):
-        check(_lib.load().lrqk_probe_event_pair(reps, ctypes.byref(us), torch.cuda.current_stream().cuda_stream))
+        check(_lib.load().lrqk_probe_event_pair(reps, kernels, ctypes.byref(us),
+                                                torch.cuda.current_stream().cuda_stream))
     return us.value
 
 

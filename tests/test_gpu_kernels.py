@@ -831,5 +831,13 @@ def test_measurement_probes(ops):
     assert 50.0 < read_gbs < 20000.0 and 50.0 < copy_gbs < 20000.0, (read_gbs, copy_gbs)
     pair = ops.probe_event_pair(16, DEV)
     assert 0.0 < pair < 500.0, pair
+    pair2 = ops.probe_event_pair(16, DEV, kernels=2)
+    assert pair < pair2 + 5.0 < 505.0, (pair, pair2)
     with pytest.raises(ValueError):
         ops.probe_event_pair(0, DEV)
+    with pytest.raises(ValueError):
+        ops.probe_event_pair(4, DEV, kernels=0)
+    # every variant of the read sweep runs and reads a plausible rate (ragged size: the last vectors are clamped)
+    table, best = ops.probe_read_sweep((64 << 20) + 4096 + 16, 2, DEV)
+    assert len(table) == 24 and all(50.0 < v < 20000.0 for v in table.values()), table
+    assert best == max(table.values())
