@@ -22,6 +22,7 @@
 #include "common.hpp"
 #include "ctx.hpp"
 #include "als_finish.hpp"
+#include "als_gram.hpp"
 #include "small_inverse.hpp"
 
 namespace lrqk {
@@ -32,19 +33,6 @@ constexpr int kGramChunk = 32;  // tokens per wave per chunk = 16 MFMA steps
 constexpr int kGramNe = 32 * 32 + 32;
 constexpr int kSolveThreads = 256;
 
-
-// Ring append folded into the Gram pass: slot `slot` (>= 0) of every head is the new token.  The
-// pass takes its K row from k_new and its token id from `token` instead of the buffers, and the
-// wave that owns the slot writes k_new, v_new and the id into them.
-struct GramAppend {
-  const void* k_new;  // [b][hkv][d]
-  const void* v_new;  // [b][hkv][d]
-  void* v_act;        // [bh][kprev_slots][d]
-  int32_t* idx_out;   // active_idx, writable
-  int slot;           // -1: nothing to append
-  int32_t token;
-  int hq, hkv;
-};
 
 // Everything the solve needs from B_Q, B_K, q and the new k -- B_Q B_Q^T and B_K B_K^T (four 32 x 32
 // MFMA tiles: matrix x half of the d axis), q B_Q^T, k B_K^T and q . k -- does not depend on the Gram
@@ -589,8 +577,9 @@ __global__ __launch_bounds__(kSolveThreads, KS <= 16 ? 2 : 1) void als_solve_ker
 }
 
 // ----------------------------------------------------------------------------- ranks beyond one matrix-core tile
-// 32 < r <= 64 (the reference's "accuracy-focused" setting is r = 64, README.md:126): the same two launches in plain
-// fp32 arithmetic, not tuned -- sums over the active rows, then one workgroup per head that forms G_K, G_Q, inverts
+// 32 < r <= 64 (the reference's "accuracy-focused" setting is r = 64, README.md:126) for the shapes that the
+// matrix-core kernels of als_decode_r64.hip do not take (fp32 storage, rows other than 128 elements, ranks that are
+// not multiples of 8): the same two launches in plain fp32 arithmetic, not tuned -- sums over the active rows, then one workgroup per head that forms G_K, G_Q, inverts
 // them (Gauss-Jordan on the matrix scaled to unit diagonal, no pivoting: symmetric positive definite) and runs the
 // alternating rank-1 solves with the formulas of als_solve_kernel.  Same outputs (iter_out, deltas), so the finish
 // stage and the scan take over from there unchanged.
@@ -1038,9 +1027,29 @@ static int als_decode_impl(lrqk_ctx* ctx, void* b_q, void* b_k, void* a_k, int64
     int rc = ctx->als_part.ensure((size_t)bh * S * ne * sizeof(float));
     if (rc) return rc;
     if ((rc = ctx->als_iter.ensure((size_t)bh * max_iter * (2 * r + 1) * sizeof(float)))) return rc;
-    float* part = (float*)ctx->als_part.p;
     float* iter_out = (float*)ctx->als_iter.p;
     float* deltas = iter_out + (size_t)bh * max_iter * 2 * r;
+    if (als_r64_supported(sizeof(T) == 2 ? LRQK_BF16 : LRQK_F32, r, d, a_k, head_stride)) {
+      // bf16 rows of 128 elements: both launches on the matrix cores
+      float* kq_out = nullptr;
+      if (defer_finish && ap.slot >= 0 && n == kprev_slots) {
+        if ((rc = ctx->als_kq.ensure((size_t)bh * n * sizeof(float)))) return rc;
+        kq_out = (float*)ctx->als_kq.p;
+      }
+      if ((rc = als_r64_update(ctx, b_q, b_k, a_k, head_stride, active_idx, idx_stride, (void*)k_prev, kprev_slots, n, q,
+                               k_new, bh, hq, hkv, r, max_iter, iter_out, deltas, ap, kq_out, st)))
+        return rc;
+      if (kq_out) {
+        ctx->kq_valid = true;
+        ctx->kq_k_act = k_prev;
+        ctx->kq_q = q;
+        ctx->kq_bh = bh;
+        ctx->kq_n = n;
+      }
+      return als_decode_finish<T>(ctx, b_q, b_k, a_k, head_stride, q, k_new, bh, hq, hkv, r, d, lpr_log2, max_iter, tol,
+                                  q_hat, k_hat, append_row, iter_out, deltas, defer_finish, st);
+    }
+    float* part = (float*)ctx->als_part.p;
     const size_t smem_g = ((size_t)kWideTile * (kWideMaxR + 4) + kWideTile + d) * sizeof(float);
     const size_t smem_s = ((size_t)2 * d * (kWideMaxR + 4) + (size_t)2 * kWideMaxR * (kWideMaxR + 1) + 2 * d + 18 * kWideMaxR) * sizeof(float);
     LRQK_REQUIRE(smem_s <= (size_t)160 * 1024 - 256, LRQK_ELIMIT, "r=%d with rows of %d elements needs too much LDS", r, d);

@@ -655,8 +655,8 @@ def test_long_run_with_wrapping_caches(lrqk, oracle):
 
 def test_accuracy_focused_setting(lrqk, oracle):
     """The reference's "accuracy-focused" setting (README.md:124-131: r 64, 4096 active tokens, 128 recent ones,
-    tol 1e-10, four iterations) at a reduced context: ranks beyond 32 run the general factor-update kernels, the
-    scan its rank-64 form with the score index."""
+    tol 1e-10, four iterations) at a reduced context: bf16 rows of 128 elements at ranks 33..64 run the factor
+    update on 2 x 2 matrix-core tiles, the scan its rank-64 form with the score index."""
     _say("accuracy-focused setting")
     _, _, n = _lockstep(lrqk, oracle, b=1, hq=4, hkv=2, d=128, l=9000, r=64, k=4096, L=128, steps=16,
                         dtype=torch.bfloat16, max_iter=(4, 4), tol=(1e-10, 1e-10), rho=96, capacity=16384, tag="r64",
@@ -675,7 +675,8 @@ def test_wide_rank_through_the_prefix_branch(lrqk, oracle):
 
 @pytest.mark.parametrize("r", [40, 48])
 def test_ranks_between_the_tuned_ones(lrqk, oracle, r):
-    """Ranks 40 and 48: the general factor-update kernels and the plain scan (the score index covers 16, 32, 64)."""
+    """Ranks 40 and 48: the factor update on 2 x 2 matrix-core tiles (zero-padded to 64) and the plain scan (the
+    score index covers 16, 32, 64)."""
     _say("rank", r)
     _, _, n = _lockstep(lrqk, oracle, b=2, hq=4, hkv=2, d=128, l=1500, r=r, k=256, L=16, steps=20,
                         dtype=torch.bfloat16, max_iter=(2, 2), tol=(1e-8, 1e-8), rho=2 * r, capacity=2048, tag="r%d" % r)

@@ -552,7 +552,8 @@ def _als_inputs(g, b, hq, hkv, n, d, r, cap, dtype):
                                                 # head widths 64 and 256 (bf16 rows that the d = 128 kernel does not take)
                                                 (torch.bfloat16, 8, 2, 300, 64, 16), (torch.bfloat16, 4, 1, 272, 256, 32),
                                                 (torch.float32, 4, 2, 150, 64, 8),
-                                                # ranks beyond 32 (the general kernels): 64, 48 and 40
+                                                # ranks beyond 32: 64 and 40 (bf16 rows of 128 elements: 2 x 2 matrix-core
+                                                # tiles), 48 in fp32 (the general kernels)
                                                 (torch.bfloat16, 8, 2, 600, 128, 64), (torch.float32, 2, 1, 200, 64, 48),
                                                 (torch.bfloat16, 4, 4, 333, 128, 40),
                                                 # ... an odd one (A_K rows one element at a time), 56, 64 in fp32
