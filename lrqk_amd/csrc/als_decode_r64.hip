@@ -239,24 +239,11 @@ constexpr int kS64Threads = 512;
 constexpr int kS64Ld = 65;  // row stride of a 64 x 64 matrix in LDS
 
 // In-place inverse of one SPD matrix of even order r <= 64 held in LDS ([64][kS64Ld]; only the leading r x r block
-// is read), by one wave.  The matrix, scaled to unit diagonal, sits in the accumulators of 2 x 2 tiles of the
-// 32x32x2 fp32 MFMA and is swept on its pivots two at a time: with P = {p, p + 1} and D = a_PP (2 x 2),
-//   a_ij -> a_ij - a_iP D^-1 a_Pj,   a_iP -> a_iP D^-1,   a_Pj -> D^-1 a_Pj,   a_PP -> -D^-1,
-// which is the composition of the sweeps on p and on p + 1, keeps the matrix symmetric and, after all pivots,
-// leaves -G^-1.  All four cases are ONE rank-2 update acc -= A B per tile -- the two k elements of the MFMA are the
-// two pivots -- with operands made from rows p and p + 1 alone (by symmetry they are also the columns):
-// B = rows P, A = (rows P)^T D^-1, except that in the pivots' own columns B holds D - I and in their own rows A
-// holds I - D^-1; that leaves 2 I - D^-1 in the pivot block, and since an entry (p, p) feeds nothing after its
-// own sweep, the 2 is taken off every diagonal entry once, at the end.  B_PP = D - I cancels badly for large D,
-// hence the scaling to unit diagonal.  Rows p and p + 1 sit in the lanes of one half of the wave; the operands need
-// row p in the lower and row p + 1 in the upper half (v_permlane32_swap).  Rows and columns >= r form an identity
+// is read), by one wave: the scheme of invert_sweep_mfma -- symmetric sweeps on the matrix scaled to unit diagonal,
+// the sweeps on p and p + 1 as the two k elements of one rank-2 MFMA update, the 2 that every sweep leaves on its
+// diagonal entry taken off at the end -- on the accumulators of 2 x 2 tiles: row p (and p + 1) of both column
+// blocks makes the operands, A_i = B_i / d for the rows of either block.  Rows and columns >= r form an identity
 // block.  sbuf: 64 floats.
-__device__ __forceinline__ float half_pair(float lo_src, float hi_src, int hp) {
-  // lanes 0..31 get lo_src, lanes 32..63 get hi_src, both taken from the half `hp` (compile-time) of the sources
-  const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo_src), __float_as_uint(hi_src), false, false);
-  return __uint_as_float(hp ? sw[1] : sw[0]);
-}
-
 __device__ __forceinline__ void invert64_sweep_mfma(float* G, int r, float* sbuf) {
   const int lane = lane_id();
   const int col = lane & 31, half = lane >> 5;
@@ -300,22 +287,28 @@ __device__ __forceinline__ void invert64_sweep_mfma(float* G, int r, float* sbuf
       const float da = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r0P), pl + 32 * hp));
       const float db = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r0P), pl + 1 + 32 * hp));
       const float dc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r1P), pl + 1 + 32 * hp));
-      const float det = fmaf(da, dc, -db * db);
-      float rd = __builtin_amdgcn_rcpf(det);
-      rd = fmaf(fmaf(-det, rd, 1.0f), rd, rd);
-      const float ia = dc * rd, ib = -db * rd, ic = da * rd;  // D^-1 = [ia ib; ib ic]
-      const float ck = half ? ic : ia;                          // D^-1[k][k] for this lane's k
+      float rc0 = __builtin_amdgcn_rcpf(da);
+      rc0 = fmaf(fmaf(-da, rc0, 1.0f), rc0, rc0);
+      const float brc = db * rc0;
+      const float c1 = fmaf(-db, brc, dc);  // the second pivot as the first sweep leaves it
+      float rc1 = __builtin_amdgcn_rcpf(c1);
+      rc1 = fmaf(fmaf(-c1, rc1, 1.0f), rc1, rc1);
+      const float rck = half ? rc1 : rc0;
       const float wp0 = col == pl ? 1.0f : 0.0f, wp1 = col == pl + 1 ? 1.0f : 0.0f;
       float Av[2], Bv[2];
       {  // the pivots' own block of columns
         const float U = half_pair(r0P, r1P, hp), V = half_pair(r1P, r0P, hp);  // [row p | row p + 1], [row p + 1 | row p]
-        Av[P] = fmaf(U, ck, V * ib) - (wp0 * (half ? ib : ia) + wp1 * (half ? ic : ib));
-        Bv[P] = U - (wp0 * in0 + wp1 * in1);
+        const float B1 = (half ? V : U) - wp0;     // the first sweep's B, in every lane
+        const float B2 = fmaf(-brc, B1, U) - wp1;  // (upper half) the second sweep's B
+        Bv[P] = half ? B2 : B1;
+        Av[P] = Bv[P] * rck;
       }
       {  // the other block of columns
         const float U = half_pair(r0X, r1X, hp), V = half_pair(r1X, r0X, hp);
-        Av[1 - P] = fmaf(U, ck, V * ib);
-        Bv[1 - P] = U;
+        const float B1 = half ? V : U;
+        const float B2 = fmaf(-brc, B1, U);
+        Bv[1 - P] = half ? B2 : B1;
+        Av[1 - P] = Bv[1 - P] * rck;
       }
       // the tiles that hold the next pivots' rows first: the other two run while those rows are being read
       const int Pn = (p + 2) >> 5 < 2 ? (p + 2) >> 5 : P;
