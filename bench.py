@@ -34,10 +34,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # Keyed by (workload, score index in use): with the index the kernel is score_prefilter_kernel and reads the
 # 8-bit copy (34 bytes per row) plus the rows it rescores; without it score_filter_kernel reads A_K itself.
 MEASURED_TRAFFIC = {
-    ("llama8b_128k_bf16", True): {"bytes": (78844.6 * 2.000 + 867.2 * 1.000) * 1024, "rows_rescored_in_that_run": 171000,
-                                  "profile": "profiles/score_filter_llama8b_128k_hbm_traffic.md"},
+    ("llama8b_128k_bf16", True): {"bytes": (78875.8 * 2.000 + 1007.1 * 1.000) * 1024, "rows_rescored_in_that_run": 153723,
+                                  "profile": "profiles/decode_step_llama8b_128k_hbm_traffic_and_sq_counters.md"},
     ("llama8b_128k_bf16", False): {"bytes": (131110.0 * 2.000 + 1060.2 * 1.000) * 1024, "rows_rescored_in_that_run": 0,
-                                   "profile": "profiles/score_filter_llama8b_128k_hbm_traffic.md"}}
+                                   "profile": "profiles/decode_step_llama8b_128k_hbm_traffic_and_sq_counters.md "
+                                              "(an earlier build's run of --no-score-index)"}}
 
 
 def parse():
@@ -537,6 +538,17 @@ def decode_bench(a, compact=False):
                      "best": {"vectors_in_flight": best[0], "nontemporal": bool(best[1]), "workgroups_per_cu": best[2]},
                      "gbs_by_in_flight_nontemporal_wg_per_cu": {f"{k[0]}/{k[1]}/{k[2]}": round(v, 0)
                                                                 for k, v in sorted(table.items())}}
+            # the same sweep with launches of the size of one score index (slices of the buffer read in turn, so
+            # that no launch finds its slice in the last-level cache): what a launch of the scan's size can reach
+            slice_b = (bh * int(m_avg) * w.r) // 16 * 16
+            if 0 < slice_b <= (a.probe_mb << 20) // 4:
+                t2, _ = ops_mod.probe_read_sweep((a.probe_mb << 20) // slice_b * slice_b, 2, dev, slice_bytes=slice_b)
+                b2 = max(t2, key=t2.get)
+                sweep["launches_of_index_size"] = {
+                    "bytes_per_launch": slice_b, "best_gbs": round(t2[b2], 1), "best_us": round(slice_b / t2[b2] / 1e3, 2),
+                    "best": {"vectors_in_flight": b2[0], "nontemporal": bool(b2[1]), "workgroups_per_cu": b2[2]},
+                    "gbs_by_in_flight_nontemporal_wg_per_cu": {f"{k[0]}/{k[1]}/{k[2]}": round(v, 0)
+                                                               for k, v in sorted(t2.items())}}
     # (between events: the profiler's duration of the same kernel is 2 to 3 us shorter; an empty kernel reads
     # pair_us between the same events, and a second one adds as much again, so the share of the bracket that is
     # not the kernel cannot be taken off by such a calibration)

@@ -271,10 +271,12 @@ int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, int reps, do
                          void* stream);
 /* Measurement helper (no counterpart in the reference): one variant of the plain read -- in_flight (4, 8 or 16)
  * 16-byte vectors per thread, plain or non-temporal loads, grid_per_cu workgroups of 256 threads per CU -- for a
- * sweep that looks for the best read rate of the GPU at hand.  sink: a few KB of device memory (never written in
- * practice).  Waits for the stream. */
-int lrqk_probe_read_variant(const void* src, void* sink, int64_t bytes, int reps, int in_flight, int nontemporal,
-                            int grid_per_cu, double* read_ms, void* stream);
+ * sweep that looks for the best read rate of the GPU at hand.  slice_bytes = 0: every launch reads the whole buffer;
+ * > 0: a launch reads one slice of that size and the launches take the slices in turn (the rate of a launch of a
+ * given size whose data does not come from the last-level cache).  read_ms: per launch.  sink: 64 KB of device
+ * memory (never written in practice).  Waits for the stream. */
+int lrqk_probe_read_variant(const void* src, void* sink, int64_t bytes, int64_t slice_bytes, int reps, int in_flight,
+                            int nontemporal, int grid_per_cu, double* read_ms, void* stream);
 /* No counterpart in the reference.  What a pair of HIP events reads around `kernels` (1..16) launches that do nothing
  * (average microseconds over `reps` <= 256 pairs on the caller's stream, each pair between two other launches; waits
  * for the stream).  The reading with one launch less the difference between two launches and one is the part of an

@@ -75,7 +75,7 @@ def _sig(lib):
         "lrqk_timing_read": ([vp, c.POINTER(c.c_double), c.POINTER(i32)], i32),
         "lrqk_probe_bandwidth": ([vp, vp, i64, i32, c.POINTER(c.c_double), c.POINTER(c.c_double), vp], i32),
         "lrqk_probe_event_pair": ([i32, i32, c.POINTER(c.c_double), vp], i32),
-        "lrqk_probe_read_variant": ([vp, vp, i64, i32, i32, i32, i32, c.POINTER(c.c_double), vp], i32),
+        "lrqk_probe_read_variant": ([vp, vp, i64, i64, i32, i32, i32, i32, c.POINTER(c.c_double), vp], i32),
         "lrqk_d0_indices_select": ([vp, vp, vp, i64, i64, i64, i32], i32),
         "lrqk_take_along_dim_with_mask": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32], i64),
     }

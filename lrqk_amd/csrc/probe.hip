@@ -142,11 +142,13 @@ extern "C" int lrqk_probe_bandwidth(const void* src, void* dst, int64_t bytes, i
   return LRQK_OK;
 }
 
-extern "C" int lrqk_probe_read_variant(const void* src, void* sink, int64_t bytes, int reps, int in_flight,
-                                       int nontemporal, int grid_per_cu, double* read_ms, void* stream) {
+extern "C" int lrqk_probe_read_variant(const void* src, void* sink, int64_t bytes, int64_t slice_bytes, int reps,
+                                       int in_flight, int nontemporal, int grid_per_cu, double* read_ms, void* stream) {
   LRQK_REQUIRE(src && sink && read_ms, LRQK_EINVAL, "null pointer");
   LRQK_REQUIRE(bytes >= 16 && bytes % 16 == 0 && reps > 0 && reps <= 1000, LRQK_EINVAL, "bad sizes bytes=%lld reps=%d",
                (long long)bytes, reps);
+  LRQK_REQUIRE(slice_bytes == 0 || (slice_bytes >= 16 && slice_bytes % 16 == 0 && slice_bytes <= bytes), LRQK_EINVAL,
+               "slice_bytes=%lld not a multiple of 16 within the buffer", (long long)slice_bytes);
   LRQK_REQUIRE((in_flight == 4 || in_flight == 8 || in_flight == 16) && grid_per_cu >= 1 && grid_per_cu <= 64, LRQK_EINVAL,
                "in_flight=%d (4, 8 or 16), grid_per_cu=%d (1..64)", in_flight, grid_per_cu);
   LRQK_REQUIRE((uintptr_t)src % 16 == 0, LRQK_EINVAL, "src must be 16-byte aligned");
@@ -154,13 +156,17 @@ extern "C" int lrqk_probe_read_variant(const void* src, void* sink, int64_t byte
   int dev = 0, n_cu = 0;
   LRQK_HIP_CHECK(hipGetDevice(&dev));
   LRQK_HIP_CHECK(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-  const int64_t n_vec = bytes / 16;
+  // a launch reads the whole buffer, or (slice_bytes > 0) one slice of it, the launches taking the slices in turn
+  const int64_t n_vec = (slice_bytes ? slice_bytes : bytes) / 16;
+  const int64_t n_slices = slice_bytes ? bytes / slice_bytes : 1;
+  int64_t turn = 0;
   const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((int64_t)n_cu * grid_per_cu,
                                                                         (n_vec + kProbeThreads - 1) / kProbeThreads));
   auto launch = [&]() {
-#define LRQK_PROBE_CASE(UU, NTT)                                                                                  \
-  hipLaunchKernelGGL((probe_read_variant_kernel<UU, NTT>), dim3(grid), dim3(kProbeThreads), 0, st, (const uint4*)src, \
-                     n_vec, (uint32_t*)sink)
+    const uint4* from = (const uint4*)src + (turn++ % n_slices) * n_vec;
+#define LRQK_PROBE_CASE(UU, NTT)                                                                           \
+  hipLaunchKernelGGL((probe_read_variant_kernel<UU, NTT>), dim3(grid), dim3(kProbeThreads), 0, st, from, n_vec, \
+                     (uint32_t*)sink)
     if (nontemporal) {
       if (in_flight == 4) LRQK_PROBE_CASE(4, true);
       else if (in_flight == 8) LRQK_PROBE_CASE(8, true);

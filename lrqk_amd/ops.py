@@ -395,19 +395,22 @@ def probe_bandwidth(nbytes: int, reps: int = 10, device="cuda:0"):
     return nbytes / (r_ms.value * 1e-3) / 1e9, 2 * nbytes / (c_ms.value * 1e-3) / 1e9
 
 
-def probe_read_sweep(nbytes: int, reps: int = 5, device="cuda:0"):
+def probe_read_sweep(nbytes: int, reps: int = 5, device="cuda:0", slice_bytes: int = 0):
     """The plain read over ``nbytes`` in every variant (4 / 8 / 16 vectors in flight, plain / non-temporal loads,
-    1 .. 8 workgroups per CU): ({(in_flight, nontemporal, grid_per_cu): GB/s}, best GB/s)."""
+    1 .. 8 workgroups per CU): ({(in_flight, nontemporal, grid_per_cu): GB/s}, best GB/s).  With ``slice_bytes`` a
+    launch reads one slice of the buffer and the launches take the slices in turn: the rate of launches of that size."""
     src = torch.empty(nbytes, dtype=torch.uint8, device=device).fill_(1)
     sink = torch.zeros(1 << 16, dtype=torch.uint8, device=device)
     table = {}
     ms = ctypes.c_double()
+    per_launch = slice_bytes or nbytes
+    n = reps * (nbytes // slice_bytes) if slice_bytes else reps
     for nt in (0, 1):
         for fl in (4, 8, 16):
             for per_cu in (1, 2, 4, 8):
-                check(_lib.load().lrqk_probe_read_variant(src.data_ptr(), sink.data_ptr(), nbytes, reps, fl, nt, per_cu,
-                                                          ctypes.byref(ms), _stream(src)))
-                table[(fl, nt, per_cu)] = nbytes / (ms.value * 1e-3) / 1e9
+                check(_lib.load().lrqk_probe_read_variant(src.data_ptr(), sink.data_ptr(), nbytes, slice_bytes, min(n, 1000), fl,
+                                                          nt, per_cu, ctypes.byref(ms), _stream(src)))
+                table[(fl, nt, per_cu)] = per_launch / (ms.value * 1e-3) / 1e9
     return table, max(table.values())
 
 

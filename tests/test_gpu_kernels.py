@@ -842,3 +842,8 @@ def test_measurement_probes(ops):
     table, best = ops.probe_read_sweep((64 << 20) + 4096 + 16, 2, DEV)
     assert len(table) == 24 and all(50.0 < v < 20000.0 for v in table.values()), table
     assert best == max(table.values())
+    # launches that take slices of the buffer in turn
+    table, best = ops.probe_read_sweep(64 << 20, 1, DEV, slice_bytes=8 << 20)
+    assert len(table) == 24 and all(20.0 < v < 20000.0 for v in table.values()), table
+    with pytest.raises(ValueError):
+        ops.probe_read_sweep(64 << 20, 1, DEV, slice_bytes=24)
