@@ -82,11 +82,13 @@ extern "C" int lrqk_ctx_reserve(lrqk_ctx* ctx, int bh, int64_t max_tokens, int t
   const int64_t key_stride = (max_tokens + 63) & ~(int64_t)63;
   if ((rc = ctx->keys.ensure((size_t)bh * key_stride * 4))) return rc;
   if ((rc = ctx->attn_part.ensure((size_t)bh * 64 * (d + 2) * sizeof(float)))) return rc;
-  if ((rc = ctx->als_part.ensure((size_t)bh * 32 * (32 * 32 + 32) * sizeof(float)))) return rc;
+  // (partial sums of the factor update: up to 32 splits of r x r + r sums, r padded to one or two matrix-core tiles)
+  const size_t tile_r = r > 32 ? 64 : 32;
+  if ((rc = ctx->als_part.ensure((size_t)bh * 32 * (tile_r * tile_r + tile_r) * sizeof(float)))) return rc;
   if ((rc = ctx->als_kq.ensure((size_t)bh * n_active * sizeof(float)))) return rc;
   if ((rc = ctx->als_iter.ensure((size_t)bh * LRQK_MAX_DECODE_ITERS * (2 * r + 1) * sizeof(float)))) return rc;
   if ((rc = ctx->new_idx.ensure((size_t)bh * topk * sizeof(int32_t)))) return rc;
-  if ((rc = ctx->misc.ensure((size_t)bh * (topk * 5 + 16)))) return rc;
+  if ((rc = ctx->misc.ensure((size_t)bh * topk * 13 + (size_t)bh * 4 + 64))) return rc;  // (as lrqk_decode_step sizes it)
   return LRQK_OK;
 }
 
